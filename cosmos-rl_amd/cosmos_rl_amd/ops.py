@@ -1,0 +1,339 @@
+"""Torch-facing operators of the FP8 hot path, named after the third-party ops the
+reference calls, each a thin shim over one C-ABI entry point.
+
+The shim allocates every output and workspace as a torch tensor, passes raw
+device pointers plus the current HIP stream, and never synchronises.  Inputs
+must live on the GPU; nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+FP8_DTYPE = torch.float8_e4m3fn
+FP8_MAX = 448.0
+BLOCK = 128
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "cosmos_fp8 operators run on the GPU only (got a tensor on "
+                f"{t.device}); there is no CPU path")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _out_code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return _lib.OUT_BF16
+    if dtype == torch.float32:
+        return _lib.OUT_F32
+    raise ValueError(f"out_dtype must be bfloat16 or float32, got {dtype}")
+
+
+# ---------------------------------------------------------------------------
+# quantizers
+# ---------------------------------------------------------------------------
+def scaled_fp8_quant(input: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                     use_per_token_if_dynamic: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Dynamic FP8 quantisation with the call shape of ``vllm._custom_ops.scaled_fp8_quant``
+    (reference call sites: cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:995-997,
+    monkey_patch_for_fp8.py:47-49).
+
+    ``use_per_token_if_dynamic=True``: one scale per row, returns (fp8 [R, C], fp32 [R, 1]).
+    ``False``: one scale for the tensor, returns (fp8 [R, C], fp32 [1]).
+    Static scales (``scale`` given) are not part of this path.
+    """
+    if scale is not None:
+        raise NotImplementedError("static-scale quantisation is not on the cosmos-rl FP8 path")
+    if input.dim() != 2:
+        raise ValueError(f"expected a 2-D tensor, got {tuple(input.shape)}")
+    if not use_per_token_if_dynamic:
+        q, s = quant_tensorwise(input)
+        return q, s
+    return quant_rowwise(input)
+
+
+def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError(f"rowwise FP8 quantisation takes bfloat16 input, got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError(f"expected a 2-D tensor, got {tuple(x.shape)}")
+    if x.stride(1) != 1 and x.shape[1] > 1:
+        x = x.contiguous()
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=x.device)
+    s = torch.empty((rows, 1), dtype=torch.float32, device=x.device)
+    ld_x = x.stride(0) if rows > 1 else max(cols, 1)
+    _lib.check(_lib.load().cfp8_quant_rowwise(x.data_ptr(), rows, cols, ld_x, q.data_ptr(), cols,
+                                             s.data_ptr(), _stream()))
+    return q, s
+
+
+def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Tensor], torch.Tensor]:
+    """Tensorwise dynamic quantisation of a list of bf16 tensors in two launches per
+    batch.  Returns (list of fp8 tensors shaped like the inputs, fp32 scales [n])."""
+    n = len(tensors)
+    if n == 0:
+        return [], torch.empty(0, dtype=torch.float32)
+    _need_gpu(*tensors)
+    dev = tensors[0].device
+    scales = torch.empty(n, dtype=torch.float32, device=dev)
+    amax_ws = torch.empty(n, dtype=torch.float32, device=dev)
+    outs: List[torch.Tensor] = []
+    keep = []
+    descs = (_lib.TensorDesc * n)()
+    sbase = scales.data_ptr()
+    for i, t in enumerate(tensors):
+        if t.dtype != torch.bfloat16:
+            raise ValueError(f"tensorwise FP8 quantisation takes bfloat16 input, got {t.dtype}")
+        tc = t if t.is_contiguous() else t.contiguous()
+        keep.append(tc)
+        q = torch.empty(t.shape, dtype=FP8_DTYPE, device=dev)
+        outs.append(q)
+        descs[i].x = tc.data_ptr()
+        descs[i].q = q.data_ptr()
+        descs[i].scale = sbase + 4 * i
+        descs[i].numel = tc.numel()
+    _lib.check(_lib.load().cfp8_quant_tensorwise_multi(descs, n, amax_ws.data_ptr(), _stream()))
+    return outs, scales
+
+
+def quant_tensorwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One global amax, one fp32 scale (shape [1]), saturated cast: the tensorwise recipe
+    selected at cosmos_rl/utils/fp8/fp8_util.py:121-137."""
+    outs, scales = quant_tensorwise_multi([x])
+    return outs[0], scales
+
+
+def per_block_cast_to_fp8(w: torch.Tensor, transpose_out: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128x128 block quantisation of [R, C] or a stack [E, R, C].
+    Returns (fp8 like w - or with the last two dims swapped when ``transpose_out`` -,
+    fp32 scales [..., ceil(R/128), ceil(C/128)])."""
+    _need_gpu(w)
+    if w.dtype != torch.bfloat16:
+        raise ValueError(f"block FP8 quantisation takes bfloat16 input, got {w.dtype}")
+    if w.dim() not in (2, 3):
+        raise ValueError(f"expected a 2-D or 3-D tensor, got {tuple(w.shape)}")
+    w = w.contiguous()
+    lead = w.shape[:-2]
+    rows, cols = w.shape[-2:]
+    batch = int(lead[0]) if lead else 1
+    oshape = (*lead, cols, rows) if transpose_out else (*lead, rows, cols)
+    q = torch.empty(oshape, dtype=FP8_DTYPE, device=w.device)
+    s = torch.empty((*lead, -(-rows // BLOCK), -(-cols // BLOCK)), dtype=torch.float32, device=w.device)
+    _lib.check(_lib.load().cfp8_quant_block128(w.data_ptr(), batch, rows, cols, q.data_ptr(), s.data_ptr(),
+                                              1 if transpose_out else 0, _stream()))
+    return q, s
+
+
+def prepare_fp8_weight(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``dsgemm_utils.prepare_fp8_weight`` (cosmos_rl/policy/kernel/group_gemms.py:132)."""
+    return per_block_cast_to_fp8(w)
+
+
+def _group128(x: torch.Tensor, mode: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    _need_gpu(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError(f"1x128 FP8 quantisation takes bfloat16 input, got {x.dtype}")
+    if x.dim() != 2:
+        raise ValueError(f"expected a 2-D tensor, got {tuple(x.shape)}")
+    if x.stride(1) != 1 and x.shape[1] > 1:
+        x = x.contiguous()
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=x.device)
+    s = torch.empty((rows, -(-cols // BLOCK)), dtype=torch.float32, device=x.device)
+    ld_x = x.stride(0) if rows > 1 else max(cols, 1)
+    _lib.check(_lib.load().cfp8_quant_group128(x.data_ptr(), rows, cols, ld_x, q.data_ptr(), cols,
+                                              s.data_ptr(), mode, _stream()))
+    return q, s
+
+
+def groupwise_activation_quant(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``dsgemm_kernels.groupwise_activation_quant`` (group_gemms.py:188-189): 1x128 groups,
+    returns (fp8 [M, K], fp32 [M, K/128]) ready to feed the block GEMM."""
+    return _group128(x, _lib.GROUP_MODE_DIV)
+
+
+def prepare_fp8_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``dsgemm_utils.prepare_fp8_input`` (group_gemms.py:190-191)."""
+    return _group128(x, _lib.GROUP_MODE_DIV)
+
+
+def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``per_token_cast_to_fp8`` of the reference's tests/test_deepep.py:75-85, including its
+    formula ``x * (448 / amax.clamp(1e-4))`` with scales ``amax / 448``."""
+    return _group128(x, _lib.GROUP_MODE_DEEPEP)
+
+
+def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128,
+                   out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``weight_dequant`` (cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259):
+    y = fp8 * s[i // 128, j // 128]; output in the default dtype unless given."""
+    _need_gpu(x, s)
+    assert x.is_contiguous() and s.is_contiguous()
+    assert x.dim() == 2 and s.dim() == 2
+    if block_size != BLOCK:
+        raise ValueError("only 128x128 blocks are supported")
+    dt = out_dtype or torch.get_default_dtype()
+    M, N = x.shape
+    if tuple(s.shape) != (-(-M // BLOCK), -(-N // BLOCK)):
+        raise ValueError(f"scale shape {tuple(s.shape)} does not match weight {tuple(x.shape)}")
+    y = torch.empty((M, N), dtype=dt, device=x.device)
+    _lib.check(_lib.load().cfp8_dequant_block128(x.data_ptr(), s.data_ptr(), M, N, y.data_ptr(),
+                                                _out_code(dt), _stream()))
+    return y
+
+
+# ---------------------------------------------------------------------------
+# GEMMs
+# ---------------------------------------------------------------------------
+def scaled_mm(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+              out_dtype: torch.dtype = torch.bfloat16, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rowwise ``torch._scaled_mm``: a fp8 [M, K] row-major, b fp8 [K, N] column-major (the
+    ``.t()`` of a contiguous [N, K] weight, monkey_patch_for_fp8.py:52), scale_a [M, 1],
+    scale_b [1, N] (or [N, 1]); out = (a @ b) * scale_a * scale_b (+ bias)."""
+    _need_gpu(a, b, scale_a, scale_b)
+    if a.dtype != FP8_DTYPE or b.dtype != FP8_DTYPE:
+        raise ValueError("scaled_mm takes float8_e4m3fn operands")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[0]:
+        raise ValueError(f"shape mismatch: {tuple(a.shape)} @ {tuple(b.shape)}")
+    M, K = a.shape
+    N = b.shape[1]
+    if not (a.stride(1) == 1 or K == 1):
+        raise ValueError("a must be row-major")
+    if not (b.stride(0) == 1 or K == 1):
+        raise ValueError("b must be column-major (pass weight.t() of a contiguous [N, K] weight)")
+    if scale_a.numel() != M or scale_b.numel() != N:
+        raise ValueError("scaled_mm needs rowwise scales: scale_a [M, 1] and scale_b [1, N]")
+    sa = scale_a.reshape(-1).contiguous().float()
+    sb = scale_b.reshape(-1).contiguous().float()
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    ld_a = a.stride(0) if M > 1 else K
+    ld_b = b.stride(1) if N > 1 else K
+    _lib.check(_lib.load().cfp8_scaled_mm_rowwise(a.data_ptr(), ld_a, sa.data_ptr(), b.data_ptr(), ld_b,
+                                                 sb.data_ptr(), out.data_ptr(), N, _out_code(out_dtype),
+                                                 M, N, K, _stream()))
+    if bias is not None:
+        out = out + bias
+    return out
+
+
+def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+               bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
+               workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``Fp8LinearOp(use_per_token_if_dynamic=True).apply`` (monkey_patch_for_fp8.py:74-79):
+    per-token dynamic quantisation of x, then the rowwise scaled mm.
+
+    weight: fp8 [K, N] column-major, i.e. ``qweight.t()`` as the reference stores it;
+    weight_scale [N, 1]; x bf16 [..., K].  Returns [..., N]."""
+    _need_gpu(x, weight, weight_scale)
+    if x.dtype != torch.bfloat16:
+        raise ValueError(f"fp8_linear takes bfloat16 activations, got {x.dtype}")
+    K, N = weight.shape
+    if weight.stride(0) != 1 and K > 1:
+        raise ValueError("weight must be the transposed view of a contiguous [N, K] fp8 tensor")
+    x2 = x.reshape(-1, K)
+    if x2.stride(1) != 1 and K > 1:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    lib = _lib.load()
+    need = lib.cfp8_linear_workspace_bytes(M, K)
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=x.device)
+    sw = weight_scale.reshape(-1)
+    if sw.dtype != torch.float32 or not sw.is_contiguous():
+        sw = sw.contiguous().float()
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    ld_x = x2.stride(0) if M > 1 else K
+    ld_w = weight.stride(1) if N > 1 else K
+    _lib.check(lib.cfp8_linear_rowwise(x2.data_ptr(), ld_x, weight.data_ptr(), ld_w, sw.data_ptr(),
+                                      out.data_ptr(), N, _out_code(out_dtype), M, N, K,
+                                      workspace.data_ptr(), workspace.numel() * workspace.element_size(),
+                                      _stream()))
+    if bias is not None:
+        out = out + bias
+    return out.reshape(*x.shape[:-1], N)
+
+
+def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Tensor, torch.Tensor],
+                         out: torch.Tensor, rhs_scale_kn: bool = False) -> torch.Tensor:
+    """Dense block-scaled GEMM.  lhs = (fp8 [M, K], fp32 [M, K/128]); rhs = (fp8 [N, K],
+    fp32 [ceil(N/128), K/128]) or, with ``rhs_scale_kn``, scales laid out [K/128, ceil(N/128)]
+    (what quantising a [K, N] weight produces).  Writes into ``out`` [M, N]."""
+    a, sa = lhs
+    b, sb = rhs
+    _need_gpu(a, sa, b, sb, out)
+    M, K = a.shape
+    N = b.shape[0]
+    if b.shape[1] != K or tuple(out.shape) != (M, N):
+        raise ValueError("shape mismatch in block-scaled GEMM")
+    a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
+    nb, kb = -(-N // BLOCK), K // BLOCK
+    if rhs_scale_kn:
+        if tuple(sb.shape) != (kb, nb):
+            raise ValueError(f"rhs scales must be [{kb}, {nb}], got {tuple(sb.shape)}")
+        stride_n, stride_k = 1, nb
+    else:
+        if tuple(sb.shape) != (nb, kb):
+            raise ValueError(f"rhs scales must be [{nb}, {kb}], got {tuple(sb.shape)}")
+        stride_n, stride_k = kb, 1
+    if tuple(sa.shape) != (M, kb):
+        raise ValueError(f"lhs scales must be [{M}, {kb}], got {tuple(sa.shape)}")
+    if not out.is_contiguous():
+        raise ValueError("out must be contiguous")
+    _lib.check(_lib.load().cfp8_gemm_block128(a.data_ptr(), K, sa.data_ptr(), b.data_ptr(), K, sb.data_ptr(),
+                                             stride_n, stride_k, out.data_ptr(), N, _out_code(out.dtype),
+                                             M, N, K, _stream()))
+    return out
+
+
+def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs: Tuple[torch.Tensor, torch.Tensor],
+                                              rhs: Tuple[torch.Tensor, torch.Tensor],
+                                              out: torch.Tensor, m_indices: torch.Tensor) -> torch.Tensor:
+    """``deep_gemm.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous`` (group_gemms.py:194-225).
+    lhs = (fp8 [M, K], fp32 [M, K/128]); rhs = (fp8 [E, N, K], fp32 [E, ceil(N/128), K/128]);
+    m_indices int32 [M], groups contiguous and 128-row aligned, negative = padding (rows left
+    untouched).  Writes into ``out`` [M, N]."""
+    a, sa = lhs
+    b, sb = rhs
+    _need_gpu(a, sa, b, sb, out, m_indices)
+    M, K = a.shape
+    E, N, Kb = b.shape
+    if Kb != K or tuple(out.shape) != (M, N) or m_indices.numel() != M:
+        raise ValueError("shape mismatch in grouped GEMM")
+    if m_indices.dtype != torch.int32:
+        m_indices = m_indices.to(torch.int32)
+    a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
+    if tuple(sb.shape) != (E, -(-N // BLOCK), K // BLOCK) or tuple(sa.shape) != (M, K // BLOCK):
+        raise ValueError("scale shape mismatch in grouped GEMM")
+    if not out.is_contiguous():
+        raise ValueError("out must be contiguous")
+    _lib.check(_lib.load().cfp8_gemm_grouped_block128(a.data_ptr(), K, sa.data_ptr(), b.data_ptr(), sb.data_ptr(),
+                                                     m_indices.contiguous().data_ptr(), out.data_ptr(), N,
+                                                     _out_code(out.dtype), M, N, K, E, _stream()))
+    return out
+
+
+def create_indices_from_offsets_nosync(m_offsets: torch.Tensor, total: Optional[int] = None) -> torch.Tensor:
+    """``dsgemm_utils.create_indices_from_offsets_nosync`` (group_gemms.py:157): expert id per
+    row from the inclusive cumulative group ends.  Pass ``total`` (the number of rows, which the
+    caller already knows from its own slice at group_gemms.py:154) to stay free of a host sync;
+    without it the last offset is read back."""
+    if total is None:
+        total = int(m_offsets[-1])
+    rows = torch.arange(total, device=m_offsets.device, dtype=m_offsets.dtype)
+    return torch.searchsorted(m_offsets, rows, right=True).to(torch.int32)

@@ -1,0 +1,115 @@
+"""Grouped-GEMM strategies for MoE experts with the interface of
+cosmos_rl/policy/kernel/group_gemms.py (``GroupGEMMStrategy`` :32-69, ``TorchBF16GroupGEMM``
+:80-118, ``DSGroupGEMM`` :121-233).  ``DSGroupGEMM`` runs 128x128 block-quantised weights,
+1x128 group-quantised activations and the grouped FP8 MFMA GEMM of this library."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from cosmos_rl_amd import _lib, ops
+
+__all__ = ["GroupGEMMStrategy", "DSGroupGEMM", "TorchBF16GroupGEMM"]
+
+
+class GroupGEMMStrategy:
+    """Base class for group gemm strategies."""
+
+    def __init__(self, custom_activation):
+        self.activation_function = custom_activation
+
+    def arrange_expert_weights(self, all_weights, submod_name, module):
+        """Turn the per-expert weight list of ``submod_name`` ('gate_proj', 'up_proj',
+        'down_proj') into the layout the strategy computes with; may register extra
+        parameters on ``module``.  Returns the arranged weight tensor."""
+        raise NotImplementedError("Requires arrange_expert_weights method")
+
+    def execute(self, contig_tokens, m_sizes, m_offsets, module):
+        """Run gate/up/activation/down over tokens laid out contiguously by expert."""
+        raise NotImplementedError("GroupGEMM strategy must implement execute method")
+
+    @staticmethod
+    def is_available() -> bool:
+        return False
+
+
+class TorchBF16GroupGEMM(GroupGEMMStrategy):
+    """bf16 baseline: one matmul per expert group (the reference uses ``torch._grouped_mm``)."""
+
+    def arrange_expert_weights(self, all_weights, submod_name, module):
+        return torch.stack(all_weights)
+
+    @staticmethod
+    def _grouped(x, w, m_offsets):
+        out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.bfloat16, device=x.device)
+        start = 0
+        for e, end in enumerate(m_offsets.tolist()):
+            if end > start:
+                out[start:end] = x[start:end] @ w[e].t()
+            start = end
+        return out
+
+    def execute(self, contig_tokens, m_sizes, m_offsets, module):
+        w_gate = module.get_parameter("gate_proj_weight")
+        w_up = module.get_parameter("up_proj_weight")
+        w_down = module.get_parameter("down_proj_weight")
+        hidden = self.activation_function(self._grouped(contig_tokens, w_gate, m_offsets)) * \
+            self._grouped(contig_tokens, w_up, m_offsets)
+        return self._grouped(hidden, w_down, m_offsets)
+
+    @staticmethod
+    def is_available() -> bool:
+        return True
+
+
+class DSGroupGEMM(GroupGEMMStrategy):
+    """FP8 grouped GEMM: block-quantised expert weights, 1x128 activation groups."""
+
+    def __init__(self, custom_activation, use_triton_quant=True):
+        # ``use_triton_quant`` selected between two third-party quantisers in the reference
+        # (group_gemms.py:188-191); both map to the one HIP group quantiser here.
+        self.activation_function = custom_activation
+        self.use_triton_quant = use_triton_quant
+
+    def arrange_expert_weights(self, all_weights, submod_name, module):
+        combined_weights = torch.stack(all_weights)
+        fp8, scales = ops.prepare_fp8_weight(combined_weights)
+        module.register_parameter(f"{submod_name}_fp8", nn.Parameter(fp8, requires_grad=False))
+        module.register_parameter(f"{submod_name}_scales", nn.Parameter(scales, requires_grad=False))
+        return combined_weights
+
+    def _quant(self, x):
+        return ops.groupwise_activation_quant(x) if self.use_triton_quant else ops.prepare_fp8_input(x)
+
+    def execute(self, contig_tokens, m_sizes, m_offsets, module):
+        total = int(m_offsets[-1])
+        valid_tokens = contig_tokens[:total]
+        m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
+
+        gate_fp8, gate_s = module.get_parameter("gate_proj_fp8"), module.get_parameter("gate_proj_scales")
+        up_fp8, up_s = module.get_parameter("up_proj_fp8"), module.get_parameter("up_proj_scales")
+        down_fp8, down_s = module.get_parameter("down_proj_fp8"), module.get_parameter("down_proj_scales")
+
+        intermediate_size = module.get_parameter("gate_proj_weight").shape[1]
+        hidden_size = module.get_parameter("down_proj_weight").shape[1]
+        dev, dt = contig_tokens.device, contig_tokens.dtype
+
+        gate_out = torch.empty((total, intermediate_size), device=dev, dtype=dt)
+        up_out = torch.empty_like(gate_out)
+        down_out = torch.empty((total, hidden_size), device=dev, dtype=dt)
+
+        gate_up_input = self._quant(valid_tokens)
+        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (gate_fp8, gate_s), gate_out, m_indices)
+        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (up_fp8, up_s), up_out, m_indices)
+        hidden_states = self.activation_function(gate_out) * up_out
+        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(self._quant(hidden_states), (down_fp8, down_s), down_out,
+                                                      m_indices)
+        contig_tokens[:total] = down_out
+        return contig_tokens
+
+    @staticmethod
+    def is_available() -> bool:
+        if not _lib.LIB_PATH.exists() or not torch.cuda.is_available():
+            return False
+        name = getattr(torch.cuda.get_device_properties(torch.cuda.current_device()), "gcnArchName", "")
+        return name.startswith("gfx950")

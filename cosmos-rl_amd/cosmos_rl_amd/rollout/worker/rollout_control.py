@@ -1,0 +1,87 @@
+"""Quantise-on-receive step of policy->rollout weight sync.
+
+Counterpart of the low-precision branch of ``recv_weight_shard.completion_lambda``
+(cosmos_rl/rollout/worker/rollout_control.py:684-695, 822-898) without the transport around
+it: the NCCL receive that fills the high-precision staging buffers, the instruction planner and
+the command loop stay with their owner; this class is what runs once every shard of one full
+weight has landed.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Iterable, List, Optional
+
+import torch
+
+
+class QuantizedWeightReceiver:
+    """Holds the maps the rollout worker builds at ``prepare_shard_infos_for_weight_sync_insts``
+    (rollout_control.py:374-438) and performs "quantise the full weight, check it on the first
+    sync, copy bytes and scales into the engine's parameters".
+
+    rollout            object with ``fp8_quantization(weight) -> (q_t, scale)`` and
+                       ``model_param_map(weight_mapper) -> {name: tensor}``
+    weight_mapper      object with ``get_unsplited_weight_name(name)``
+    hp_weight_map      full weight name -> bf16 staging parameter [out_dim, in_dim]
+    quantized_weight_map  full weight name -> the engine's fp8 parameter
+    """
+
+    def __init__(self, rollout, weight_mapper, hp_weight_map: Dict[str, torch.Tensor],
+                 quantized_weight_map: Dict[str, torch.Tensor], quantization_type: Optional[str] = "fp8"):
+        if quantization_type not in (None, "fp8"):
+            raise NotImplementedError(f"quantization_type={quantization_type!r} is not on this path")
+        self.rollout = rollout
+        self.weight_mapper = weight_mapper
+        self.hp_weight_map = hp_weight_map
+        self.quantized_weight_map = quantized_weight_map
+        self.quantization_type = quantization_type
+
+    # -- rollout_control.py:684-695 -------------------------------------------------------
+    def full_weight_name_of_group(self, param_names: Iterable[str]) -> str:
+        """An instruction group carries every split (q/k/v, gate/up) of one engine parameter;
+        any of its names identifies the unsplit weight."""
+        first = next(iter(param_names))
+        return self.weight_mapper.get_unsplited_weight_name(first)
+
+    def check_inside_group(self, param_names: Iterable[str], do_weight_sync_check: bool) -> bool:
+        """The plain element-wise recv check only applies to weights that are not re-quantised."""
+        if self.quantization_type is None:
+            return do_weight_sync_check
+        full = self.full_weight_name_of_group(param_names)
+        return do_weight_sync_check and full not in self.quantized_weight_map
+
+    def plan_group(self, param_names: List[str], do_weight_sync_check: bool = False) -> Callable[[], None]:
+        """Returns the completion callback for one instruction group, to be run (on the copy
+        stream) after every shard of the group has been received - rollout_control.py:822-827."""
+        post: List[str] = []
+        if self.quantization_type is not None and not self.check_inside_group(param_names, do_weight_sync_check):
+            post.append(self.full_weight_name_of_group(param_names))
+
+        def completion() -> None:
+            for name in post:
+                self.quantize_full_weight(name, do_weight_sync_check)
+
+        return completion
+
+    # -- rollout_control.py:856-898 -------------------------------------------------------
+    def quantize_full_weight(self, full_weight_name: str, do_weight_sync_check: bool = False) -> bool:
+        """Quantise one fully received weight into the engine.  Returns False when the name is
+        not a quantised weight (nothing to do)."""
+        if self.quantization_type != "fp8" or full_weight_name not in self.hp_weight_map:
+            return False
+        weight_to_quantize = self.hp_weight_map[full_weight_name]  # [out_dim, in_dim]
+        quantized_weight, weight_scale = self.rollout.fp8_quantization(weight_to_quantize)
+        model_param_map = self.rollout.model_param_map(self.weight_mapper)
+        native = model_param_map[full_weight_name]
+        if do_weight_sync_check:
+            # allclose has no fp8 kernel: promote both sides
+            if not torch.allclose(native.to(torch.bfloat16), quantized_weight.to(torch.bfloat16)):
+                raise ValueError(
+                    "FP8 weight doesn't match after weight sync and dynamic quantization for full weight "
+                    f"name: {full_weight_name}.")
+        native.copy_(quantized_weight)
+        scale_key = full_weight_name.replace(".weight", ".weight_scale")
+        scale_tensor = model_param_map[scale_key]
+        assert scale_tensor.shape == weight_scale.shape, (
+            f"scale_tensor.shape: {scale_tensor.shape}, weight_scale.shape: {weight_scale.shape}")
+        scale_tensor.copy_(weight_scale)
+        return True

@@ -1,0 +1,153 @@
+// Shared device helpers and host-side error plumbing for libcosmosfp8 (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cosmos_fp8.h"
+
+namespace cfp8 {
+
+// ---- host side -----------------------------------------------------------
+int set_error(int code, const char* fmt, ...);
+int check_launch(const char* what);
+int check_device();  // CFP8_OK when the current device is gfx950
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- device side ---------------------------------------------------------
+typedef uint32_t u32;
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kE4M3Max = 448.0f;
+constexpr float kAmaxFloor = 1e-12f;
+constexpr u32 kCanonNaN = 0x7FC00000u;
+
+__device__ __forceinline__ float bf16_lo(u32 w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(u32 w) { return __uint_as_float(w & 0xFFFF0000u); }
+
+// max over |bf16| bit patterns, two lanes of 16 bits at a time.  Unsigned
+// integer order equals numeric order for non-negative floats, and every NaN
+// pattern (> 0x7F80) sorts above infinity, so NaN propagates by construction.
+__device__ __forceinline__ u32 pk_absmax(u32 acc, u32 w) {
+    u16x2 a = __builtin_bit_cast(u16x2, acc);
+    u16x2 b = __builtin_bit_cast(u16x2, w & 0x7FFF7FFFu);
+    return __builtin_bit_cast(u32, __builtin_elementwise_max(a, b));
+}
+__device__ __forceinline__ u32 pk_fold(u32 acc) {  // -> bf16 bits of the max, in the low half
+    u32 lo = acc & 0xFFFFu, hi = acc >> 16;
+    return lo > hi ? lo : hi;
+}
+
+template <int CTRL>
+__device__ __forceinline__ u32 dpp(u32 v) {
+    return (u32)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+__device__ __forceinline__ u32 umax(u32 a, u32 b) { return a > b ? a : b; }
+
+// all-reduce max inside each aligned group of 16 lanes (one DPP row)
+__device__ __forceinline__ u32 row16_max(u32 v) {
+    v = umax(v, dpp<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = umax(v, dpp<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = umax(v, dpp<0x141>(v));  // row_half_mirror
+    v = umax(v, dpp<0x140>(v));  // row_mirror
+    return v;
+}
+// all-reduce max over the 64 lanes; the result is wave-uniform
+__device__ __forceinline__ u32 wave_max(u32 v) {
+    v = row16_max(v);
+    u32 a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    u32 c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return umax(umax(a, b), umax(c, d));
+}
+
+// amax bits (bf16 pattern in the low half) -> fp32 amax; NaN patterns stay NaN
+__device__ __forceinline__ float amax_from_bits(u32 bits16) { return __uint_as_float(bits16 << 16); }
+
+// scale = max(amax, 1e-12) / 448, NaN propagating and canonical
+__device__ __forceinline__ float scale_from_amax(float amax) {
+    if (amax != amax) return __uint_as_float(kCanonNaN);
+    return fmaxf(amax, kAmaxFloor) / kE4M3Max;
+}
+
+// Per reduction set divider.  x / s is needed correctly rounded (the bytes must
+// equal those of an IEEE fp32 division followed by an RNE cast).  With r = 1/s
+// correctly rounded, q0 = x*r, e = fma(-q0, s, x), q1 = fma(e, r, q0) is the
+// correctly rounded quotient wherever it is a normal number (Markstein); below
+// 2^-11 every quotient rounds to a zero byte and only the sign matters, which
+// copysign restores.  Non-finite scales (amax Inf or NaN) take the slow path.
+struct Divider {
+    float s, r;
+    bool finite;
+    __device__ __forceinline__ explicit Divider(float scale) {
+        s = scale;
+        finite = (__float_as_uint(scale) & 0x7F800000u) != 0x7F800000u;
+        r = 1.0f / scale;
+    }
+    // quotient clamped to +-448; valid for finite x when `finite`
+    __device__ __forceinline__ float fast(float x) const {
+        float q0 = x * r;
+        float e = __builtin_fmaf(-q0, s, x);
+        float q1 = __builtin_fmaf(e, r, q0);
+        q1 = __builtin_copysignf(q1, x);
+        return __builtin_amdgcn_fmed3f(q1, -kE4M3Max, kE4M3Max);
+    }
+};
+
+// two fp32 -> two OCP e4m3fn bytes (RNE) in the low or high half of `old`
+template <bool HI>
+__device__ __forceinline__ u32 cvt2(float a, float b, u32 old) {
+    return (u32)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, HI);
+}
+
+// slow path byte for non-finite scales: NaN -> 0x7F, else clamp and convert
+__device__ __forceinline__ u32 slow_byte(float x, float s) {
+    float y = x / s;
+    if (y != y) return 0x7Fu;
+    y = __builtin_amdgcn_fmed3f(y, -kE4M3Max, kE4M3Max);
+    return cvt2<false>(y, 0.0f, 0u) & 0xFFu;
+}
+
+// 8 bf16 (one 16-byte vector) -> 8 fp8 bytes (uint2), element order preserved
+__device__ __forceinline__ uint2 cast8(const uint4& v, const Divider& d) {
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+    u32 o[2];
+    if (d.finite) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            u32 p = cvt2<false>(d.fast(bf16_lo(w[2 * i])), d.fast(bf16_hi(w[2 * i])), 0u);
+            o[i] = cvt2<true>(d.fast(bf16_lo(w[2 * i + 1])), d.fast(bf16_hi(w[2 * i + 1])), p);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            o[i] = slow_byte(bf16_lo(w[2 * i]), d.s) | (slow_byte(bf16_hi(w[2 * i]), d.s) << 8) |
+                   (slow_byte(bf16_lo(w[2 * i + 1]), d.s) << 16) |
+                   (slow_byte(bf16_hi(w[2 * i + 1]), d.s) << 24);
+        }
+    }
+    return make_uint2(o[0], o[1]);
+}
+
+__device__ __forceinline__ u32 absmax8(u32 acc, const uint4& v) {
+    acc = pk_absmax(acc, v.x);
+    acc = pk_absmax(acc, v.y);
+    acc = pk_absmax(acc, v.z);
+    return pk_absmax(acc, v.w);
+}
+
+// fp32 -> bf16 bits, round to nearest even, NaN kept quiet
+__device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
+    u32 u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ u32 pack_bf16x2(float a, float b) {
+    return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+}
+
+}  // namespace cfp8

@@ -1,0 +1,375 @@
+// FP8 (OCP e4m3) GEMMs on the gfx950 matrix cores: rowwise-scaled, 128-block
+// scaled and grouped block-scaled.  One kernel template serves all three.
+//
+//   out[m, n] = sum_k x[m, k] * w[n, k]   (both operands K-major, "nt")
+//
+// MFMA: v_mfma_f32_16x16x128_f8f6f4 (A and B in e4m3).  The weight tile is fed as
+// the MFMA "A" operand and the activation tile as "B", so that a lane's four
+// accumulators are four consecutive n of one output row m: the epilogue stores
+// 8 contiguous bytes of bf16 per lane.  Lane l of a 16x16x128 MFMA supplies row
+// (l & 15) and the 32 K-bytes of quarter (l >> 4) for both operands; any
+// permutation of K shared by both operands leaves the dot products unchanged.
+//
+// Tiles: BM x BN x 128 per workgroup, LDS double-buffered.  An LDS tile is
+// [rows][128 bytes]; the 16-byte chunk c of row r is stored at chunk slot
+// c ^ ((r >> 1) & 7), which makes both the 16-byte stores (8 lanes per row) and
+// the MFMA operand reads (16 lanes = 16 rows, same chunk) bank-conflict free.
+//
+// Scaling: fp32 scales cannot ride in the MFMA (its scale operands are E8M0), so
+//   rowwise:  acc over all of K, epilogue acc * sa[m] * sb[n];
+//   block:    every K step is one 128-block; its MFMA result is folded into the
+//             running sum as acc += part * (sa[m, kb] * sb[n / 128, kb]).
+#include "cfp8_common.h"
+
+namespace cfp8 {
+
+enum : int { kRowwise = 0, kBlock = 1, kGrouped = 2 };
+
+struct GemmArgs {
+    const uint8_t* a;   // activations fp8 [M, K]
+    const uint8_t* b;   // weights fp8 [N, K] (grouped: [E, N, K])
+    const float* sa;    // rowwise [M]; block [M, K/128]
+    const float* sb;    // rowwise [N]; block: see strides
+    const int32_t* m_indices;
+    void* out;
+    int64_t ld_a, ld_b, ld_out;
+    int64_t sb_stride_n, sb_stride_k, sb_stride_e;
+    int M, N, K;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ i32x8 lds_frag(const uint8_t* tile, int row, int quarter) {
+    const int sw = (row >> 1) & 7;
+    const uint8_t* base = tile + row * 128;
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + (((2 * quarter) ^ sw) << 4));
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + (((2 * quarter + 1) ^ sw) << 4));
+    i32x8 r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+}
+
+// Workgroup id -> (tile_m, tile_n).  Consecutive workgroup ids are dealt round
+// robin to the 8 XCDs, each with its own L2: give every XCD one contiguous range
+// of tiles, and walk a range in bands of GM tile-rows so that co-resident
+// workgroups share activation rows and weight rows in that L2.
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    const int lin = xcd * base + (xcd < rem ? xcd : rem) + local;
+    constexpr int GM = 8;
+    const int band = GM * tiles_n;
+    const int g = lin / band, first = g * GM;
+    const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;
+    const int in = lin - g * band;
+    tm = first + in % gsz;
+    tn = in / gsz;
+}
+
+template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs p) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
+    constexpr int TM = WTM / 16, TN = WTN / 16;  // MFMA tiles per wave
+    constexpr int A_CH = BM * 8, B_CH = BN * 8;  // 16-byte chunks per K step
+    constexpr int A_IT = (A_CH + NT - 1) / NT, B_IT = (B_CH + NT - 1) / NT;
+    static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the MFMA tile");
+    static_assert(MODE == kRowwise || WTN <= 128, "a wave's n range must stay inside one 128-block");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int STAGE = (BM + BN) * 128;
+    auto As = [&](int s) { return smem + s * STAGE; };
+    auto Bs = [&](int s) { return smem + s * STAGE + BM * 128; };
+
+    int tm, tn;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const uint8_t* bptr = p.b;
+    const float* sbp = p.sb;
+    int expert = 0;
+    if (MODE == kGrouped) {
+        expert = p.m_indices[m0];  // groups start on multiples of 128 = BM rows
+        if (expert < 0) return;    // a tile of padding (uniform for the workgroup)
+        bptr += (int64_t)expert * p.N * p.ld_b;
+        sbp += (int64_t)expert * p.sb_stride_e;
+    }
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+
+    // global -> register staging of one K step
+    uint4 ra[A_IT], rb[B_IT];
+    auto load_tile = [&](int kt) {
+        const int64_t k = (int64_t)kt << 7;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) {
+            const int id = t + NT * i;
+            const int r = id >> 3, c = id & 7;
+            const bool ok = (A_CH % NT == 0 || id < A_CH) && (m0 + r) < p.M;
+            ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + (int64_t)(m0 + r) * p.ld_a + k + c * 16)
+                       : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) {
+            const int id = t + NT * i;
+            const int r = id >> 3, c = id & 7;
+            const bool ok = (B_CH % NT == 0 || id < B_CH) && (n0 + r) < p.N;
+            rb[i] = ok ? *reinterpret_cast<const uint4*>(bptr + (int64_t)(n0 + r) * p.ld_b + k + c * 16)
+                       : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto store_tile = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) {
+            const int id = t + NT * i;
+            const int r = id >> 3, c = id & 7;
+            if (A_CH % NT == 0 || id < A_CH)
+                *reinterpret_cast<uint4*>(As(stage) + r * 128 + ((c ^ ((r >> 1) & 7)) << 4)) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) {
+            const int id = t + NT * i;
+            const int r = id >> 3, c = id & 7;
+            if (B_CH % NT == 0 || id < B_CH)
+                *reinterpret_cast<uint4*>(Bs(stage) + r * 128 + ((c ^ ((r >> 1) & 7)) << 4)) = rb[i];
+        }
+    };
+
+    f32x4 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) load_tile(kt + 1);
+
+        float s_m[TM];
+        float s_n = 0.f;
+        if (MODE != kRowwise) {
+            const int KB = KT;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int m = m0 + wm * WTM + j * 16 + lrow;
+                s_m[j] = m < p.M ? p.sa[(int64_t)m * KB + kt] : 0.f;
+            }
+            const int nb = (n0 + wn * WTN) >> 7;
+            s_n = sbp[(int64_t)nb * p.sb_stride_n + (int64_t)kt * p.sb_stride_k];
+        }
+
+        // weight fragments stay live for the whole step; activation fragments are
+        // read one 16-row tile at a time to bound register pressure
+        i32x8 fa[TN];
+#pragma unroll
+        for (int i = 0; i < TN; ++i) fa[i] = lds_frag(Bs(cur), wn * WTN + i * 16 + lrow, quarter);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const i32x8 fb = lds_frag(As(cur), wm * WTM + j * 16 + lrow, quarter);
+            if (MODE == kRowwise) {
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, acc[i][j], 0, 0, 0, 0, 0, 0);
+            } else {
+                const float s = s_m[j] * s_n;
+#pragma unroll
+                for (int i = 0; i < TN; ++i) {
+                    const f32x4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        fa[i], fb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], s, acc[i][j][e]);
+                }
+            }
+        }
+
+        if (kt + 1 < KT) store_tile(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int m = m0 + wm * WTM + j * 16 + lrow;
+        if (m >= p.M) continue;
+        if (MODE == kGrouped && p.m_indices[m] != expert) continue;
+        float sam = 1.f;
+        if (MODE == kRowwise) sam = p.sa[m];
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int n = n0 + wn * WTN + i * 16 + quarter * 4;
+            if (n >= p.N) continue;  // N % 16 == 0: a group of four is inside or outside as a whole
+            f32x4 v = acc[i][j];
+            if (MODE == kRowwise) {
+                const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam * sbn[e];
+            }
+            if (OUT_F32) {
+                *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            } else {
+                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int MODE>
+static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    constexpr int NT = WM * WN * 64;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
+    auto kf = gemm_kernel<BM, BN, WM, WN, MODE, true>;
+    auto kb = gemm_kernel<BM, BN, WM, WN, MODE, false>;
+    if (lds > 64 * 1024) {
+        static bool done_f = false, done_b = false;
+        bool& done = out_dtype == CFP8_OUT_F32 ? done_f : done_b;
+        if (!done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(out_dtype == CFP8_OUT_F32 ? kf : kb),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            done = true;
+        }
+    }
+    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(NT), lds, st, p);
+    else hipLaunchKernelGGL(kb, dim3((unsigned)blocks), dim3(NT), lds, st, p);
+    return check_launch("gemm");
+}
+
+template <int MODE>
+static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
+    if (MODE == kGrouped) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
+    if (p.M <= 16) return launch_cfg<16, 64, 1, 4, MODE>(p, out_dtype, st);
+    if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
+    if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
+    return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);
+}
+
+static int check_common(const char* who, const void* a, const void* b, const float* sa, const float* sb,
+                        const void* out, int64_t ld_a, int64_t ld_b, int64_t ld_out, int out_dtype, int64_t M,
+                        int64_t N, int64_t K) {
+    if (M < 0 || N < 0 || K < 0) return set_error(CFP8_EINVAL, "%s: negative shape", who);
+    if (M == 0 || N == 0) return CFP8_OK;  // nothing to compute: pointers may be null
+    if (!a || !b || !sa || !sb || !out) return set_error(CFP8_EINVAL, "%s: null pointer", who);
+    if (K % 128 || N % 16) return set_error(CFP8_EINVAL, "%s: K=%lld must be a multiple of 128 and N=%lld of 16", who, (long long)K, (long long)N);
+    if (ld_a % 16 || ld_b % 16 || ld_a < K || ld_b < K || ld_out < N || ld_out % 4)
+        return set_error(CFP8_EINVAL, "%s: bad leading dimension (ld_a=%lld ld_b=%lld ld_out=%lld)", who, (long long)ld_a, (long long)ld_b, (long long)ld_out);
+    if (!aligned16(a) || !aligned16(b) || !aligned16(out) || !aligned16(sb))
+        return set_error(CFP8_EINVAL, "%s: operands must be 16-byte aligned", who);
+    if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "%s: unknown out_dtype %d", who, out_dtype);
+    if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "%s: dimension exceeds int32", who);
+    return CFP8_OK;
+}
+
+int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
+                         float* scales, hipStream_t st);
+
+}  // namespace cfp8
+
+extern "C" int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* sa, const void* b, int64_t ld_b,
+                                      const float* sb, void* out, int64_t ld_out, int out_dtype, int64_t M,
+                                      int64_t N, int64_t K, void* stream) {
+    using namespace cfp8;
+    if (int rc = check_common("scaled_mm_rowwise", a, b, sa, sb, out, ld_a, ld_b, ld_out, out_dtype, M, N, K)) return rc;
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (K == 0) return set_error(CFP8_EINVAL, "scaled_mm_rowwise: K must be positive");
+    if (int rc = check_device()) return rc;
+    GemmArgs p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.sa = sa;
+    p.sb = sb;
+    p.out = out;
+    p.ld_a = ld_a; p.ld_b = ld_b; p.ld_out = ld_out;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    return launch_gemm<kRowwise>(p, out_dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t cfp8_linear_workspace_bytes(int64_t M, int64_t K) {
+    if (M <= 0 || K <= 0) return 0;
+    const size_t q = ((size_t)M * (size_t)K + 255) & ~(size_t)255;
+    return q + (((size_t)M * 4 + 255) & ~(size_t)255);
+}
+
+extern "C" int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, int64_t ld_w, const float* w_scale,
+                                   void* out, int64_t ld_out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace cfp8;
+    if (M < 0 || N < 0 || K <= 0) return set_error(CFP8_EINVAL, "linear_rowwise: bad shape");
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (!workspace || workspace_bytes < cfp8_linear_workspace_bytes(M, K))
+        return set_error(CFP8_EWORKSPACE, "linear_rowwise: workspace of %zu bytes needed, %zu given", cfp8_linear_workspace_bytes(M, K), workspace_bytes);
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u) return set_error(CFP8_EINVAL, "linear_rowwise: workspace must be 256-byte aligned");
+    if (!x || !aligned16(x) || ld_x % 8 || ld_x < K) return set_error(CFP8_EINVAL, "linear_rowwise: bad activation pointer or leading dimension");
+    uint8_t* qx = static_cast<uint8_t*>(workspace);
+    float* sx = reinterpret_cast<float*>(qx + (((size_t)M * (size_t)K + 255) & ~(size_t)255));
+    if (int rc = check_common("linear_rowwise", qx, w, sx, w_scale, out, K, ld_w, ld_out, out_dtype, M, N, K)) return rc;
+    if (int rc = check_device()) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (int rc = launch_quant_rowwise(x, M, K, ld_x, qx, K, sx, st)) return rc;
+    GemmArgs p{};
+    p.a = qx;
+    p.b = static_cast<const uint8_t*>(w);
+    p.sa = sx;
+    p.sb = w_scale;
+    p.out = out;
+    p.ld_a = K; p.ld_b = ld_w; p.ld_out = ld_out;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    return launch_gemm<kRowwise>(p, out_dtype, st);
+}
+
+extern "C" int cfp8_gemm_block128(const void* a, int64_t ld_a, const float* sa, const void* b, int64_t ld_b,
+                                  const float* sb, int64_t sb_stride_n, int64_t sb_stride_k, void* out,
+                                  int64_t ld_out, int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+    using namespace cfp8;
+    if (int rc = check_common("gemm_block128", a, b, sa, sb, out, ld_a, ld_b, ld_out, out_dtype, M, N, K)) return rc;
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (K == 0) return set_error(CFP8_EINVAL, "gemm_block128: K must be positive");
+    if (int rc = check_device()) return rc;
+    GemmArgs p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.sa = sa;
+    p.sb = sb;
+    p.out = out;
+    p.ld_a = ld_a; p.ld_b = ld_b; p.ld_out = ld_out;
+    p.sb_stride_n = sb_stride_n; p.sb_stride_k = sb_stride_k;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    return launch_gemm<kBlock>(p, out_dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cfp8_gemm_grouped_block128(const void* a, int64_t ld_a, const float* sa, const void* b,
+                                          const float* sb, const int32_t* m_indices, void* out, int64_t ld_out,
+                                          int out_dtype, int64_t M, int64_t N, int64_t K, int64_t E, void* stream) {
+    using namespace cfp8;
+    if (int rc = check_common("gemm_grouped_block128", a, b, sa, sb, out, ld_a, K, ld_out, out_dtype, M, N, K)) return rc;
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (!m_indices) return set_error(CFP8_EINVAL, "gemm_grouped_block128: null m_indices");
+    if (E <= 0) return set_error(CFP8_EINVAL, "gemm_grouped_block128: E must be positive");
+    if (M % 128) return set_error(CFP8_EINVAL, "gemm_grouped_block128: M=%lld must be a multiple of the 128-row group alignment", (long long)M);
+    if (K == 0) return set_error(CFP8_EINVAL, "gemm_grouped_block128: K must be positive");
+    if (int rc = check_device()) return rc;
+    GemmArgs p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.sa = sa;
+    p.sb = sb;
+    p.m_indices = m_indices;
+    p.out = out;
+    p.ld_a = ld_a; p.ld_b = K; p.ld_out = ld_out;
+    const int64_t nb = (N + 127) / 128, kb = K / 128;
+    p.sb_stride_n = kb; p.sb_stride_k = 1; p.sb_stride_e = nb * kb;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    return launch_gemm<kGrouped>(p, out_dtype, static_cast<hipStream_t>(stream));
+}

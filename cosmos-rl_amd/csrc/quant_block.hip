@@ -1,0 +1,257 @@
+// 128x128 block quantisation (weights), 1x128 group quantisation (activations)
+// and the block dequantiser.  All three are HBM-bound streaming kernels.
+#include "cfp8_common.h"
+
+namespace cfp8 {
+
+// ---------------------------------------------------------------------------
+// 128x128 blocks.  One 256-thread workgroup per tile; thread (rg, cv) holds the
+// 8 consecutive rows rg*8.. and the 8 consecutive columns cv*8.. of the tile as
+// packed bf16 (32 VGPRs), so the tile is read from HBM once.  For every row,
+// 16 lanes read 256 contiguous bytes.
+// Plain output: 8-byte stores, 128 contiguous bytes per row.
+// Transposed output ([cols, rows], the K-major operand of the block GEMM): the
+// fp8 tile is turned in LDS (128 x 144 bytes) and leaves as 16-byte stores,
+// 128 contiguous bytes per output row.
+// ---------------------------------------------------------------------------
+constexpr int kTStride = 144;  // bytes per LDS row of the transposed tile (16-byte aligned)
+
+template <bool TRANSPOSE>
+__global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restrict__ x, int64_t rows, int64_t cols,
+                                                       uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                       int tiles_r, int tiles_c) {
+    __shared__ u32 red[4];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[TRANSPOSE ? 128 * kTStride : 16];
+    const int t = threadIdx.x;
+    const int cv = t & 15, rg = t >> 4;
+    const int64_t b = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * 128, c0 = (int64_t)blockIdx.x * 128;
+    const uint16_t* xb = x + b * rows * cols;
+    const int64_t col = c0 + cv * 8;
+    const bool col_ok = col < cols;  // cols % 8 == 0: a vector is inside or outside as a whole
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int64_t r = r0 + rg * 8 + i;
+        v[i] = (col_ok && r < rows) ? *reinterpret_cast<const uint4*>(xb + r * cols + col) : make_uint4(0, 0, 0, 0);
+    }
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = absmax8(m, v[i]);
+    m = wave_max(pk_fold(m));
+    if ((t & 63) == 0) red[t >> 6] = m;
+    __syncthreads();
+    const float amax = amax_from_bits(umax(umax(red[0], red[1]), umax(red[2], red[3])));
+    const float scale = scale_from_amax(amax);
+    if (t == 0) scales[(b * tiles_r + blockIdx.y) * tiles_c + blockIdx.x] = scale;
+    const Divider d(scale);
+    if (!TRANSPOSE) {
+        uint8_t* qb = q + b * rows * cols;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t r = r0 + rg * 8 + i;
+            if (col_ok && r < rows) *reinterpret_cast<uint2*>(qb + r * cols + col) = cast8(v[i], d);
+        }
+    } else {
+        // bytes[i] = row i, 8 columns; regroup to 8 rows of one column (8 bytes) per LDS store
+        uint2 bytes[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bytes[i] = cast8(v[i], d);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            u32 lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32 wlo = j < 4 ? bytes[i].x : bytes[i].y;
+                const u32 whi = j < 4 ? bytes[i + 4].x : bytes[i + 4].y;
+                lo |= ((wlo >> (8 * (j & 3))) & 0xFFu) << (8 * i);
+                hi |= ((whi >> (8 * (j & 3))) & 0xFFu) << (8 * i);
+            }
+            *reinterpret_cast<uint2*>(&tile[(cv * 8 + j) * kTStride + rg * 8]) = make_uint2(lo, hi);
+        }
+        __syncthreads();
+        uint8_t* qb = q + b * rows * cols;  // [cols, rows]
+        const int chunk = t & 7;            // 16 rows of the tile per chunk
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int c = (t >> 3) + 32 * p;
+            const int64_t oc = c0 + c, orow = r0 + chunk * 16;
+            if (oc < cols && orow < rows)  // rows % 16 == 0: a chunk is inside or outside as a whole
+                *reinterpret_cast<uint4*>(qb + oc * rows + orow) =
+                    *reinterpret_cast<const uint4*>(&tile[c * kTStride + chunk * 16]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// 1x128 groups.  16 lanes own one group (one 16-byte vector each), the max runs
+// over the 16-lane DPP row.  Every thread handles 4 groups of 4 consecutive
+// group-rows so that four loads are in flight per lane.
+// ---------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__ x, int64_t rows, int nvec,
+                                                       int ngroups, int64_t ldx, uint2* __restrict__ q, int64_t ldq,
+                                                       float* __restrict__ scales, int64_t total_groups) {
+    const int sub = threadIdx.x & 15;
+    const int64_t g0 = ((int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)) * 4;
+    uint4 v[4];
+    int64_t row[4];
+    int gcol[4];
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int64_t g = g0 + i;
+        row[i] = g / ngroups;
+        gcol[i] = (int)(g - row[i] * ngroups);
+        const int vec = gcol[i] * 16 + sub;
+        ok[i] = g < total_groups && vec < nvec;
+        v[i] = ok[i] ? x[row[i] * ldx + vec] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32 m = row16_max(pk_fold(absmax8(0u, v[i])));
+        const float amax = amax_from_bits(m);
+        uint2 out;
+        float scale;
+        if (MODE == CFP8_GROUP_MODE_DIV) {
+            scale = scale_from_amax(amax);
+            const Divider d(scale);
+            out = cast8(v[i], d);
+        } else {
+            // x * (448 / clamp(amax, 1e-4)) as torch evaluates `448.0 / tensor`:
+            // reciprocal first, then times 448.  No clamp before the cast: the product
+            // exceeds 448 by at most a few fp32 roundings, far below the NaN threshold 464
+            if (amax != amax) {
+                scale = __uint_as_float(kCanonNaN);
+                out = make_uint2(0x7F7F7F7Fu, 0x7F7F7F7Fu);
+            } else {
+                const float a = fmaxf(amax, 1e-4f);
+                const float mul = (1.0f / a) * kE4M3Max;
+                scale = a / kE4M3Max;
+                const u32 w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+                u32 o[2];
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    u32 p = cvt2<false>(bf16_lo(w[2 * k]) * mul, bf16_hi(w[2 * k]) * mul, 0u);
+                    o[k] = cvt2<true>(bf16_lo(w[2 * k + 1]) * mul, bf16_hi(w[2 * k + 1]) * mul, p);
+                }
+                out = make_uint2(o[0], o[1]);
+            }
+        }
+        if (ok[i]) q[row[i] * ldq + gcol[i] * 16 + sub] = out;
+        if (sub == 0 && g0 + i < total_groups) scales[row[i] * ngroups + gcol[i]] = scale;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// block dequantiser: y[i, j] = fp8[i, j] * s[i / 128, j / 128]
+// ---------------------------------------------------------------------------
+template <typename OutVec, bool F32>
+__global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __restrict__ q,
+                                                               const float* __restrict__ s, int64_t rows,
+                                                               int64_t cols, int tiles_c, void* __restrict__ y) {
+    const int64_t nvec_row = cols / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= rows * nvec_row) return;
+    const int64_t r = idx / nvec_row, cv = idx - r * nvec_row;
+    const uint2 w = *reinterpret_cast<const uint2*>(q + r * cols + cv * 8);
+    const float sc = s[(r >> 7) * tiles_c + (cv >> 4)];
+    float f[8];
+    f32x2 p;
+    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, false); f[0] = p[0]; f[1] = p[1];
+    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, true);  f[2] = p[0]; f[3] = p[1];
+    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, false); f[4] = p[0]; f[5] = p[1];
+    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, true);  f[6] = p[0]; f[7] = p[1];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] *= sc;
+    if (F32) {
+        float4* o = reinterpret_cast<float4*>(static_cast<float*>(y) + r * cols + cv * 8);
+        o[0] = make_float4(f[0], f[1], f[2], f[3]);
+        o[1] = make_float4(f[4], f[5], f[6], f[7]);
+    } else {
+        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(y) + r * cols + cv * 8);
+        *o = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                        pack_bf16x2(f[6], f[7]));
+    }
+}
+
+int launch_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
+                          float* scales, int mode, hipStream_t st) {
+    const int64_t ngroups = (cols + 127) / 128;
+    const int64_t total = rows * ngroups;
+    const int64_t blocks = (total + 63) / 64;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_group128: too many groups for one launch");
+    const uint4* xv = static_cast<const uint4*>(x);
+    uint2* qv = static_cast<uint2*>(q);
+    if (mode == CFP8_GROUP_MODE_DIV)
+        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DIV>, dim3((unsigned)blocks), dim3(256), 0, st, xv, rows,
+                           (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
+    else
+        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DEEPEP>, dim3((unsigned)blocks), dim3(256), 0, st, xv,
+                           rows, (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
+    return check_launch("quant_group128");
+}
+
+}  // namespace cfp8
+
+extern "C" int cfp8_quant_block128(const void* x, int64_t batch, int64_t rows, int64_t cols, void* q,
+                                   float* scales, int transpose_out, void* stream) {
+    using namespace cfp8;
+    if (batch < 0 || rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "quant_block128: negative shape");
+    if (batch == 0 || rows == 0 || cols == 0) return CFP8_OK;
+    if (!x || !q || !scales) return set_error(CFP8_EINVAL, "quant_block128: null pointer");
+    if (cols % 8) return set_error(CFP8_EINVAL, "quant_block128: cols=%lld must be a multiple of 8", (long long)cols);
+    if (transpose_out && rows % 16) return set_error(CFP8_EINVAL, "quant_block128: rows=%lld must be a multiple of 16 for the transposed output", (long long)rows);
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & (transpose_out ? 15u : 7u)))
+        return set_error(CFP8_EINVAL, "quant_block128: misaligned pointer");
+    const int64_t tr = (rows + 127) / 128, tc = (cols + 127) / 128;
+    if (tr > 65535 || batch > 65535 || tc > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_block128: shape exceeds the grid limits");
+    if (int rc = check_device()) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 grid((unsigned)tc, (unsigned)tr, (unsigned)batch);
+    if (transpose_out)
+        hipLaunchKernelGGL(block128_kernel<true>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, cols,
+                           static_cast<uint8_t*>(q), scales, (int)tr, (int)tc);
+    else
+        hipLaunchKernelGGL(block128_kernel<false>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(x), rows, cols,
+                           static_cast<uint8_t*>(q), scales, (int)tr, (int)tc);
+    return check_launch("quant_block128");
+}
+
+extern "C" int cfp8_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q,
+                                   int64_t ld_q, float* scales, int mode, void* stream) {
+    using namespace cfp8;
+    if (rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "quant_group128: negative shape");
+    if (rows == 0 || cols == 0) return CFP8_OK;
+    if (!x || !q || !scales) return set_error(CFP8_EINVAL, "quant_group128: null pointer");
+    if (mode != CFP8_GROUP_MODE_DIV && mode != CFP8_GROUP_MODE_DEEPEP) return set_error(CFP8_EINVAL, "quant_group128: unknown mode %d", mode);
+    if (cols % 8 || ld_x % 8 || ld_q % 8 || ld_x < cols || ld_q < cols)
+        return set_error(CFP8_EINVAL, "quant_group128: cols=%lld ld_x=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
+                         (long long)cols, (long long)ld_x, (long long)ld_q);
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "quant_group128: misaligned pointer");
+    if (int rc = check_device()) return rc;
+    return launch_quant_group128(x, rows, cols, ld_x, q, ld_q, scales, mode, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cfp8_dequant_block128(const void* q, const float* scales, int64_t rows, int64_t cols, void* y,
+                                     int out_dtype, void* stream) {
+    using namespace cfp8;
+    if (rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "dequant_block128: negative shape");
+    if (rows == 0 || cols == 0) return CFP8_OK;
+    if (!q || !scales || !y) return set_error(CFP8_EINVAL, "dequant_block128: null pointer");
+    if (cols % 8) return set_error(CFP8_EINVAL, "dequant_block128: cols=%lld must be a multiple of 8", (long long)cols);
+    if ((reinterpret_cast<uintptr_t>(q) & 7u) || !aligned16(y)) return set_error(CFP8_EINVAL, "dequant_block128: misaligned pointer");
+    if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "dequant_block128: unknown out_dtype %d", out_dtype);
+    const int64_t blocks = (rows * (cols / 8) + 255) / 256;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "dequant_block128: too large for one launch");
+    if (int rc = check_device()) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int tc = (int)((cols + 127) / 128);
+    if (out_dtype == CFP8_OUT_F32)
+        hipLaunchKernelGGL((dequant_block128_kernel<float4, true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                           static_cast<const uint8_t*>(q), scales, rows, cols, tc, y);
+    else
+        hipLaunchKernelGGL((dequant_block128_kernel<uint4, false>), dim3((unsigned)blocks), dim3(256), 0, st,
+                           static_cast<const uint8_t*>(q), scales, rows, cols, tc, y);
+    return check_launch("dequant_block128");
+}

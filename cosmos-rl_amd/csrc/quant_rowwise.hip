@@ -1,0 +1,137 @@
+// Rowwise dynamic FP8 quantisation: per row amax -> scale -> e4m3.
+//
+// HBM-bound: 2 bytes read and 1 byte written per element plus 4 bytes per row.
+// Each row is read from HBM once: it is held in registers as packed bf16
+// between the amax sweep and the cast sweep.
+//   * rows of up to 4096 elements: one 64-lane wavefront per row, no LDS, no
+//     barrier; four rows per 256-thread workgroup.
+//   * rows of up to 32768 elements: one workgroup per row, cross-wave max
+//     through LDS.
+//   * longer rows: one workgroup per row, second sweep re-reads the row.
+#include "cfp8_common.h"
+
+namespace cfp8 {
+
+template <int V>
+__global__ __launch_bounds__(256) void rowwise_wave_kernel(const uint4* __restrict__ x, int64_t rows,
+                                                           int nvec, int64_t ldx, uint2* __restrict__ q,
+                                                           int64_t ldq, float* __restrict__ scales) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;  // wave-uniform
+    const uint4* xr = x + row * ldx;
+    uint4 v[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        int idx = lane + 64 * i;
+        v[i] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+    }
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) m = absmax8(m, v[i]);
+    const float amax = amax_from_bits(wave_max(pk_fold(m)));
+    const float scale = scale_from_amax(amax);
+    if (lane == 0) scales[row] = scale;
+    const Divider d(scale);
+    uint2* qr = q + row * ldq;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        int idx = lane + 64 * i;
+        if (idx < nvec) qr[idx] = cast8(v[i], d);
+    }
+}
+
+__device__ __forceinline__ u32 block_max_256(u32 wave_val, u32* lds) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds[wave] = wave_val;
+    __syncthreads();
+    return umax(umax(lds[0], lds[1]), umax(lds[2], lds[3]));
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void rowwise_block_kernel(const uint4* __restrict__ x, int nvec,
+                                                            int64_t ldx, uint2* __restrict__ q,
+                                                            int64_t ldq, float* __restrict__ scales) {
+    __shared__ u32 red[4];
+    const int64_t row = blockIdx.x;
+    const int t = threadIdx.x;
+    const uint4* xr = x + row * ldx;
+    uint4 v[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        int idx = t + 256 * i;
+        v[i] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+    }
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < V; ++i) m = absmax8(m, v[i]);
+    const float amax = amax_from_bits(block_max_256(wave_max(pk_fold(m)), red));
+    const float scale = scale_from_amax(amax);
+    if (t == 0) scales[row] = scale;
+    const Divider d(scale);
+    uint2* qr = q + row * ldq;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        int idx = t + 256 * i;
+        if (idx < nvec) qr[idx] = cast8(v[i], d);
+    }
+}
+
+__global__ __launch_bounds__(256) void rowwise_stream_kernel(const uint4* __restrict__ x, int64_t nvec,
+                                                             int64_t ldx, uint2* __restrict__ q,
+                                                             int64_t ldq, float* __restrict__ scales) {
+    __shared__ u32 red[4];
+    const int64_t row = blockIdx.x;
+    const int t = threadIdx.x;
+    const uint4* xr = x + row * ldx;
+    u32 m = 0;
+    for (int64_t idx = t; idx < nvec; idx += 256) m = absmax8(m, xr[idx]);
+    const float amax = amax_from_bits(block_max_256(wave_max(pk_fold(m)), red));
+    const float scale = scale_from_amax(amax);
+    if (t == 0) scales[row] = scale;
+    const Divider d(scale);
+    uint2* qr = q + row * ldq;
+    for (int64_t idx = t; idx < nvec; idx += 256) qr[idx] = cast8(xr[idx], d);
+}
+
+int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
+                         float* scales, hipStream_t st) {
+    const uint4* xv = static_cast<const uint4*>(x);
+    uint2* qv = static_cast<uint2*>(q);
+    const int64_t nvec = cols / 8, ldx = ld_x / 8, ldq = ld_q / 8;
+    if (rows > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_rowwise: rows=%lld exceeds the grid limit", (long long)rows);
+#define CFP8_WAVE(V)                                                                                   \
+    hipLaunchKernelGGL(rowwise_wave_kernel<V>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, xv, \
+                       rows, (int)nvec, ldx, qv, ldq, scales)
+#define CFP8_BLOCK(V) \
+    hipLaunchKernelGGL(rowwise_block_kernel<V>, dim3((unsigned)rows), dim3(256), 0, st, xv, (int)nvec, ldx, qv, ldq, scales)
+    if (nvec <= 64) CFP8_WAVE(1);
+    else if (nvec <= 128) CFP8_WAVE(2);
+    else if (nvec <= 256) CFP8_WAVE(4);
+    else if (nvec <= 512) CFP8_WAVE(8);
+    else if (nvec <= 1024) CFP8_BLOCK(4);
+    else if (nvec <= 2048) CFP8_BLOCK(8);
+    else if (nvec <= 4096) CFP8_BLOCK(16);
+    else
+        hipLaunchKernelGGL(rowwise_stream_kernel, dim3((unsigned)rows), dim3(256), 0, st, xv, nvec, ldx, qv, ldq, scales);
+#undef CFP8_WAVE
+#undef CFP8_BLOCK
+    return check_launch("quant_rowwise");
+}
+
+}  // namespace cfp8
+
+extern "C" int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q,
+                                  int64_t ld_q, float* scales, void* stream) {
+    using namespace cfp8;
+    if (rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "quant_rowwise: negative shape");
+    if (rows == 0) return CFP8_OK;
+    if (!x || !q || !scales) return set_error(CFP8_EINVAL, "quant_rowwise: null pointer");
+    if (cols % 8 || ld_x % 8 || ld_q % 8 || ld_x < cols || ld_q < cols)
+        return set_error(CFP8_EINVAL, "quant_rowwise: cols=%lld ld_x=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
+                         (long long)cols, (long long)ld_x, (long long)ld_q);
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u))
+        return set_error(CFP8_EINVAL, "quant_rowwise: x must be 16-byte and q 8-byte aligned");
+    if (int rc = check_device()) return rc;
+    return launch_quant_rowwise(x, rows, cols, ld_x, q, ld_q, scales, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,178 @@
+// Tensorwise dynamic FP8 quantisation of many tensors: two launches per batch of
+// up to 48 tensors (and a bounded number of bytes), no host round trip between them.
+//
+//   pass 1 (amax)  reads 2 B/element.  Every workgroup reduces one contiguous
+//                  chunk of one tensor and publishes its maximum with one
+//                  atomic max on the bit pattern (valid because |x| >= 0, and
+//                  NaN patterns sort above infinity, so NaN propagates).
+//   pass 2 (cast)  reads 2 B and writes 1 B per element; every workgroup forms
+//                  the scale from the tensor's amax slot on its own.
+// The table of tensors travels in the kernel arguments (scalar loads), so the
+// library needs no device-side descriptor buffer.
+#include <stdlib.h>
+
+#include "cfp8_common.h"
+
+namespace cfp8 {
+
+constexpr int kMaxBatch = 48;
+constexpr int kChunkVecs = 256 * 8;  // 16-byte vectors per workgroup: 32 KiB of bf16
+
+struct TensorTable {
+    const uint4* x[kMaxBatch];
+    uint2* q[kMaxBatch];
+    float* scale[kMaxBatch];
+    int64_t nvec[kMaxBatch];
+    u32* amax[kMaxBatch];
+    unsigned first_block[kMaxBatch + 1];  // exclusive prefix of workgroups per tensor
+    int n;
+};
+
+__device__ __forceinline__ int find_tensor(const TensorTable& tb, unsigned b) {
+    int lo = 0, hi = tb.n - 1;
+    while (lo < hi) {  // last t with first_block[t] <= b; uniform across the workgroup
+        int mid = (lo + hi + 1) >> 1;
+        if (tb.first_block[mid] <= b) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+__global__ __launch_bounds__(64) void tensorwise_zero_kernel(u32* slots, int n) {
+    for (int i = threadIdx.x; i < n; i += 64) slots[i] = 0u;
+}
+
+__global__ __launch_bounds__(256) void tensorwise_amax_kernel(const TensorTable tb) {
+    __shared__ u32 red[4];
+    const int t = find_tensor(tb, blockIdx.x);
+    const int64_t base = (int64_t)(blockIdx.x - tb.first_block[t]) * kChunkVecs;
+    const int64_t nvec = tb.nvec[t];
+    const uint4* x = tb.x[t] + base;
+    const int64_t left = nvec - base;
+    uint4 v[8];
+    if (left >= kChunkVecs) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = x[threadIdx.x + 256 * i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int idx = threadIdx.x + 256 * i;
+            v[i] = idx < left ? x[idx] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m = absmax8(m, v[i]);
+    m = wave_max(pk_fold(m));
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;  // fp32 bit pattern of the chunk amax
+        u32* slot = tb.amax[t];
+        // the slot only grows, so a stale read can only cause a redundant atomic
+        if (m > __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(slot, m);
+    }
+}
+
+__global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable tb) {
+    const int t = find_tensor(tb, blockIdx.x);
+    const unsigned local = blockIdx.x - tb.first_block[t];
+    const int64_t base = (int64_t)local * kChunkVecs;
+    const int64_t nvec = tb.nvec[t];
+    const uint4* x = tb.x[t] + base;
+    uint2* q = tb.q[t] + base;
+    const int64_t left = nvec - base;
+    const float amax = __uint_as_float(*tb.amax[t]);
+    const float scale = scale_from_amax(amax);
+    if (local == 0 && threadIdx.x == 0) *tb.scale[t] = scale;
+    const Divider d(scale);
+    uint4 v[8];
+    if (left >= kChunkVecs) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = x[threadIdx.x + 256 * i];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[threadIdx.x + 256 * i] = cast8(v[i], d);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int idx = threadIdx.x + 256 * i;
+            if (idx < left) q[idx] = cast8(x[idx], d);
+        }
+    }
+}
+
+// bf16 bytes per batch; CFP8_TW_BATCH_MB overrides the default (read once)
+static int64_t batch_bytes() {
+    static int64_t v = [] {
+        const char* e = getenv("CFP8_TW_BATCH_MB");
+        long mb = e ? atol(e) : 0;
+        if (mb <= 0) mb = 160;
+        return (int64_t)mb << 20;
+    }();
+    return v;
+}
+
+}  // namespace cfp8
+
+extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws,
+                                           void* stream) {
+    using namespace cfp8;
+    if (n < 0) return set_error(CFP8_EINVAL, "quant_tensorwise: negative tensor count");
+    if (n == 0) return CFP8_OK;
+    if (!descs || !amax_ws) return set_error(CFP8_EINVAL, "quant_tensorwise: null descriptor table or amax workspace");
+    for (int64_t i = 0; i < n; ++i) {
+        const cfp8_tensor_desc& d = descs[i];
+        if (d.numel < 0 || d.numel % 8) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld numel=%lld must be a non-negative multiple of 8", (long long)i, (long long)d.numel);
+        if (!d.scale) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null scale pointer", (long long)i);
+        if (d.numel && (!d.x || !d.q)) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null data pointer", (long long)i);
+        if (!aligned16(d.x) || (reinterpret_cast<uintptr_t>(d.q) & 7u)) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld is misaligned (x 16 bytes, q 8 bytes)", (long long)i);
+        if ((d.numel / 8 + kChunkVecs - 1) / kChunkVecs > 0x3FFFFFFFll) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld is too large for one launch", (long long)i);
+    }
+    if (int rc = check_device()) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    u32* slots = reinterpret_cast<u32*>(amax_ws);
+    // zero every slot with a kernel (a memset node misbehaves under graph capture)
+    for (int64_t off = 0; off < n; off += 1 << 20) {
+        int cnt = (int)((n - off) < (1 << 20) ? (n - off) : (1 << 20));
+        hipLaunchKernelGGL(tensorwise_zero_kernel, dim3(1), dim3(64), 0, st, slots + off, cnt);
+    }
+    // Tensors are taken in batches of at most kMaxBatch entries and batch_bytes()
+    // of bf16; each batch runs pass 1 then pass 2 back to back, so a batch that
+    // fits the 256 MiB memory-side cache is read from HBM once.
+    const int64_t budget_vecs = batch_bytes() / 16;
+    int64_t i = 0;
+    while (i < n) {
+        TensorTable tb;
+        tb.n = 0;
+        unsigned blocks = 0;
+        int64_t vecs = 0;
+        while (i < n && tb.n < kMaxBatch) {
+            const cfp8_tensor_desc& d = descs[i];
+            int64_t nvec = d.numel / 8;
+            // a tensor with no element still owns one workgroup: it writes the scale
+            unsigned nb = (unsigned)((nvec + kChunkVecs - 1) / kChunkVecs);
+            if (nb == 0) nb = 1;
+            if (tb.n > 0 && ((uint64_t)blocks + nb > 0x7FFFFFFFull || vecs + nvec > budget_vecs)) break;
+            tb.x[tb.n] = static_cast<const uint4*>(d.x);
+            tb.q[tb.n] = static_cast<uint2*>(d.q);
+            tb.scale[tb.n] = d.scale;
+            tb.nvec[tb.n] = nvec;
+            tb.amax[tb.n] = slots + i;
+            tb.first_block[tb.n] = blocks;
+            blocks += nb;
+            vecs += nvec;
+            ++tb.n;
+            ++i;
+        }
+        tb.first_block[tb.n] = blocks;
+        hipLaunchKernelGGL(tensorwise_amax_kernel, dim3(blocks), dim3(256), 0, st, tb);
+        hipLaunchKernelGGL(tensorwise_cast_kernel, dim3(blocks), dim3(256), 0, st, tb);
+    }
+    return check_launch("quant_tensorwise");
+}
+
+extern "C" int cfp8_quant_tensorwise(const void* x, int64_t numel, void* q, float* scale, float* amax_ws,
+                                     void* stream) {
+    cfp8_tensor_desc d{x, q, scale, numel};
+    return cfp8_quant_tensorwise_multi(&d, 1, amax_ws, stream);
+}

@@ -1,0 +1,157 @@
+/* libcosmosfp8 - C ABI of the MI355X (gfx950) FP8 hot path.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream
+ * (hipStream_t passed as void*; NULL = the null stream).  The library never
+ * allocates or frees device memory through these calls, never synchronises the
+ * device and never reads a result back to the host; the caller owns every
+ * buffer, including workspaces.  Return value: 0 on success, a negative
+ * CFP8_E* code otherwise; cfp8_last_error() returns a thread-local message for
+ * the last failure on the calling thread.
+ *
+ * Common contract: bf16 inputs are row-major with the stated leading
+ * dimension (in elements), base pointers 16-byte aligned, leading dimensions
+ * and column counts multiples of 8 for bf16 / 16 for fp8 unless stated.
+ * fp8 = OCP e4m3fn (max 448, NaN 0x7F), never fnuz.
+ *
+ * Scale formula (all granularities, mode 0):
+ *     amax = max|x|;  scale = max(amax, 1e-12) / 448  (fp32, IEEE division)
+ *     byte = e4m3fn_rne(clamp(fp32(x) / scale, -448, 448))
+ * A NaN in a reduction set gives scale 0x7FC00000 and bytes 0x7F.
+ *
+ * "Replaces" cites the call in nvidia-cosmos/cosmos-rl that a binding of the
+ * entry point stands in for.
+ */
+#ifndef COSMOS_FP8_H
+#define COSMOS_FP8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CFP8_OK 0
+#define CFP8_EINVAL (-1)    /* null pointer, bad shape, bad alignment          */
+#define CFP8_EARCH (-2)     /* device is not gfx950                            */
+#define CFP8_ELAUNCH (-3)   /* HIP reported a launch failure                   */
+#define CFP8_EWORKSPACE (-4)/* workspace missing or too small                  */
+
+/* output element types of the GEMM epilogues */
+#define CFP8_OUT_BF16 0
+#define CFP8_OUT_F32 1
+
+/* 1x128 group formulas */
+#define CFP8_GROUP_MODE_DIV 0    /* the scale formula above                                 */
+#define CFP8_GROUP_MODE_DEEPEP 1 /* x*(448/clamp(amax,1e-4)), scale=amax/448, no pre-clamp  */
+
+int cfp8_version(void);
+const char* cfp8_last_error(void);
+
+/* Rowwise dynamic quantisation: per row amax -> scale -> e4m3.
+ * x bf16 [rows, cols] (ld_x), q fp8 [rows, cols] (ld_q), scales fp32 [rows].
+ * Replaces vllm._custom_ops.scaled_fp8_quant(w, scale=None,
+ * use_per_token_if_dynamic=True) at
+ * cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:995-997 and
+ * cosmos_rl/rollout/vllm_rollout/monkey_patch_for_fp8.py:47-49 (weights), and the
+ * per-token activation quantisation inside Fp8LinearOp.apply installed at
+ * monkey_patch_for_fp8.py:74-79.  cols % 8 == 0. */
+int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
+                       void* q, int64_t ld_q, float* scales, void* stream);
+
+/* Tensorwise dynamic quantisation of many tensors in two passes (grid amax,
+ * then cast), without a host round trip in between.
+ * Replaces the torchao tensorwise recipe selected at
+ * cosmos_rl/utils/fp8/fp8_util.py:121-137 (hp_tensor_to_float8_dynamic).
+ * The descriptor array lives in HOST memory; amax_ws is a device array of n
+ * floats (scratch, overwritten).  numel % 8 == 0 for every tensor. */
+typedef struct cfp8_tensor_desc {
+    const void* x;   /* bf16, contiguous, 16-byte aligned */
+    void* q;         /* fp8 out, numel bytes              */
+    float* scale;    /* device, 1 float out               */
+    int64_t numel;
+} cfp8_tensor_desc;
+
+int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
+                                float* amax_ws, void* stream);
+
+/* Single-tensor form of the above. */
+int cfp8_quant_tensorwise(const void* x, int64_t numel, void* q, float* scale,
+                          float* amax_ws, void* stream);
+
+/* 128x128 block quantisation of a batch of matrices.
+ * x bf16 [batch, rows, cols] contiguous; scales fp32
+ * [batch, ceil(rows/128), ceil(cols/128)] row-major (the layout
+ * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:236-243 reads).
+ * transpose_out == 0: q is [batch, rows, cols]; != 0: q is [batch, cols, rows]
+ * (the K-major "nt" operand of the block GEMM when the weight arrives [K, N]).
+ * Replaces dsgemm_utils.prepare_fp8_weight at
+ * cosmos_rl/policy/kernel/group_gemms.py:132.  cols % 8 == 0 (and rows % 16 == 0
+ * when transposing). */
+int cfp8_quant_block128(const void* x, int64_t batch, int64_t rows, int64_t cols,
+                        void* q, float* scales, int transpose_out, void* stream);
+
+/* 1x128 group quantisation of activations.  x bf16 [rows, cols] (ld_x),
+ * q fp8 [rows, cols] (ld_q), scales fp32 [rows, ceil(cols/128)] row-major.
+ * Replaces dsgemm_kernels.groupwise_activation_quant / dsgemm_utils.prepare_fp8_input
+ * at cosmos_rl/policy/kernel/group_gemms.py:188-191, 213-218; mode
+ * CFP8_GROUP_MODE_DEEPEP is per_token_cast_to_fp8 of tests/test_deepep.py:75-85. */
+int cfp8_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
+                        void* q, int64_t ld_q, float* scales, int mode, void* stream);
+
+/* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
+ * CFP8_OUT_F32.  Replaces weight_dequant at
+ * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */
+int cfp8_dequant_block128(const void* q, const float* scales, int64_t rows, int64_t cols,
+                          void* y, int out_dtype, void* stream);
+
+/* Rowwise scaled mm on quantised operands:
+ *   out[m, n] = (sum_k a[m,k] b[n,k]) * sa[m] * sb[n]
+ * a fp8 [M, K] (ld_a), b fp8 [N, K] (ld_b) - the contiguous buffer whose .t()
+ * the reference passes -, sa [M], sb [N], out [M, N] (ld_out).
+ * Replaces torch._scaled_mm(qx, w.t(), scale_a, scale_b, out_dtype=bf16) reached
+ * through cosmos_rl/rollout/vllm_rollout/monkey_patch_for_fp8.py:26-34.
+ * K % 128 == 0, N % 16 == 0. */
+int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* sa,
+                           const void* b, int64_t ld_b, const float* sb,
+                           void* out, int64_t ld_out, int out_dtype,
+                           int64_t M, int64_t N, int64_t K, void* stream);
+
+/* FP8 linear: per-token dynamic quantisation of x (bf16 [M, K]) into the
+ * workspace followed by the rowwise scaled mm, as one call.
+ * Replaces Fp8LinearOp.apply (monkey_patch_for_fp8.py:74-79).
+ * workspace: cfp8_linear_workspace_bytes(M, K) bytes, 256-byte aligned. */
+size_t cfp8_linear_workspace_bytes(int64_t M, int64_t K);
+int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, int64_t ld_w,
+                        const float* w_scale, void* out, int64_t ld_out, int out_dtype,
+                        int64_t M, int64_t N, int64_t K,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Block-scaled "nt" GEMM on quantised operands:
+ *   out[m, n] = sum_kb (a[m, kb] . b[n, kb]) * sa[m, kb] * sb[n/128, kb]
+ * a fp8 [M, K], sa fp32 [M, K/128]; b fp8 [N, K]; sb addressed as
+ * sb[(n/128) * sb_stride_n + kb * sb_stride_k] so both [N/128, K/128] and
+ * [K/128, N/128] layouts work.  K % 128 == 0, N % 16 == 0.
+ * The dense (one expert) case of deep_gemm's fp8 GEMM used at
+ * cosmos_rl/policy/kernel/group_gemms.py:194-225. */
+int cfp8_gemm_block128(const void* a, int64_t ld_a, const float* sa,
+                       const void* b, int64_t ld_b, const float* sb,
+                       int64_t sb_stride_n, int64_t sb_stride_k,
+                       void* out, int64_t ld_out, int out_dtype,
+                       int64_t M, int64_t N, int64_t K, void* stream);
+
+/* Grouped contiguous block-scaled GEMM.  Row r of a belongs to expert
+ * m_indices[r] (int32, device); groups are contiguous and start on multiples of
+ * 128 rows; rows with a negative index are padding and are not written.
+ * b fp8 [E, N, K] contiguous, sb fp32 [E, ceil(N/128), K/128].
+ * Replaces deep_gemm.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous at
+ * cosmos_rl/policy/kernel/group_gemms.py:194-225. */
+int cfp8_gemm_grouped_block128(const void* a, int64_t ld_a, const float* sa,
+                               const void* b, const float* sb, const int32_t* m_indices,
+                               void* out, int64_t ld_out, int out_dtype,
+                               int64_t M, int64_t N, int64_t K, int64_t E, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COSMOS_FP8_H */

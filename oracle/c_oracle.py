@@ -1,0 +1,94 @@
+"""ctypes wrapper of the scalar C restatement (oracle/fp8_ref.c).  TEST INFRASTRUCTURE ONLY.
+
+``build()`` compiles it with gcc; the arrays are numpy (uint16 views of bf16 in, uint8 / float32 out).
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from ctypes import c_float, c_int, c_int64, c_uint8, c_void_p
+from pathlib import Path
+
+import numpy as np
+
+HERE = Path(__file__).resolve().parent
+SRC = HERE / "fp8_ref.c"
+LIB = HERE / "libfp8ref.so"
+
+_lib = None
+
+
+def build() -> Path:
+    cmd = ["gcc", "-O2", "-fPIC", "-shared", "-ffp-contract=off", "-o", str(LIB), str(SRC), "-lm"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"gcc failed on {SRC}:\n{res.stderr}")
+    return LIB
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB.exists():
+            build()
+        lib = ctypes.CDLL(str(LIB))
+        lib.fp8ref_e4m3_from_f32.restype = c_uint8
+        lib.fp8ref_e4m3_from_f32.argtypes = [c_float]
+        lib.fp8ref_e4m3_to_f32.restype = c_float
+        lib.fp8ref_e4m3_to_f32.argtypes = [c_uint8]
+        lib.fp8ref_quant_rowwise.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+        lib.fp8ref_quant_tensorwise.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+        lib.fp8ref_quant_block128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+        lib.fp8ref_quant_group128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int]
+        lib.fp8ref_check_fast_div.restype = c_int64
+        lib.fp8ref_check_fast_div.argtypes = [c_void_p, c_int64, c_void_p]
+        _lib = lib
+    return _lib
+
+
+def _u16(x: np.ndarray) -> np.ndarray:
+    assert x.dtype == np.uint16
+    return np.ascontiguousarray(x)
+
+
+def quant_rowwise(x_u16: np.ndarray):
+    x = _u16(x_u16)
+    R, C = x.shape
+    q = np.empty((R, C), np.uint8)
+    s = np.empty((R, 1), np.float32)
+    load().fp8ref_quant_rowwise(x.ctypes.data, R, C, q.ctypes.data, s.ctypes.data)
+    return q, s
+
+
+def quant_tensorwise(x_u16: np.ndarray):
+    x = _u16(x_u16)
+    q = np.empty(x.shape, np.uint8)
+    s = np.empty(1, np.float32)
+    load().fp8ref_quant_tensorwise(x.ctypes.data, x.size, q.ctypes.data, s.ctypes.data)
+    return q, s
+
+
+def quant_block128(x_u16: np.ndarray):
+    x = _u16(x_u16)
+    R, C = x.shape
+    q = np.empty((R, C), np.uint8)
+    s = np.empty((-(-R // 128), -(-C // 128)), np.float32)
+    load().fp8ref_quant_block128(x.ctypes.data, R, C, q.ctypes.data, s.ctypes.data)
+    return q, s
+
+
+def quant_group128(x_u16: np.ndarray, mode: int = 0):
+    x = _u16(x_u16)
+    M, K = x.shape
+    q = np.empty((M, K), np.uint8)
+    s = np.empty((M, -(-K // 128)), np.float32)
+    load().fp8ref_quant_group128(x.ctypes.data, M, K, q.ctypes.data, s.ctypes.data, mode)
+    return q, s
+
+
+def check_fast_div(scales_f32: np.ndarray):
+    """(bad byte count, fp32 mismatches with |x/s| >= 2^-11) over all 65536 bf16 x per scale."""
+    s = np.ascontiguousarray(scales_f32, dtype=np.float32)
+    soft = ctypes.c_int64(0)
+    bad = load().fp8ref_check_fast_div(s.ctypes.data, s.size, ctypes.byref(soft))
+    return int(bad), int(soft.value)

@@ -1,0 +1,85 @@
+"""The scalar C restatement (oracle/fp8_ref.c) against the torch oracle, and the CPU proof of the
+division shortcut the kernels use."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle as C
+from oracle import fp8_oracle as O
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _built():
+    C.build()
+
+
+def u16(x):
+    return x.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_encoder_exhaustive_bf16_and_random_fp32():
+    lib = C.load()
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    want = O.e4m3_bytes(pats).numpy()
+    got = np.array([lib.fp8ref_e4m3_from_f32(float(v)) for v in pats.numpy()], dtype=np.uint8)
+    assert (got == want).all()
+    g = torch.Generator().manual_seed(0)
+    v = torch.cat([(torch.rand(50000, generator=g) * 2 - 1) * 500, (torch.rand(50000, generator=g) * 2 - 1) * 0.05])
+    want = O.e4m3_bytes(v).numpy()
+    got = np.array([lib.fp8ref_e4m3_from_f32(float(x)) for x in v.numpy()], dtype=np.uint8)
+    assert (got == want).all()
+    back = np.array([lib.fp8ref_e4m3_to_f32(b) for b in range(256)], dtype=np.float32)
+    tb = O.e4m3_to_f32(torch.arange(256, dtype=torch.uint8)).numpy()
+    assert ((back == tb) | (np.isnan(back) & np.isnan(tb))).all()
+
+
+def _weights(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(*shape, generator=g) * torch.exp(torch.randn(shape[0], 1, generator=g) * 3)
+    w = w.to(torch.bfloat16)
+    w[0] = 0
+    if shape[0] > 3:
+        w[1, 0] = float("nan")
+        w[2, 1] = float("inf")
+    return w
+
+
+def test_rowwise_and_tensorwise_agree():
+    w = _weights((64, 200), 1)
+    q, s = C.quant_rowwise(u16(w))
+    qo, so = O.quant_rowwise(w)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+    w = O.make_weight((40, 72), seed=2)
+    q, s = C.quant_tensorwise(u16(w))
+    qo, so = O.quant_tensorwise(w)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+
+
+def test_block_and_group_agree():
+    w = _weights((200, 264), 3)
+    q, s = C.quant_block128(u16(w))
+    qo, so = O.quant_block128(w)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+    x = _weights((33, 328), 4)
+    q, s = C.quant_group128(u16(x), 0)
+    qo, so = O.quant_group128(x)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+    x = O.make_activation(33, 328, seed=5)
+    x[3] = 0
+    q, s = C.quant_group128(u16(x), 1)
+    qo, so = O.group128_cast_deepep(x)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+
+
+def test_division_shortcut_is_exact():
+    """r = 1/s; q0 = x*r; e = fma(-q0, s, x); q1 = copysign(fma(e, r, q0), x) equals the IEEE
+    quotient x/s bit for bit wherever |x/s| >= 2^-11, and gives the same e4m3 byte everywhere,
+    for all 65536 bf16 x and 1500 scales spanning the fp32 range."""
+    g = torch.Generator().manual_seed(0)
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    pos = pats[(pats > 0) & torch.isfinite(pats)]
+    amax = torch.cat([torch.rand(500, generator=g) * 2, torch.exp(torch.rand(500, generator=g) * 170 - 85).clamp(max=3e38),
+                      pos[::66], torch.tensor([0.0, 1e-12, 1e-13, 3.3895e38, 448.0])])
+    scales = O.scale_from_amax(amax).numpy()
+    bad, soft = C.check_fast_div(scales)
+    assert bad == 0 and soft == 0

@@ -1,0 +1,234 @@
+"""Parity of the FP8 MFMA GEMMs with the oracle (dequantised matmul of the same quantised
+operands, accumulated in fp64).  Tolerance: relative Frobenius error <= 1e-3 (TOL) on the
+fp32-epilogue output, and bf16(kernel) against bf16(oracle) to the same bar.  The matrix core
+sums the 128 products of one instruction with less than fp32 precision (observed ~2e-5
+relative), so TIGHT = 1e-4 is asserted as a regression bar well inside TOL.  All calls go
+through the C ABI."""
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from cosmos_rl_amd import ops
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+TIGHT = 1e-4
+
+
+def f8(t_u8, dev):
+    return t_u8.to(dev).view(torch.float8_e4m3fn)
+
+
+def check_bf16(out_bf16, ref_f32, what):
+    """bf16(kernel) against bf16(oracle): relative Frobenius error <= 1e-3, and no entry further
+    than 2 bf16 ulps of the reference magnitude."""
+    ref = ref_f32.to(torch.bfloat16).float()
+    got = out_bf16.float().cpu()
+    err = O.rel_frobenius(got, ref)
+    assert err <= TOL, f"{what}: bf16 rel Frobenius {err:.3e}"
+    tol = ref.abs() * 2 ** -6 + ref_f32.abs().max() * 2 ** -12
+    assert bool(((got - ref).abs() <= tol).all()), f"{what}: bf16 outlier"
+
+
+def rowwise_operands(M, N, K, seed, dev):
+    x = O.make_activation(M, K, seed=seed, chan_outlier_frac=0.005, outlier_mul=30.0)
+    w = O.make_weight((N, K), seed=seed + 1)
+    qx, sx = O.quant_rowwise(x)
+    qw, sw = O.quant_rowwise(w)
+    return x, w, qx, sx, qw, sw
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 64, 256), (17, 80, 384), (64, 128, 512), (100, 272, 896),
+                                   (128, 128, 128), (300, 1024, 1024), (513, 528, 640), (1024, 768, 3584)])
+def test_scaled_mm_rowwise(dev, M, N, K):
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
+    ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
+    a, b = f8(qx, dev), f8(qw, dev)
+    out32 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    err = O.rel_frobenius(out32.cpu(), ref)
+    assert err <= TOL, f"fp32 epilogue rel Frobenius {err:.3e}"
+    assert err <= TIGHT, f"fp32 epilogue rel Frobenius {err:.3e} above the regression bar"
+    out16 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.bfloat16)
+    check_bf16(out16, ref, f"rowwise {M}x{N}x{K}")
+
+
+def test_scaled_mm_one_hot_and_pow2(dev):
+    """One-hot activation rows reproduce single weight entries exactly; power-of-two scales make
+    the epilogue exact, so the fp32 output must equal the oracle bit for bit."""
+    M, N, K = 32, 64, 256
+    g = torch.Generator().manual_seed(3)
+    qw = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+    qw[(qw & 0x7F) == 0x7F] = 0x3F
+    qx = torch.zeros(M, K, dtype=torch.uint8)
+    ks = torch.randint(0, K, (M,), generator=g)
+    qx[torch.arange(M), ks] = 0x38  # 1.0
+    sx = (2.0 ** torch.randint(-6, 6, (M, 1), generator=g)).float()
+    sw = (2.0 ** torch.randint(-6, 6, (N, 1), generator=g)).float()
+    out = ops.scaled_mm(f8(qx, dev), f8(qw, dev).t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32).cpu()
+    want = O.e4m3_to_f32(qw)[:, ks].t() * sx * sw.t()
+    assert torch.equal(out, want)
+    # dense exact case: small integers, power-of-two scales -> every partial sum is exact in fp32
+    qa = torch.randint(0x30, 0x48, (M, K), generator=g, dtype=torch.uint8)
+    ref = O.scaled_mm_rowwise(qa, sx, qw & 0x3F | 0x20, sw, accum=torch.float64)
+    out = ops.scaled_mm(f8(qa, dev), f8(qw & 0x3F | 0x20, dev).t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    assert O.rel_frobenius(out.cpu(), ref) <= TIGHT
+
+
+@pytest.mark.parametrize("M", [1, 64, 1024])
+def test_fp8_linear_cfg3_shapes(dev, M):
+    """BASELINE config 3 at reduced N (the full N runs in the property test below): per-token
+    activation quantisation inside the call, bytes of the intermediate checked through the result."""
+    N, K = 2048, 3584
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=1236 + M, dev=dev)
+    ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
+    out32 = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)
+    err = O.rel_frobenius(out32.cpu(), ref)
+    assert err <= TIGHT, f"M={M}: {err:.3e}"
+    out16 = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev))
+    assert out16.dtype == torch.bfloat16 and tuple(out16.shape) == (M, N)
+    check_bf16(out16, ref, f"linear M={M}")
+    # leading batch dims and bias
+    if M == 64:
+        bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+        o3 = ops.fp8_linear(x.to(dev).view(4, 16, K), f8(qw, dev).t(), sw.to(dev), bias=bias.to(dev))
+        assert tuple(o3.shape) == (4, 16, N)
+        assert torch.equal(o3.view(M, N), out16 + bias.to(dev))
+
+
+def test_fp8_linear_full_cfg3_properties(dev):
+    """Full Qwen2.5-7B MLP shape [8192, 3584] x [18944, 3584]^T on the GPU only.  Linearity in the
+    weight scales (doubling sw doubles the fp32 output exactly), row-subset consistency with an
+    M=64 call (different tile configuration, same numbers), and a sampled block against fp64."""
+    M, N, K = 8192, 18944, 3584
+    g = torch.Generator(device=dev).manual_seed(21)
+    x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    qw, sw = ops.quant_rowwise(w)
+    out = ops.fp8_linear(x, qw.t(), sw, out_dtype=torch.float32)
+    out2 = ops.fp8_linear(x, qw.t(), sw * 2, out_dtype=torch.float32)
+    assert torch.equal(out2, out * 2)
+    sub = ops.fp8_linear(x[4096:4160], qw.t(), sw, out_dtype=torch.float32)
+    assert O.rel_frobenius(sub.cpu(), out[4096:4160].cpu()) <= TIGHT
+    rows = torch.arange(0, M, 257, device=dev)[:24]
+    cols = torch.arange(0, N, 601, device=dev)[:32]
+    qx, sx = ops.quant_rowwise(x[rows])
+    ref = (qx.double() @ qw[cols].double().t()) * sx.double() * sw[cols].double().t()
+    got = out[rows][:, cols].double()
+    assert O.rel_frobenius(got.cpu(), ref.cpu()) <= TIGHT
+
+
+# ---------------------------------------------------------------------------- block-scaled
+def block_operands(M, N, K, seed):
+    x = O.make_activation(M, K, seed=seed)
+    w = O.make_weight((N, K), seed=seed + 1)
+    qx, sx = O.quant_group128(x)
+    qw, sw = O.quant_block128(w)
+    return qx, sx, qw, sw
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 128, 256), (70, 208, 384), (128, 256, 1024), (300, 512, 768),
+                                   (640, 1536, 2048)])
+def test_gemm_block128(dev, M, N, K):
+    qx, sx, qw, sw = block_operands(M, N, K, seed=M * 3 + N + K)
+    ref = O.scaled_mm_block128(qx, sx, qw, sw, accum=torch.float64)
+    out32 = torch.empty(M, N, dtype=torch.float32, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out32)
+    err = O.rel_frobenius(out32.cpu(), ref)
+    assert err <= TIGHT, f"block fp32 {err:.3e}"
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out16)
+    check_bf16(out16, ref, f"block {M}x{N}x{K}")
+
+
+def test_gemm_block128_kn_weight_layout(dev):
+    """Config 4 layout: weight given [K, N], quantised with the transposing quantiser; scales stay
+    [K/128, N/128].  y = x @ W."""
+    M, K, N = 192, 512, 384
+    x = O.make_activation(M, K, seed=40)
+    w = O.make_weight((K, N), seed=41)
+    qx, sx = ops.groupwise_activation_quant(x.to(dev))
+    qwt, sw = ops.per_block_cast_to_fp8(w.to(dev), transpose_out=True)  # [N, K], scales [K/128, N/128]
+    assert tuple(qwt.shape) == (N, K) and tuple(sw.shape) == (K // 128, N // 128)
+    out = torch.empty(M, N, dtype=torch.float32, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((qx, sx), (qwt, sw), out, rhs_scale_kn=True)
+    qxo, sxo = O.quant_group128(x)
+    qwo, swo = O.quant_block128(w)
+    ref = (O.group128_dequant(qxo, sxo).double() @ O.weight_dequant(qwo, swo).double())
+    assert O.rel_frobenius(out.cpu(), ref) <= TIGHT
+
+
+def test_gemm_block128_cfg4_properties(dev):
+    """Config 4 at full size [4096, 7168] x [7168, 18432]: sampled rows/cols against fp64 and
+    exact linearity in a power-of-two rescale of one activation K-block's scales."""
+    M, K, N = 4096, 7168, 18432
+    g = torch.Generator(device=dev).manual_seed(44)
+    x = torch.randn(M, K, generator=g, device=dev).to(torch.bfloat16)
+    w = (torch.randn(K, N, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    qx, sx = ops.groupwise_activation_quant(x)
+    qwt, sw = ops.per_block_cast_to_fp8(w, transpose_out=True)
+    out = torch.empty(M, N, dtype=torch.float32, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((qx, sx), (qwt, sw), out, rhs_scale_kn=True)
+    out2 = torch.empty_like(out)
+    ops.gemm_fp8_fp8_bf16_nt((qx, sx * 4), (qwt, sw * 0.5), out2, rhs_scale_kn=True)
+    assert torch.equal(out2, out * 2)
+    rows = torch.arange(0, M, 173, device=dev)[:20]
+    cols = torch.arange(0, N, 577, device=dev)[:30]
+    a = qx[rows].double() * sx[rows].double().repeat_interleave(128, dim=1)
+    swn = sw.t().contiguous()  # [N/128, K/128]
+    b = qwt[cols].double() * swn[cols // 128].double().repeat_interleave(128, dim=1)
+    ref = a @ b.t()
+    assert O.rel_frobenius(out[rows][:, cols].double().cpu(), ref.cpu()) <= TIGHT
+
+
+# ---------------------------------------------------------------------------- grouped
+def test_grouped_gemm(dev):
+    """Ragged groups: top-2 routing of 300 tokens over 6 experts plus an empty expert, groups
+    padded to 128 rows; padding rows (index -1) must be left untouched."""
+    T, E, K, N, topk = 300, 7, 512, 384, 2
+    g = torch.Generator().manual_seed(77)
+    logits = torch.rand(T, E, generator=g)
+    logits[:, 3] = -1.0  # expert 3 gets no token
+    token_of_row, m_indices, m_sizes, m_offsets = O.route_topk_contiguous(logits, topk, 128)
+    assert int(m_sizes[3]) == 128 and int((m_indices == 3).sum()) == 0
+    x = O.make_activation(T, K, seed=78)
+    xs = torch.zeros(token_of_row.numel(), K, dtype=torch.bfloat16)
+    valid = token_of_row >= 0
+    xs[valid] = x[token_of_row[valid]]
+    w = O.make_weight((E, N, K), seed=79)
+    qx, sx = O.quant_group128(xs)
+    qw, sw = O.quant_block128(w)
+    ref = O.grouped_mm_block128(qx, sx, qw, sw, m_indices, accum=torch.float64)
+    out = torch.full((xs.shape[0], N), 7.0, dtype=torch.float32, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out,
+                                                  m_indices.to(dev))
+    out = out.cpu()
+    assert bool((out[~valid] == 7.0).all()), "padding rows were written"
+    assert O.rel_frobenius(out[valid], ref[valid]) <= TIGHT
+    out16 = torch.zeros((xs.shape[0], N), dtype=torch.bfloat16, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out16,
+                                                  m_indices.to(dev))
+    check_bf16(out16, ref, "grouped")
+    # permuting tokens inside one expert's group permutes the output rows and nothing else
+    rows0 = (m_indices == 0).nonzero().flatten()
+    perm = rows0[torch.randperm(rows0.numel(), generator=g)]
+    qx2, sx2 = qx.clone(), sx.clone()
+    qx2[rows0], sx2[rows0] = qx[perm], sx[perm]
+    out2 = torch.zeros((xs.shape[0], N), dtype=torch.float32, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((f8(qx2, dev), sx2.to(dev)), (f8(qw, dev), sw.to(dev)), out2,
+                                                  m_indices.to(dev))
+    assert torch.equal(out2.cpu()[rows0], out[perm])
+
+
+def test_gemm_errors(dev):
+    a = torch.zeros(16, 100, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    b = torch.zeros(32, 100, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    with pytest.raises(ValueError):  # K % 128
+        ops.scaled_mm(a, b.t(), torch.ones(16, 1, device=dev), torch.ones(1, 32, device=dev))
+    a = torch.zeros(16, 128, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    b = torch.zeros(128, 32, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)  # row-major [K, N]
+    with pytest.raises(ValueError):
+        ops.scaled_mm(a, b, torch.ones(16, 1, device=dev), torch.ones(1, 32, device=dev))
+    out = ops.scaled_mm(torch.zeros(0, 128, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn),
+                        torch.zeros(32, 128, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn).t(),
+                        torch.ones(0, 1, device=dev), torch.ones(1, 32, device=dev))
+    assert tuple(out.shape) == (0, 32)

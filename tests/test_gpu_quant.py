@@ -1,0 +1,282 @@
+"""Parity of the HIP quantizers with the CPU oracle: fp8 bytes and fp32 scales bit-exact.
+Every call goes through the C ABI (cosmos_rl_amd.ops -> ctypes -> libcosmosfp8.so)."""
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from cosmos_rl_amd import ops, _lib
+
+pytestmark = pytest.mark.gpu
+
+
+def u8(t):
+    return t.contiguous().view(torch.uint8).cpu()
+
+
+def bits(t):
+    return t.contiguous().view(torch.int32).cpu()
+
+
+def assert_bytes(got, want, what):
+    got, want = u8(got), want
+    if not torch.equal(got, want):
+        bad = (got != want).nonzero()
+        i = tuple(bad[0].tolist())
+        raise AssertionError(f"{what}: {bad.shape[0]} byte mismatches, first at {i}: got {int(got[i]):#x} want {int(want[i]):#x}")
+
+
+def assert_scales(got, want, what):
+    g, w = bits(got).reshape(-1), want.contiguous().view(torch.int32).reshape(-1)
+    if not torch.equal(g, w):
+        bad = (g != w).nonzero()
+        i = int(bad[0])
+        raise AssertionError(f"{what}: {bad.shape[0]} scale mismatches, first at {i}: got {int(g[i]):#x} want {int(w[i]):#x}")
+
+
+def all_bf16_patterns():
+    return torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------- rowwise
+def test_rowwise_cfg1(dev):
+    """BASELINE config 1: [4864, 896], N(0, 0.02) with 0.1% x20 outliers, seed 1235."""
+    w = O.make_weight((4864, 896), seed=1235, outlier_frac=1e-3, outlier_mul=20.0)
+    q, s = ops.scaled_fp8_quant(w.to(dev), scale=None, use_per_token_if_dynamic=True)
+    assert q.dtype == torch.float8_e4m3fn and tuple(s.shape) == (4864, 1)
+    qo, so = O.quant_rowwise(w)
+    assert_scales(s, so, "cfg1 scales")
+    assert_bytes(q, qo, "cfg1 bytes")
+
+
+@pytest.mark.parametrize("cols", [8, 64, 136, 512, 896, 1024, 2048, 3584, 4096, 4104, 8192, 18944, 32768, 32776, 40000])
+def test_rowwise_widths(dev, cols):
+    """Every kernel variant: wave-per-row (V=1,2,4,8), block-per-row (V=4,8,16), streaming."""
+    rows = 37 if cols < 20000 else 5
+    g = torch.Generator().manual_seed(cols)
+    w = (torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g) * 3)).to(torch.bfloat16)
+    q, s = ops.quant_rowwise(w.to(dev))
+    qo, so = O.quant_rowwise(w)
+    assert_scales(s, so, f"cols={cols} scales")
+    assert_bytes(q, qo, f"cols={cols} bytes")
+
+
+def test_rowwise_exhaustive_patterns(dev):
+    """All 65536 bf16 patterns as data under 256 different row scales.  For one planted amax
+    `a`, the patterns whose magnitude does not exceed `a` (others become 0) are spread over 16
+    rows of 4096 columns; element 0 of each row is overwritten with `a` so that every row has
+    exactly that amax, and a 17th row carries the 16 overwritten patterns."""
+    pats = all_bf16_patterns()
+    pf = pats.float()
+    g = torch.Generator().manual_seed(7)
+    finite_pos = pats[torch.isfinite(pf) & (pf > 0)]
+    amaxes = torch.cat([torch.exp(torch.rand(200, generator=g) * 60 - 40).to(torch.bfloat16),
+                        torch.tensor([448.0, 1.0, 2.0 ** -20, 3.0e38]).to(torch.bfloat16),
+                        finite_pos[torch.randint(0, finite_pos.numel(), (52,), generator=g)]])
+    blocks = []
+    for a in amaxes:
+        keep = torch.isfinite(pf) & (pf.abs() <= a.float())
+        body = torch.where(keep, pats, torch.zeros_like(pats)).view(16, 4096).clone()
+        extra = torch.zeros(1, 4096, dtype=torch.bfloat16)
+        extra[0, 1:17] = body[:, 0]
+        extra[0, 0] = a
+        body[:, 0] = a
+        blocks += [body, extra]
+    w = torch.cat(blocks)
+    q, s = ops.quant_rowwise(w.to(dev))
+    qo, so = O.quant_rowwise(w)
+    assert_scales(s, so, "exhaustive scales")
+    assert_bytes(q, qo, "exhaustive bytes")
+
+
+def test_rowwise_edge_rows(dev):
+    """zero row (scale 0x2720D7C5, bytes 0x00/0x80), NaN row, Inf row, subnormals, ragged stride."""
+    cols = 256
+    w = torch.zeros(6, cols, dtype=torch.bfloat16)
+    w[0, 3] = -0.0
+    w[1, 5] = float("nan"); w[1, 6] = 1.0
+    w[2, 7] = float("inf"); w[2, 8] = -2.0; w[2, 9] = float("-inf")
+    w[3] = torch.linspace(-1e-38, 1e-38, cols).to(torch.bfloat16)
+    w[4] = torch.linspace(-3, 3, cols).to(torch.bfloat16)
+    w[5, 0] = 1e-13
+    q, s = ops.quant_rowwise(w.to(dev))
+    qo, so = O.quant_rowwise(w)
+    assert int(bits(s)[0]) == 0x2720D7C5
+    assert set(u8(q)[0].tolist()) <= {0x00, 0x80} and int(u8(q)[0, 3]) == 0x80
+    assert_scales(s, so, "edge scales")
+    assert_bytes(q, qo, "edge bytes")
+    # non-contiguous rows (a column slice keeps stride(1) == 1)
+    big = O.make_weight((64, 1024), seed=3)
+    view = big.to(dev)[:, 128:640]
+    q2, s2 = ops.quant_rowwise(view)
+    qo2, so2 = O.quant_rowwise(big[:, 128:640].contiguous())
+    assert_scales(s2, so2, "strided scales")
+    assert_bytes(q2, qo2, "strided bytes")
+
+
+def test_rowwise_empty_and_errors(dev):
+    q, s = ops.quant_rowwise(torch.empty(0, 128, dtype=torch.bfloat16, device=dev))
+    assert q.shape == (0, 128) and s.shape == (0, 1)
+    with pytest.raises(ValueError):
+        ops.quant_rowwise(torch.zeros(4, 12, dtype=torch.bfloat16, device=dev))  # cols % 8
+    with pytest.raises(ValueError):
+        ops.quant_rowwise(torch.zeros(4, 16, dtype=torch.float32, device=dev))
+    with pytest.raises(RuntimeError):
+        ops.quant_rowwise(torch.zeros(4, 16, dtype=torch.bfloat16))  # CPU tensor: no fallback
+
+
+def test_rowwise_properties_full_size(dev):
+    """Qwen2.5-7B gate_up [37888, 3584] on the GPU only: every non-zero row holds a +-448 byte,
+    re-quantising the dequantised tensor is idempotent, and row permutation commutes."""
+    g = torch.Generator(device=dev).manual_seed(11)
+    w = (torch.randn(37888, 3584, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    q, s = ops.quant_rowwise(w)
+    qb = q.view(torch.uint8)
+    assert bool((((qb & 0x7F) == 0x7E).any(dim=1)).all())
+    deq = (q.float() * s).to(torch.bfloat16)
+    q2, s2 = ops.quant_rowwise(deq)
+    # dequantised values are bf16-rounded, so compare through one more round trip
+    q3, s3 = ops.quant_rowwise((q2.float() * s2).to(torch.bfloat16))
+    assert torch.equal(q2.view(torch.uint8), q3.view(torch.uint8))
+    perm = torch.randperm(37888, generator=g, device=dev)
+    qp, sp = ops.quant_rowwise(w[perm])
+    assert torch.equal(qp.view(torch.uint8), qb[perm]) and torch.equal(sp, s[perm])
+
+
+# ---------------------------------------------------------------------------- tensorwise
+def test_tensorwise_multi(dev):
+    """A Qwen2.5-7B-shaped layer set at reduced width plus ragged extras, in one call."""
+    shapes = [(3584, 512), (512, 512), (512, 512), (3584, 512), (1184, 512), (1184, 512), (512, 1184),
+              (8, 8), (1, 8), (300, 72), (2048 * 8 + 8,), (0, 16)]
+    ws = [O.make_weight(sh, seed=100 + i, std=0.02 * (i + 1)) for i, sh in enumerate(shapes)]
+    qs, scales = ops.quant_tensorwise_multi([w.to(dev) for w in ws])
+    for i, w in enumerate(ws):
+        qo, so = O.quant_tensorwise(w)
+        assert_scales(scales[i:i + 1], so, f"tensor {i} scale")
+        assert_bytes(qs[i], qo, f"tensor {i} bytes")
+        assert qs[i].shape == w.shape
+
+
+def test_tensorwise_many_tensors_and_batches(dev, monkeypatch):
+    """More tensors than one descriptor table holds (48), so several batches are launched."""
+    ws = [O.make_weight((16 + 8 * (i % 5), 64), seed=500 + i, std=0.01 * (1 + i % 7)) for i in range(131)]
+    qs, scales = ops.quant_tensorwise_multi([w.to(dev) for w in ws])
+    for i, w in enumerate(ws):
+        qo, so = O.quant_tensorwise(w)
+        assert_scales(scales[i:i + 1], so, f"tensor {i} scale")
+        assert_bytes(qs[i], qo, f"tensor {i} bytes")
+
+
+def test_tensorwise_edges(dev):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16)
+    q, s = ops.quant_tensorwise(w.to(dev))
+    assert int(bits(s)[0]) == 0x2720D7C5 and int(u8(q).max()) == 0
+    w[5, 5] = float("nan")
+    q, s = ops.quant_tensorwise(w.to(dev))
+    qo, so = O.quant_tensorwise(w)
+    assert_scales(s, so, "nan scale"); assert_bytes(q, qo, "nan bytes")
+    w[5, 5] = float("inf"); w[6, 6] = 3.0
+    q, s = ops.quant_tensorwise(w.to(dev))
+    qo, so = O.quant_tensorwise(w)
+    assert_scales(s, so, "inf scale"); assert_bytes(q, qo, "inf bytes")
+    # scaled_fp8_quant without per-token = tensorwise
+    w = O.make_weight((96, 160), seed=9)
+    q, s = ops.scaled_fp8_quant(w.to(dev))
+    qo, so = O.quant_tensorwise(w)
+    assert tuple(s.shape) == (1,)
+    assert_scales(s, so, "per-tensor scale"); assert_bytes(q, qo, "per-tensor bytes")
+
+
+def test_tensorwise_full_size_properties(dev):
+    """lm_head-sized tensor [152064, 3584] on the GPU only: scale equals the closed form of the
+    torch amax, the set holds +-448, and the bytes equal a rowwise-kernel-free recomputation on a
+    slice checked against the oracle."""
+    g = torch.Generator(device=dev).manual_seed(5)
+    w = (torch.randn(152064, 3584, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    q, s = ops.quant_tensorwise(w)
+    amax = w.abs().amax().float()
+    want = torch.clamp(amax, min=1e-12) / 448.0
+    assert torch.equal(s.view(torch.int32), want.reshape(1).view(torch.int32))
+    assert bool(((q.view(torch.uint8) & 0x7F) == 0x7E).any())
+    rows = torch.tensor([0, 1, 77777, 152063])
+    sl = w[rows.to(dev)].cpu()
+    want_bytes = O._cast_with_scale(sl, s.cpu())
+    assert_bytes(q[rows.to(dev)], want_bytes, "lm_head slice")
+
+
+# ---------------------------------------------------------------------------- block 128x128
+@pytest.mark.parametrize("shape", [(128, 128), (256, 384), (200, 136), (1, 8), (130, 1032), (3, 256, 384), (2, 200, 136)])
+def test_block128(dev, shape):
+    w = O.make_weight(shape, seed=sum(shape), std=0.02)
+    # per-block dynamic range
+    w = (w.float() * torch.exp(torch.randn(*shape, generator=torch.Generator().manual_seed(1)) * 0.5)).to(torch.bfloat16)
+    q, s = ops.per_block_cast_to_fp8(w.to(dev))
+    qo, so = O.quant_block128(w)
+    assert s.shape == so.shape
+    assert_scales(s, so, f"block {shape} scales")
+    assert_bytes(q, qo, f"block {shape} bytes")
+
+
+@pytest.mark.parametrize("shape", [(128, 128), (256, 384), (208, 136), (2, 144, 264)])
+def test_block128_transposed(dev, shape):
+    w = O.make_weight(shape, seed=sum(shape) + 1, std=0.05)
+    q, s = ops.per_block_cast_to_fp8(w.to(dev), transpose_out=True)
+    qo, so = O.quant_block128(w)
+    assert_scales(s, so, f"blockT {shape} scales")
+    assert_bytes(q, qo.transpose(-1, -2).contiguous(), f"blockT {shape} bytes")
+
+
+def test_block128_cfg4_and_dequant_roundtrip(dev):
+    """BASELINE config 4 weight [7168, 18432] -> scales [56, 144]; a 512x512 corner against the
+    oracle, the whole tensor through weight_dequant (the in-tree inverse pins the layout)."""
+    w = O.make_weight((7168, 18432), seed=1238)
+    wd = w.to(dev)
+    q, s = ops.prepare_fp8_weight(wd)
+    assert tuple(s.shape) == (56, 144)
+    qo, so = O.quant_block128(w[:512, 17920:])
+    assert_scales(s[:4, 140:], so, "cfg4 corner scales")
+    assert_bytes(q[:512, 17920:], qo, "cfg4 corner bytes")
+    y = ops.weight_dequant(q, s, out_dtype=torch.float32)
+    blocks_amax = wd.float().abs().view(56, 128, 144, 128).amax(dim=(1, 3))
+    err = (y - wd.float()).abs().view(56, 128, 144, 128).amax(dim=(1, 3))
+    # half an e4m3 ulp at the top binade is 16/448 of amax; values are far below that bound mostly
+    assert bool((err <= blocks_amax * (16.0 / 448.0) * 1.001 + 1e-30).all())
+    yo = O.weight_dequant(u8(q[:256, :256]), s[:2, :2].cpu())
+    assert torch.equal(y[:256, :256].cpu(), yo)
+    yb = ops.weight_dequant(q[:256, :256].contiguous(), s[:2, :2].contiguous(), out_dtype=torch.bfloat16)
+    assert torch.equal(yb.cpu(), yo.to(torch.bfloat16))
+
+
+# ---------------------------------------------------------------------------- 1x128 groups
+@pytest.mark.parametrize("shape", [(4, 128), (33, 896), (7, 200), (1, 8), (129, 2048), (64, 7168)])
+def test_group128(dev, shape):
+    x = O.make_activation(*shape, seed=shape[0] * 31 + shape[1], chan_outlier_frac=0.01, outlier_mul=30.0)
+    q, s = ops.groupwise_activation_quant(x.to(dev))
+    qo, so = O.quant_group128(x)
+    assert_scales(s, so, f"group {shape} scales")
+    assert_bytes(q, qo, f"group {shape} bytes")
+
+
+@pytest.mark.parametrize("shape", [(4, 128), (33, 896), (7, 200), (129, 2048)])
+def test_group128_deepep_formula(dev, shape):
+    """per_token_cast_to_fp8 exactly as the reference's tests/test_deepep.py states it."""
+    x = O.make_activation(*shape, seed=shape[0] * 17 + shape[1])
+    x[0, :8] = 0
+    if shape[1] >= 256:
+        x[1, 128:256] = 1e-6  # below the 1e-4 amax floor
+    q, s = ops.per_token_cast_to_fp8(x.to(dev))
+    qo, so = O.group128_cast_deepep(x)
+    assert_scales(s, so, f"deepep {shape} scales")
+    assert_bytes(q, qo, f"deepep {shape} bytes")
+
+
+def test_group128_edges(dev):
+    x = torch.zeros(5, 384, dtype=torch.bfloat16)
+    x[1, 130] = float("nan")
+    x[2, 10] = float("inf"); x[2, 11] = 1.0
+    x[3, 300] = -0.0
+    q, s = ops.prepare_fp8_input(x.to(dev))
+    qo, so = O.quant_group128(x)
+    assert_scales(s, so, "group edge scales")
+    assert_bytes(q, qo, "group edge bytes")
+    q, s = ops.prepare_fp8_input(torch.empty(0, 256, dtype=torch.bfloat16, device=dev))
+    assert q.shape == (0, 256) and s.shape == (0, 2)
