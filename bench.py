@@ -1,0 +1,345 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 hot path on one MI355X.
+
+Headline workload (BASELINE config 2): tensorwise FP8 quantisation of every linear weight of a
+Qwen2.5-7B-shaped decoder (197 bf16 tensors, 7 070 285 824 elements, random init N(0, 0.02),
+already resident in HBM).  One step = one `cfp8_quant_tensorwise_multi` call over all tensors
+(grid amax -> scale -> e4m3 cast), i.e. one full weight-sync quantisation pass.
+
+`value` = algorithmic bytes of the two-pass algorithm (5 B/element: 2 read by the amax pass,
+2 read + 1 written by the cast pass) per second over the timed steps.
+`roofline` is for the dominant kernel (the cast pass, 3 B/element), timed per launch with
+events on the launch stream.  `extra` carries the other kernels of the path (rowwise / block /
+group quantisers in GB/s, the FP8 GEMMs in TFLOP/s).  `cpu_baseline` times the torch CPU oracle
+on one tensor of each distinct shape and scales by multiplicity.
+
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (str(ROOT), str(ROOT / "cosmos-rl_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
+
+QWEN25_7B = [("q_proj", (3584, 3584), 28), ("o_proj", (3584, 3584), 28), ("k_proj", (512, 3584), 28),
+             ("v_proj", (512, 3584), 28), ("gate_proj", (18944, 3584), 28), ("up_proj", (18944, 3584), 28),
+             ("down_proj", (3584, 18944), 28), ("lm_head", (152064, 3584), 1)]
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary kernels")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no cross-GPU step on a single "
+              "MI355X; see DESIGN.md for how it shards). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    from cosmos_rl_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev).manual_seed(1236)
+
+    # ------------------------------------------------------------------ headline: config 2
+    tensors = []
+    for name, (r, c), mult in QWEN25_7B:
+        for _ in range(mult):
+            t = torch.empty(r, c, dtype=torch.bfloat16, device=dev)
+            t.normal_(0.0, 0.02, generator=gen)
+            tensors.append(t)
+    n = len(tensors)
+    numel = sum(t.numel() for t in tensors)
+    assert n == 197 and numel == 7_070_285_824
+    outs = [torch.empty(t.shape, dtype=torch.float8_e4m3fn, device=dev) for t in tensors]
+    scales = torch.empty(n, dtype=torch.float32, device=dev)
+    amax_ws = torch.empty(n * _lib.TENSORWISE_AMAX_SLOTS, dtype=torch.float32, device=dev)
+    descs = (_lib.TensorDesc * n)()
+    for i, (t, q) in enumerate(zip(tensors, outs)):
+        descs[i].x, descs[i].q, descs[i].scale, descs[i].numel = t.data_ptr(), q.data_ptr(), scales.data_ptr() + 4 * i, t.numel()
+
+    def step():
+        _lib.check(lib.cfp8_quant_tensorwise_multi(descs, n, amax_ws.data_ptr(), stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    algo_bytes_step = 5 * numel + 4 * n
+    value = algo_bytes_step / (ms_per_step * 1e-3) / 1e9
+
+    # sanity on the result of the timed region: scales equal the closed form of torch's amax
+    idx = [0, 56, 112, 196]
+    for i in idx:
+        # formed on the CPU: torch's GPU division by a python scalar multiplies by a reciprocal
+        want = torch.clamp(tensors[i].abs().amax().float().cpu(), min=1e-12) / 448.0
+        assert torch.equal(scales[i].cpu().view(torch.int32), want.view(torch.int32)), f"scale {i} mismatch"
+        assert bool(((outs[i].view(torch.uint8) & 0x7F) == 0x7E).any())
+
+    # ---- per-kernel timing of the two passes with events on the launch stream -------------
+    def time_phase(fn, reps):
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return [a.elapsed_time(b) for a, b in evs]
+
+    reps = max(3, args.steps)
+    amax_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_amax_multi(descs, n, amax_ws.data_ptr(), stream)), reps)
+    cast_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_cast_multi(descs, n, amax_ws.data_ptr(), stream)), reps)
+    # launches per pass: batches of <= 48 tensors (and <= CFP8_TW_BATCH_MB of bf16 if that knob is set)
+    budget = (int(os.environ.get("CFP8_TW_BATCH_MB", "0")) or (1 << 40)) << 20
+    launches, cnt, by = 0, 0, 0
+    for t in tensors:
+        b = t.numel() * 2
+        if cnt and (cnt == 48 or by + b > budget):
+            launches, cnt, by = launches + 1, 0, 0
+        cnt, by = cnt + 1, by + b
+    launches += 1
+    cast_med = statistics.median(cast_ms)
+    amax_med = statistics.median(amax_ms)
+    cast_bytes = 3 * numel + 4 * n
+    roofline = {
+        "kernel": "tensorwise_cast_kernel",
+        "bound": "hbm",
+        "achieved": round(cast_bytes / (cast_med * 1e-3) / 1e9, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(cast_bytes / (cast_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "bytes_per_launch": cast_bytes // launches,
+        "launches_per_step": launches,
+        "avg_launch_ms": round(cast_med / launches, 4),
+        "amax_kernel": {"achieved": round(2 * numel / (amax_med * 1e-3) / 1e9, 1), "unit": "GB/s",
+                        "frac": round(2 * numel / (amax_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        "avg_launch_ms": round(amax_med / launches, 4)},
+    }
+
+    del outs
+    extra = {}
+    if not args.no_extra:
+        extra = run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors)
+    del tensors
+    torch.cuda.empty_cache()
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(torch)
+
+    line = {
+        "metric": "weight-quant HBM GB/s + fp8 scaled-GEMM TFLOP/s, Qwen2.5-7B shapes, 1 GPU",
+        "value": round(value, 1),
+        "unit": "GB/s (tensorwise weight quantisation, 5 B/element two-pass accounting)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16->e4m3 (fp32 arithmetic)", "data": "synthetic",
+        "config": {"workload": "configs[1]: tensorwise FP8 quantisation of all 197 Qwen2.5-7B linear weights "
+                               "(7 070 285 824 bf16 elements, N(0,0.02)), one full weight-sync pass per step",
+                   "elements": numel, "tensors": n,
+                   "single_read_lower_bound_GBps": round((3 * numel) / (ms_per_step * 1e-3) / 1e9, 1)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def _time_events(torch, fn, warmup, iters, flush=None):
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(iters):
+        if flush is not None:
+            flush.add_(1)          # 512 MiB write: evicts L2 / memory-side cache between iterations
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        times.append((a, b))
+    torch.cuda.synchronize()
+    ms = [a.elapsed_time(b) for a, b in times]
+    return statistics.median(ms), min(ms)
+
+
+def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors):
+    """Secondary kernels of the path; each entry carries its own roofline fraction."""
+    check = _lib.check
+    flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=dev)
+    out = {}
+
+    def hbm(name, bytes_, fn, iters=20):
+        med, mn = _time_events(torch, fn, 3, iters, flush)
+        out[name] = {"ms": round(med, 4), "GB/s": round(bytes_ / (med * 1e-3) / 1e9, 1),
+                     "frac_hbm": round(bytes_ / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    def mfma(name, flops, bytes_, fn, iters=20):
+        med, mn = _time_events(torch, fn, 3, iters, flush)
+        tf = flops / (med * 1e-3) / 1e12
+        gbs = bytes_ / (med * 1e-3) / 1e9
+        bound = "mfma" if flops / bytes_ > FP8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9) else "hbm"
+        out[name] = {"ms": round(med, 4), "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
+                     "frac": round(tf / FP8_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS, 4)}
+
+    # rowwise weight quantisation at the shapes of one weight sync (vLLM packed layers)
+    for nm, (r, c) in [("rowwise_cfg1_4864x896", (4864, 896)), ("rowwise_qkv_4608x3584", (4608, 3584)),
+                       ("rowwise_gate_up_37888x3584", (37888, 3584)), ("rowwise_down_3584x18944", (3584, 18944)),
+                       ("rowwise_lm_head_152064x3584", (152064, 3584))]:
+        x = tensors[-1][:r] if (r, c) == (152064, 3584) else torch.empty(r, c, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+        q = torch.empty(r, c, dtype=torch.float8_e4m3fn, device=dev)
+        s = torch.empty(r, 1, dtype=torch.float32, device=dev)
+        hbm(nm, 3 * r * c + 4 * r,
+            lambda: check(lib.cfp8_quant_rowwise(x.data_ptr(), r, c, c, q.data_ptr(), c, s.data_ptr(), stream)))
+        del x, q, s
+
+    # config 4: block quantisation of W [7168, 18432] (transposed fp8 out) + block-scaled GEMM
+    K4, N4, M4 = 7168, 18432, 4096
+    w4 = torch.empty(K4, N4, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+    q4 = torch.empty(N4, K4, dtype=torch.float8_e4m3fn, device=dev)
+    s4 = torch.empty(K4 // 128, N4 // 128, dtype=torch.float32, device=dev)
+    hbm("block128_cfg4_7168x18432_T", 3 * K4 * N4 + 4 * s4.numel(),
+        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4.data_ptr(), s4.data_ptr(), 1, stream)))
+    q4n = torch.empty(K4, N4, dtype=torch.float8_e4m3fn, device=dev)
+    hbm("block128_cfg4_7168x18432", 3 * K4 * N4 + 4 * s4.numel(),
+        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4n.data_ptr(), s4.data_ptr(), 0, stream)))
+    del q4n, w4
+    x4 = torch.randn(M4, K4, generator=gen, device=dev).to(torch.bfloat16)
+    qx4 = torch.empty(M4, K4, dtype=torch.float8_e4m3fn, device=dev)
+    sx4 = torch.empty(M4, K4 // 128, dtype=torch.float32, device=dev)
+    hbm("group128_cfg4_4096x7168", 3 * M4 * K4 + 4 * sx4.numel(),
+        lambda: check(lib.cfp8_quant_group128(x4.data_ptr(), M4, K4, K4, qx4.data_ptr(), K4, sx4.data_ptr(), 0, stream)))
+    o4 = torch.empty(M4, N4, dtype=torch.bfloat16, device=dev)
+
+    def gemm4():
+        check(lib.cfp8_quant_group128(x4.data_ptr(), M4, K4, K4, qx4.data_ptr(), K4, sx4.data_ptr(), 0, stream))
+        check(lib.cfp8_gemm_block128(qx4.data_ptr(), K4, sx4.data_ptr(), q4.data_ptr(), K4, s4.data_ptr(), 1, N4 // 128,
+                                     o4.data_ptr(), N4, 0, M4, N4, K4, stream))
+    mfma("gemm_block128_cfg4_4096x18432x7168_incl_act_quant", 2.0 * M4 * N4 * K4, N4 * K4 + M4 * K4 * 2 + M4 * N4 * 2, gemm4, iters=10)
+    del x4, qx4, sx4, o4, q4, s4
+
+    # config 3: FP8 linear [M, 3584] x [18944, 3584]^T, per-token activation quant inside the call
+    N3, K3 = 18944, 3584
+    w3 = torch.empty(N3, K3, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+    qw3, sw3 = ops.quant_rowwise(w3)
+    del w3
+    for M in (1, 64, 1024, 8192):
+        x = torch.randn(M, K3, generator=gen, device=dev)
+        chan = torch.rand(K3, generator=gen, device=dev) < 0.005
+        x = torch.where(chan[None, :], x * 30, x).to(torch.bfloat16)
+        o = torch.empty(M, N3, dtype=torch.bfloat16, device=dev)
+        wsb = lib.cfp8_linear_workspace_bytes(M, K3)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+        mfma(f"linear_rowwise_cfg3_M{M}", 2.0 * M * N3 * K3, N3 * K3 + 4 * N3 + M * K3 * 2 + M * N3 * 2,
+             lambda: check(lib.cfp8_linear_rowwise(x.data_ptr(), K3, qw3.data_ptr(), K3, sw3.data_ptr(), o.data_ptr(), N3, 0,
+                                                   M, N3, K3, ws.data_ptr(), wsb, stream)), iters=20 if M < 8192 else 10)
+        del x, o, ws
+    del qw3, sw3
+
+    # config 5: Qwen3-30B-A3B experts, 8192 tokens routed top-8 over 128 experts
+    E, H, I, T, TOPK = 128, 2048, 768, 8192, 8
+    wgu = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+    wd = torch.empty(E, H, I, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+    qgu = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    sgu = torch.empty(E, 2 * I // 128, H // 128, dtype=torch.float32, device=dev)
+    qd = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    sd = torch.empty(E, H // 128, I // 128, dtype=torch.float32, device=dev)
+
+    def quant5():
+        check(lib.cfp8_quant_block128(wgu.data_ptr(), E, 2 * I, H, qgu.data_ptr(), sgu.data_ptr(), 0, stream))
+        check(lib.cfp8_quant_block128(wd.data_ptr(), E, H, I, qd.data_ptr(), sd.data_ptr(), 0, stream))
+    hbm("block128_cfg5_experts", 3 * (wgu.numel() + wd.numel()) + 4 * (sgu.numel() + sd.numel()), quant5, iters=10)
+    del wgu, wd
+    logits = torch.rand(T, E, generator=gen, device=dev)
+    topi = torch.topk(logits, TOPK, dim=1).indices.reshape(-1)
+    counts = torch.bincount(topi, minlength=E)
+    padded = torch.clamp_min(((counts + 127) // 128) * 128, 128)
+    offs = torch.cumsum(padded, 0)
+    total = int(offs[-1])
+    rows = torch.arange(total, device=dev)
+    e_of_row = torch.searchsorted(offs, rows, right=True)
+    start = offs - padded
+    m_idx = torch.where(rows - start[e_of_row] < counts[e_of_row], e_of_row, torch.full_like(e_of_row, -1)).to(torch.int32)
+    routed = int(counts.sum())
+    xs = torch.randn(total, H, generator=gen, device=dev).to(torch.bfloat16)
+    qxs = torch.empty(total, H, dtype=torch.float8_e4m3fn, device=dev)
+    sxs = torch.empty(total, H // 128, dtype=torch.float32, device=dev)
+    gu = torch.empty(total, 2 * I, dtype=torch.bfloat16, device=dev)
+    hdn = torch.randn(total, I, generator=gen, device=dev).to(torch.bfloat16)
+    qh = torch.empty(total, I, dtype=torch.float8_e4m3fn, device=dev)
+    sh = torch.empty(total, I // 128, dtype=torch.float32, device=dev)
+    dn = torch.empty(total, H, dtype=torch.bfloat16, device=dev)
+
+    def moe():
+        check(lib.cfp8_quant_group128(xs.data_ptr(), total, H, H, qxs.data_ptr(), H, sxs.data_ptr(), 0, stream))
+        check(lib.cfp8_gemm_grouped_block128(qxs.data_ptr(), H, sxs.data_ptr(), qgu.data_ptr(), sgu.data_ptr(), m_idx.data_ptr(),
+                                             gu.data_ptr(), 2 * I, 0, total, 2 * I, H, E, stream))
+        check(lib.cfp8_quant_group128(hdn.data_ptr(), total, I, I, qh.data_ptr(), I, sh.data_ptr(), 0, stream))
+        check(lib.cfp8_gemm_grouped_block128(qh.data_ptr(), I, sh.data_ptr(), qd.data_ptr(), sd.data_ptr(), m_idx.data_ptr(),
+                                             dn.data_ptr(), H, 0, total, H, I, E, stream))
+    flops5 = 2.0 * routed * (H * 2 * I + I * H)
+    mfma("grouped_cfg5_gate_up_down_incl_act_quant", flops5,
+         qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=10)
+    out["grouped_cfg5_gate_up_down_incl_act_quant"]["routed_rows"] = routed
+    out["grouped_cfg5_gate_up_down_incl_act_quant"]["padded_rows"] = total
+    return out
+
+
+def cpu_baseline(torch):
+    """The torch CPU oracle (a port of the reference's torch-op path) on one tensor of each
+    distinct Qwen2.5-7B shape, median of 3, scaled by multiplicity to a full pass."""
+    from oracle import fp8_oracle as O
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    shapes = {}
+    for _, shp, mult in QWEN25_7B:
+        shapes[shp] = shapes.get(shp, 0) + mult
+    total_s, numel = 0.0, 0
+    g = torch.Generator().manual_seed(1)
+    for shp, mult in shapes.items():
+        w = (torch.randn(*shp, generator=g) * 0.02).to(torch.bfloat16)
+        ts = []
+        for _ in range(3 if w.numel() < 2e8 else 2):
+            t0 = time.perf_counter()
+            O.quant_tensorwise(w)
+            ts.append(time.perf_counter() - t0)
+        total_s += statistics.median(ts) * mult
+        numel += w.numel() * mult
+        del w
+    return {"value": round(5 * numel / total_s / 1e9, 2),
+            "unit": "GB/s (same 5 B/element accounting)", "cores": cores, "kind": "port",
+            "sample": "torch CPU oracle quant_tensorwise on one tensor of each of the 5 distinct shapes "
+                      "(median of 2-3 runs), scaled by multiplicity to the 197-tensor pass",
+            "estimated_full_pass_s": round(total_s, 2)}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -15,6 +15,7 @@ OUT_BF16 = 0
 OUT_F32 = 1
 GROUP_MODE_DIV = 0
 GROUP_MODE_DEEPEP = 1
+TENSORWISE_AMAX_SLOTS = 64
 
 EINVAL, EARCH, ELAUNCH, EWORKSPACE = -1, -2, -3, -4
 
@@ -29,6 +30,8 @@ SIGNATURES = {
     "cfp8_last_error": (c_char_p, []),
     "cfp8_quant_rowwise": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
+    "cfp8_tensorwise_amax_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
+    "cfp8_tensorwise_cast_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "cfp8_quant_block128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p]),
     "cfp8_quant_group128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p]),

@@ -92,7 +92,7 @@ def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.
     _need_gpu(*tensors)
     dev = tensors[0].device
     scales = torch.empty(n, dtype=torch.float32, device=dev)
-    amax_ws = torch.empty(n, dtype=torch.float32, device=dev)
+    amax_ws = torch.empty(n * _lib.TENSORWISE_AMAX_SLOTS, dtype=torch.float32, device=dev)
     outs: List[torch.Tensor] = []
     keep = []
     descs = (_lib.TensorDesc * n)()

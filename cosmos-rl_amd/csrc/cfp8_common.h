@@ -98,6 +98,42 @@ struct Divider {
     }
 };
 
+// Streaming (non-temporal) accesses: the quantisers read every input byte once and
+// their output is consumed much later, so neither side should displace other data
+// from L2 or the memory-side cache (and a no-allocate load never has to evict a
+// dirty line first).
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+template <bool NT>
+__device__ __forceinline__ uint4 ld16(const uint4* p) {
+    if (NT) {
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        return make_uint4(v[0], v[1], v[2], v[3]);
+    }
+    return *p;
+}
+template <bool NT>
+__device__ __forceinline__ void st8(uint2* p, uint2 o) {
+    if (NT) {
+        u32x2 v;
+        v[0] = o.x;
+        v[1] = o.y;
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+    } else {
+        *p = o;
+    }
+}
+template <bool NT>
+__device__ __forceinline__ void st16(uint4* p, uint4 o) {
+    if (NT) {
+        u32x4 v;
+        v[0] = o.x; v[1] = o.y; v[2] = o.z; v[3] = o.w;
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+    } else {
+        *p = o;
+    }
+}
+
 // two fp32 -> two OCP e4m3fn bytes (RNE) in the low or high half of `old`
 template <bool HI>
 __device__ __forceinline__ u32 cvt2(float a, float b, u32 old) {

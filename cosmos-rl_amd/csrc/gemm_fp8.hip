@@ -273,7 +273,7 @@ static int check_common(const char* who, const void* a, const void* b, const flo
 }
 
 int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
-                         float* scales, hipStream_t st);
+                         float* scales, bool streaming_out, hipStream_t st);
 
 }  // namespace cfp8
 
@@ -317,7 +317,7 @@ extern "C" int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, i
     if (int rc = check_common("linear_rowwise", qx, w, sx, w_scale, out, K, ld_w, ld_out, out_dtype, M, N, K)) return rc;
     if (int rc = check_device()) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (int rc = launch_quant_rowwise(x, M, K, ld_x, qx, K, sx, st)) return rc;
+    if (int rc = launch_quant_rowwise(x, M, K, ld_x, qx, K, sx, false, st)) return rc;
     GemmArgs p{};
     p.a = qx;
     p.b = static_cast<const uint8_t*>(w);

@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int64_t r = r0 + rg * 8 + i;
-        v[i] = (col_ok && r < rows) ? *reinterpret_cast<const uint4*>(xb + r * cols + col) : make_uint4(0, 0, 0, 0);
+        v[i] = (col_ok && r < rows) ? ld16<true>(reinterpret_cast<const uint4*>(xb + r * cols + col)) : make_uint4(0, 0, 0, 0);
     }
     u32 m = 0;
 #pragma unroll
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int64_t r = r0 + rg * 8 + i;
-            if (col_ok && r < rows) *reinterpret_cast<uint2*>(qb + r * cols + col) = cast8(v[i], d);
+            if (col_ok && r < rows) st8<true>(reinterpret_cast<uint2*>(qb + r * cols + col), cast8(v[i], d));
         }
     } else {
         // bytes[i] = row i, 8 columns; regroup to 8 rows of one column (8 bytes) per LDS store
@@ -77,8 +77,8 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
             const int c = (t >> 3) + 32 * p;
             const int64_t oc = c0 + c, orow = r0 + chunk * 16;
             if (oc < cols && orow < rows)  // rows % 16 == 0: a chunk is inside or outside as a whole
-                *reinterpret_cast<uint4*>(qb + oc * rows + orow) =
-                    *reinterpret_cast<const uint4*>(&tile[c * kTStride + chunk * 16]);
+                st16<true>(reinterpret_cast<uint4*>(qb + oc * rows + orow),
+                           *reinterpret_cast<const uint4*>(&tile[c * kTStride + chunk * 16]));
         }
     }
 }
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__
         gcol[i] = (int)(g - row[i] * ngroups);
         const int vec = gcol[i] * 16 + sub;
         ok[i] = g < total_groups && vec < nvec;
-        v[i] = ok[i] ? x[row[i] * ldx + vec] : make_uint4(0, 0, 0, 0);
+        v[i] = ok[i] ? ld16<true>(x + row[i] * ldx + vec) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

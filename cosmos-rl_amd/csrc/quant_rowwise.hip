@@ -12,7 +12,7 @@
 
 namespace cfp8 {
 
-template <int V>
+template <int V, bool NTS>
 __global__ __launch_bounds__(256) void rowwise_wave_kernel(const uint4* __restrict__ x, int64_t rows,
                                                            int nvec, int64_t ldx, uint2* __restrict__ q,
                                                            int64_t ldq, float* __restrict__ scales) {
@@ -24,7 +24,7 @@ __global__ __launch_bounds__(256) void rowwise_wave_kernel(const uint4* __restri
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         int idx = lane + 64 * i;
-        v[i] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+        v[i] = idx < nvec ? ld16<true>(xr + idx) : make_uint4(0, 0, 0, 0);
     }
     u32 m = 0;
 #pragma unroll
@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void rowwise_wave_kernel(const uint4* __restri
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         int idx = lane + 64 * i;
-        if (idx < nvec) qr[idx] = cast8(v[i], d);
+        if (idx < nvec) st8<NTS>(qr + idx, cast8(v[i], d));
     }
 }
 
@@ -48,7 +48,7 @@ __device__ __forceinline__ u32 block_max_256(u32 wave_val, u32* lds) {
     return umax(umax(lds[0], lds[1]), umax(lds[2], lds[3]));
 }
 
-template <int V>
+template <int V, bool NTS>
 __global__ __launch_bounds__(256) void rowwise_block_kernel(const uint4* __restrict__ x, int nvec,
                                                             int64_t ldx, uint2* __restrict__ q,
                                                             int64_t ldq, float* __restrict__ scales) {
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void rowwise_block_kernel(const uint4* __restr
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         int idx = t + 256 * i;
-        v[i] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+        v[i] = idx < nvec ? ld16<true>(xr + idx) : make_uint4(0, 0, 0, 0);
     }
     u32 m = 0;
 #pragma unroll
@@ -73,10 +73,11 @@ __global__ __launch_bounds__(256) void rowwise_block_kernel(const uint4* __restr
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         int idx = t + 256 * i;
-        if (idx < nvec) qr[idx] = cast8(v[i], d);
+        if (idx < nvec) st8<NTS>(qr + idx, cast8(v[i], d));
     }
 }
 
+template <bool NTS>
 __global__ __launch_bounds__(256) void rowwise_stream_kernel(const uint4* __restrict__ x, int64_t nvec,
                                                              int64_t ldx, uint2* __restrict__ q,
                                                              int64_t ldq, float* __restrict__ scales) {
@@ -85,26 +86,26 @@ __global__ __launch_bounds__(256) void rowwise_stream_kernel(const uint4* __rest
     const int t = threadIdx.x;
     const uint4* xr = x + row * ldx;
     u32 m = 0;
-    for (int64_t idx = t; idx < nvec; idx += 256) m = absmax8(m, xr[idx]);
+    for (int64_t idx = t; idx < nvec; idx += 256) m = absmax8(m, xr[idx]);  // kept cacheable: re-read below
     const float amax = amax_from_bits(block_max_256(wave_max(pk_fold(m)), red));
     const float scale = scale_from_amax(amax);
     if (t == 0) scales[row] = scale;
     const Divider d(scale);
     uint2* qr = q + row * ldq;
-    for (int64_t idx = t; idx < nvec; idx += 256) qr[idx] = cast8(xr[idx], d);
+    for (int64_t idx = t; idx < nvec; idx += 256) st8<NTS>(qr + idx, cast8(ld16<true>(xr + idx), d));
 }
 
-int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
-                         float* scales, hipStream_t st) {
-    const uint4* xv = static_cast<const uint4*>(x);
-    uint2* qv = static_cast<uint2*>(q);
-    const int64_t nvec = cols / 8, ldx = ld_x / 8, ldq = ld_q / 8;
-    if (rows > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_rowwise: rows=%lld exceeds the grid limit", (long long)rows);
-#define CFP8_WAVE(V)                                                                                   \
-    hipLaunchKernelGGL(rowwise_wave_kernel<V>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, xv, \
+// streaming_out: write the fp8 bytes with non-temporal stores (weights, consumed much
+// later); false keeps them cacheable (activations feeding the GEMM of the same call).
+template <bool NTS>
+static void launch_rowwise_variant(const uint4* xv, int64_t rows, int64_t nvec, int64_t ldx, uint2* qv, int64_t ldq,
+                                   float* scales, hipStream_t st) {
+#define CFP8_WAVE(V)                                                                                        \
+    hipLaunchKernelGGL((rowwise_wave_kernel<V, NTS>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, xv, \
                        rows, (int)nvec, ldx, qv, ldq, scales)
-#define CFP8_BLOCK(V) \
-    hipLaunchKernelGGL(rowwise_block_kernel<V>, dim3((unsigned)rows), dim3(256), 0, st, xv, (int)nvec, ldx, qv, ldq, scales)
+#define CFP8_BLOCK(V)                                                                                          \
+    hipLaunchKernelGGL((rowwise_block_kernel<V, NTS>), dim3((unsigned)rows), dim3(256), 0, st, xv, (int)nvec, ldx, \
+                       qv, ldq, scales)
     if (nvec <= 64) CFP8_WAVE(1);
     else if (nvec <= 128) CFP8_WAVE(2);
     else if (nvec <= 256) CFP8_WAVE(4);
@@ -113,9 +114,19 @@ int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x
     else if (nvec <= 2048) CFP8_BLOCK(8);
     else if (nvec <= 4096) CFP8_BLOCK(16);
     else
-        hipLaunchKernelGGL(rowwise_stream_kernel, dim3((unsigned)rows), dim3(256), 0, st, xv, nvec, ldx, qv, ldq, scales);
+        hipLaunchKernelGGL(rowwise_stream_kernel<NTS>, dim3((unsigned)rows), dim3(256), 0, st, xv, nvec, ldx, qv, ldq, scales);
 #undef CFP8_WAVE
 #undef CFP8_BLOCK
+}
+
+int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
+                         float* scales, bool streaming_out, hipStream_t st) {
+    const uint4* xv = static_cast<const uint4*>(x);
+    uint2* qv = static_cast<uint2*>(q);
+    const int64_t nvec = cols / 8, ldx = ld_x / 8, ldq = ld_q / 8;
+    if (rows > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_rowwise: rows=%lld exceeds the grid limit", (long long)rows);
+    if (streaming_out) launch_rowwise_variant<true>(xv, rows, nvec, ldx, qv, ldq, scales, st);
+    else launch_rowwise_variant<false>(xv, rows, nvec, ldx, qv, ldq, scales, st);
     return check_launch("quant_rowwise");
 }
 
@@ -133,5 +144,7 @@ extern "C" int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u))
         return set_error(CFP8_EINVAL, "quant_rowwise: x must be 16-byte and q 8-byte aligned");
     if (int rc = check_device()) return rc;
-    return launch_quant_rowwise(x, rows, cols, ld_x, q, ld_q, scales, static_cast<hipStream_t>(stream));
+    // outputs of 32 MiB and more cannot stay cache resident anyway: stream them out
+    return launch_quant_rowwise(x, rows, cols, ld_x, q, ld_q, scales, rows * cols >= (32ll << 20),
+                                static_cast<hipStream_t>(stream));
 }

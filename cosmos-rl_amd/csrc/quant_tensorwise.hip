@@ -3,10 +3,13 @@
 //
 //   pass 1 (amax)  reads 2 B/element.  Every workgroup reduces one contiguous
 //                  chunk of one tensor and publishes its maximum with one
-//                  atomic max on the bit pattern (valid because |x| >= 0, and
-//                  NaN patterns sort above infinity, so NaN propagates).
-//   pass 2 (cast)  reads 2 B and writes 1 B per element; every workgroup forms
-//                  the scale from the tensor's amax slot on its own.
+//                  fire-and-forget atomic max on the bit pattern (valid because
+//                  |x| >= 0, and NaN patterns sort above infinity, so NaN
+//                  propagates).  A tensor owns kAmaxSlots slots and a workgroup
+//                  picks one by its index: thousands of co-resident workgroups
+//                  hitting a single address serialise at the memory side.
+//   pass 2 (cast)  reads 2 B and writes 1 B per element; every workgroup folds
+//                  the tensor's slots and forms the scale on its own.
 // The table of tensors travels in the kernel arguments (scalar loads), so the
 // library needs no device-side descriptor buffer.
 #include <stdlib.h>
@@ -17,13 +20,14 @@ namespace cfp8 {
 
 constexpr int kMaxBatch = 48;
 constexpr int kChunkVecs = 256 * 8;  // 16-byte vectors per workgroup: 32 KiB of bf16
+constexpr int kAmaxSlots = CFP8_TENSORWISE_AMAX_SLOTS;  // one wavefront reads them in one load
 
 struct TensorTable {
     const uint4* x[kMaxBatch];
     uint2* q[kMaxBatch];
     float* scale[kMaxBatch];
     int64_t nvec[kMaxBatch];
-    u32* amax[kMaxBatch];
+    u32* amax[kMaxBatch];  // kAmaxSlots slots each
     unsigned first_block[kMaxBatch + 1];  // exclusive prefix of workgroups per tensor
     int n;
 };
@@ -38,26 +42,29 @@ __device__ __forceinline__ int find_tensor(const TensorTable& tb, unsigned b) {
     return lo;
 }
 
-__global__ __launch_bounds__(64) void tensorwise_zero_kernel(u32* slots, int n) {
-    for (int i = threadIdx.x; i < n; i += 64) slots[i] = 0u;
+__global__ __launch_bounds__(64) void tensorwise_zero_kernel(u32* slots, int64_t n) {
+    const int64_t base = (int64_t)blockIdx.x * 64 * 1024;
+    for (int64_t i = base + threadIdx.x; i < n && i < base + 64 * 1024; i += 64) slots[i] = 0u;
 }
 
+template <bool LDNT>
 __global__ __launch_bounds__(256) void tensorwise_amax_kernel(const TensorTable tb) {
     __shared__ u32 red[4];
     const int t = find_tensor(tb, blockIdx.x);
-    const int64_t base = (int64_t)(blockIdx.x - tb.first_block[t]) * kChunkVecs;
+    const unsigned local = blockIdx.x - tb.first_block[t];
+    const int64_t base = (int64_t)local * kChunkVecs;
     const int64_t nvec = tb.nvec[t];
     const uint4* x = tb.x[t] + base;
     const int64_t left = nvec - base;
     uint4 v[8];
     if (left >= kChunkVecs) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = x[threadIdx.x + 256 * i];
+        for (int i = 0; i < 8; ++i) v[i] = ld16<LDNT>(x + threadIdx.x + 256 * i);
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             int idx = threadIdx.x + 256 * i;
-            v[i] = idx < left ? x[idx] : make_uint4(0, 0, 0, 0);
+            v[i] = idx < left ? ld16<LDNT>(x + idx) : make_uint4(0, 0, 0, 0);
         }
     }
     u32 m = 0;
@@ -68,12 +75,11 @@ __global__ __launch_bounds__(256) void tensorwise_amax_kernel(const TensorTable 
     __syncthreads();
     if (threadIdx.x == 0) {
         m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;  // fp32 bit pattern of the chunk amax
-        u32* slot = tb.amax[t];
-        // the slot only grows, so a stale read can only cause a redundant atomic
-        if (m > __hip_atomic_load(slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(slot, m);
+        if (m) atomicMax(tb.amax[t] + (local & (kAmaxSlots - 1)), m);  // result unused: the wave does not wait
     }
 }
 
+template <bool LDNT, bool STNT>
 __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable tb) {
     const int t = find_tensor(tb, blockIdx.x);
     const unsigned local = blockIdx.x - tb.first_block[t];
@@ -82,21 +88,22 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
     const uint4* x = tb.x[t] + base;
     uint2* q = tb.q[t] + base;
     const int64_t left = nvec - base;
-    const float amax = __uint_as_float(*tb.amax[t]);
+    static_assert(kAmaxSlots == 64, "one slot per lane");
+    const float amax = __uint_as_float(wave_max(tb.amax[t][threadIdx.x & 63]));
     const float scale = scale_from_amax(amax);
     if (local == 0 && threadIdx.x == 0) *tb.scale[t] = scale;
     const Divider d(scale);
     uint4 v[8];
     if (left >= kChunkVecs) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = x[threadIdx.x + 256 * i];
+        for (int i = 0; i < 8; ++i) v[i] = ld16<LDNT>(x + threadIdx.x + 256 * i);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[threadIdx.x + 256 * i] = cast8(v[i], d);
+        for (int i = 0; i < 8; ++i) st8<STNT>(q + threadIdx.x + 256 * i, cast8(v[i], d));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             int idx = threadIdx.x + 256 * i;
-            if (idx < left) q[idx] = cast8(x[idx], d);
+            if (idx < left) st8<STNT>(q + idx, cast8(ld16<LDNT>(x + idx), d));
         }
     }
 }
@@ -106,39 +113,50 @@ static int64_t batch_bytes() {
     static int64_t v = [] {
         const char* e = getenv("CFP8_TW_BATCH_MB");
         long mb = e ? atol(e) : 0;
-        if (mb <= 0) mb = 160;
+        if (mb <= 0) return (int64_t)1 << 60;  // default: no byte limit, 48 tensors per launch
         return (int64_t)mb << 20;
     }();
     return v;
 }
 
-}  // namespace cfp8
+// Access policy, CFP8_TW_MODE overrides (read once).  bit 0: pass 1 loads stream past the
+// caches; bit 1: pass 2 loads do; bit 2: pass 2 stores do.
+static int access_mode() {
+    static int v = [] {
+        const char* e = getenv("CFP8_TW_MODE");
+        return e ? atoi(e) : 7;
+    }();
+    return v;
+}
 
-extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws,
-                                           void* stream) {
-    using namespace cfp8;
-    if (n < 0) return set_error(CFP8_EINVAL, "quant_tensorwise: negative tensor count");
+enum : int { kPhaseAmax = 1, kPhaseCast = 2 };
+
+static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream, int phases) {
+    if (n < 0 || n > (1ll << 24)) return set_error(CFP8_EINVAL, "quant_tensorwise: bad tensor count");
     if (n == 0) return CFP8_OK;
     if (!descs || !amax_ws) return set_error(CFP8_EINVAL, "quant_tensorwise: null descriptor table or amax workspace");
     for (int64_t i = 0; i < n; ++i) {
         const cfp8_tensor_desc& d = descs[i];
         if (d.numel < 0 || d.numel % 8) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld numel=%lld must be a non-negative multiple of 8", (long long)i, (long long)d.numel);
-        if (!d.scale) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null scale pointer", (long long)i);
-        if (d.numel && (!d.x || !d.q)) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null data pointer", (long long)i);
+        if ((phases & kPhaseCast) && !d.scale) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null scale pointer", (long long)i);
+        if (d.numel && (!d.x || ((phases & kPhaseCast) && !d.q))) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld has a null data pointer", (long long)i);
         if (!aligned16(d.x) || (reinterpret_cast<uintptr_t>(d.q) & 7u)) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld is misaligned (x 16 bytes, q 8 bytes)", (long long)i);
         if ((d.numel / 8 + kChunkVecs - 1) / kChunkVecs > 0x3FFFFFFFll) return set_error(CFP8_EINVAL, "quant_tensorwise: tensor %lld is too large for one launch", (long long)i);
     }
     if (int rc = check_device()) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     u32* slots = reinterpret_cast<u32*>(amax_ws);
-    // zero every slot with a kernel (a memset node misbehaves under graph capture)
-    for (int64_t off = 0; off < n; off += 1 << 20) {
-        int cnt = (int)((n - off) < (1 << 20) ? (n - off) : (1 << 20));
-        hipLaunchKernelGGL(tensorwise_zero_kernel, dim3(1), dim3(64), 0, st, slots + off, cnt);
+    if (phases & kPhaseAmax) {
+        // zero every slot with a kernel (a memset node misbehaves under graph capture)
+        const int64_t total = n * kAmaxSlots;
+        const int64_t per = 64 * 1024;
+        hipLaunchKernelGGL(tensorwise_zero_kernel, dim3((unsigned)((total + per - 1) / per)), dim3(64), 0, st, slots, total);
     }
-    // Tensors are taken in batches of at most kMaxBatch entries and batch_bytes()
-    // of bf16; each batch runs pass 1 then pass 2 back to back, so a batch that
-    // fits the 256 MiB memory-side cache is read from HBM once.
+    // Tensors are taken in batches of at most kMaxBatch entries (and batch_bytes() of
+    // bf16 when that tuning knob is set); with both phases requested each batch runs
+    // pass 1 then pass 2 back to back.  Measured on MI355X: few large launches with
+    // streaming accesses beat small batches that would let pass 2 hit the 256 MiB
+    // memory-side cache, because every launch pays a ramp-up and a tail.
     const int64_t budget_vecs = batch_bytes() / 16;
     int64_t i = 0;
     while (i < n) {
@@ -157,7 +175,7 @@ extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_
             tb.q[tb.n] = static_cast<uint2*>(d.q);
             tb.scale[tb.n] = d.scale;
             tb.nvec[tb.n] = nvec;
-            tb.amax[tb.n] = slots + i;
+            tb.amax[tb.n] = slots + i * kAmaxSlots;
             tb.first_block[tb.n] = blocks;
             blocks += nb;
             vecs += nvec;
@@ -165,10 +183,35 @@ extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_
             ++i;
         }
         tb.first_block[tb.n] = blocks;
-        hipLaunchKernelGGL(tensorwise_amax_kernel, dim3(blocks), dim3(256), 0, st, tb);
-        hipLaunchKernelGGL(tensorwise_cast_kernel, dim3(blocks), dim3(256), 0, st, tb);
+        const int mode = access_mode();
+        if (phases & kPhaseAmax) {
+            if (mode & 1) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
+            else hipLaunchKernelGGL(tensorwise_amax_kernel<false>, dim3(blocks), dim3(256), 0, st, tb);
+        }
+        if (phases & kPhaseCast) {
+            switch ((mode >> 1) & 3) {
+                case 0: hipLaunchKernelGGL((tensorwise_cast_kernel<false, false>), dim3(blocks), dim3(256), 0, st, tb); break;
+                case 1: hipLaunchKernelGGL((tensorwise_cast_kernel<true, false>), dim3(blocks), dim3(256), 0, st, tb); break;
+                case 2: hipLaunchKernelGGL((tensorwise_cast_kernel<false, true>), dim3(blocks), dim3(256), 0, st, tb); break;
+                default: hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb); break;
+            }
+        }
     }
     return check_launch("quant_tensorwise");
+}
+
+}  // namespace cfp8
+
+extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {
+    return cfp8::run_tensorwise(descs, n, amax_ws, stream, cfp8::kPhaseAmax | cfp8::kPhaseCast);
+}
+
+extern "C" int cfp8_tensorwise_amax_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {
+    return cfp8::run_tensorwise(descs, n, amax_ws, stream, cfp8::kPhaseAmax);
+}
+
+extern "C" int cfp8_tensorwise_cast_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {
+    return cfp8::run_tensorwise(descs, n, amax_ws, stream, cfp8::kPhaseCast);
 }
 
 extern "C" int cfp8_quant_tensorwise(const void* x, int64_t numel, void* q, float* scale, float* amax_ws,

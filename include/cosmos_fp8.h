@@ -63,8 +63,10 @@ int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
  * then cast), without a host round trip in between.
  * Replaces the torchao tensorwise recipe selected at
  * cosmos_rl/utils/fp8/fp8_util.py:121-137 (hp_tensor_to_float8_dynamic).
- * The descriptor array lives in HOST memory; amax_ws is a device array of n
- * floats (scratch, overwritten).  numel % 8 == 0 for every tensor. */
+ * The descriptor array lives in HOST memory; amax_ws is a device array of
+ * n * CFP8_TENSORWISE_AMAX_SLOTS floats (scratch, overwritten).
+ * numel % 8 == 0 for every tensor. */
+#define CFP8_TENSORWISE_AMAX_SLOTS 64
 typedef struct cfp8_tensor_desc {
     const void* x;   /* bf16, contiguous, 16-byte aligned */
     void* q;         /* fp8 out, numel bytes              */
@@ -75,7 +77,20 @@ typedef struct cfp8_tensor_desc {
 int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
                                 float* amax_ws, void* stream);
 
-/* Single-tensor form of the above. */
+/* Split-phase forms of the above.  Pass 1 alone leaves partial maxima of |x| of
+ * tensor i in amax_ws[i*SLOTS .. i*SLOTS+SLOTS-1] (non-negative fp32 bit
+ * patterns, a NaN pattern if the tensor holds one; their maximum as unsigned
+ * integers is the tensor's amax); pass 2 alone folds those slots, writes scale and
+ * bytes.  Between the two a caller may combine amax_ws across devices with an
+ * elementwise all-reduce max over the uint32 view - the tensor-parallel Float8 case of
+ * cosmos_rl/policy/model/gpt/parallelize.py:268-280.  q and scale may be null
+ * in pass 1. */
+int cfp8_tensorwise_amax_multi(const cfp8_tensor_desc* descs, int64_t n,
+                               float* amax_ws, void* stream);
+int cfp8_tensorwise_cast_multi(const cfp8_tensor_desc* descs, int64_t n,
+                               float* amax_ws, void* stream);
+
+/* Single-tensor form of cfp8_quant_tensorwise_multi. */
 int cfp8_quant_tensorwise(const void* x, int64_t numel, void* q, float* scale,
                           float* amax_ws, void* stream);
 
