@@ -1,0 +1,88 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and rejects
+bad arguments with error codes (never an abort) before it touches a device."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from cosmos_rl_amd import _lib, ops
+
+HEADER = Path(__file__).resolve().parent.parent / "include" / "cosmos_fp8.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(cfp8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    syms = declared_symbols()
+    assert len(syms) >= 15
+    lib = _lib.load()
+    for s in syms:
+        assert hasattr(lib, s), f"{s} declared in the header but not exported"
+        assert s in _lib.SIGNATURES, f"{s} has no ctypes prototype"
+    assert set(_lib.SIGNATURES) == set(syms), "python binds symbols the header does not declare"
+    assert lib.cfp8_version() >= 100
+
+
+def test_header_constants_match_binding():
+    text = HEADER.read_text()
+    val = lambda name: int(re.search(rf"#define {name}\s+\(?(-?\d+)\)?", text).group(1))
+    assert val("CFP8_EINVAL") == _lib.EINVAL and val("CFP8_EARCH") == _lib.EARCH
+    assert val("CFP8_ELAUNCH") == _lib.ELAUNCH and val("CFP8_EWORKSPACE") == _lib.EWORKSPACE
+    assert val("CFP8_OUT_BF16") == _lib.OUT_BF16 and val("CFP8_OUT_F32") == _lib.OUT_F32
+    assert val("CFP8_GROUP_MODE_DIV") == _lib.GROUP_MODE_DIV and val("CFP8_GROUP_MODE_DEEPEP") == _lib.GROUP_MODE_DEEPEP
+    assert val("CFP8_TENSORWISE_AMAX_SLOTS") == _lib.TENSORWISE_AMAX_SLOTS
+    assert ctypes.sizeof(_lib.TensorDesc) == 32
+
+
+def test_argument_errors_need_no_device():
+    lib = _lib.load()
+    # null pointers / bad shapes are rejected before any HIP call
+    assert lib.cfp8_quant_rowwise(None, 4, 16, 16, None, 16, None, None) == _lib.EINVAL
+    assert "null pointer" in _lib.last_error()
+    assert lib.cfp8_quant_rowwise(None, -1, 16, 16, None, 16, None, None) == _lib.EINVAL
+    assert lib.cfp8_quant_block128(None, 1, 128, 128, None, None, 0, None) == _lib.EINVAL
+    assert lib.cfp8_quant_group128(None, 4, 128, 128, None, 128, None, 0, None) == _lib.EINVAL
+    assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
+    assert lib.cfp8_gemm_block128(None, 128, None, None, 128, None, 1, 1, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
+    assert lib.cfp8_quant_tensorwise_multi(None, 3, None, None) == _lib.EINVAL
+    # empty problems succeed without pointers
+    assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
+    assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0
+    assert lib.cfp8_quant_tensorwise_multi(None, 0, None, None) == 0
+    with pytest.raises(ValueError):
+        _lib.check(_lib.EINVAL)
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.ELAUNCH)
+
+
+def test_linear_workspace_bytes():
+    lib = _lib.load()
+    assert lib.cfp8_linear_workspace_bytes(0, 128) == 0
+    n = lib.cfp8_linear_workspace_bytes(64, 3584)
+    assert n >= 64 * 3584 + 64 * 4 and n % 256 == 0
+    # too small a workspace is an error code of its own
+    rc = lib.cfp8_linear_rowwise(None, 3584, None, 3584, None, None, 64, 0, 64, 64, 3584, None, 0, None)
+    assert rc == _lib.EWORKSPACE
+
+
+def test_no_cpu_fallback():
+    """Operators refuse CPU tensors instead of computing somewhere else."""
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    for fn in (ops.quant_rowwise, ops.quant_tensorwise, ops.per_block_cast_to_fp8, ops.groupwise_activation_quant,
+               ops.per_token_cast_to_fp8):
+        with pytest.raises(RuntimeError, match="GPU only"):
+            fn(x)
+    with pytest.raises(NotImplementedError):
+        ops.scaled_fp8_quant(x, scale=torch.ones(1))
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = Path(_lib.__file__).resolve().parent
+    for f in list(pkg.rglob("*.py")) + list((pkg.parent / "csrc").glob("*")):
+        if f.is_file() and f.suffix in (".py", ".hip", ".h"):
+            assert "oracle" not in f.read_text(), f"{f} mentions the oracle"

@@ -1,0 +1,181 @@
+"""The reference-named Python entry points running on the HIP kernels (through the C ABI)."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import fp8_oracle as O
+from cosmos_rl_amd import ops
+from cosmos_rl_amd.policy.kernel import group_gemms
+from cosmos_rl_amd.rollout.vllm_rollout import monkey_patch_for_fp8 as mp
+from cosmos_rl_amd.rollout.vllm_rollout.vllm_rollout import FP8RolloutMixin, fp8_quantization
+from cosmos_rl_amd.rollout.worker.rollout_control import QuantizedWeightReceiver
+from cosmos_rl_amd.utils.fp8 import fp8_util
+
+pytestmark = pytest.mark.gpu
+
+
+class Lin(nn.Module):
+    def __init__(self, w):
+        super().__init__()
+        self.weight = nn.Parameter(w, requires_grad=False)
+        self.quant_method = mp.Fp8LinearMethod()
+
+    def forward(self, x):
+        return self.quant_method.apply(self, x)
+
+
+class Model(nn.Module):
+    def __init__(self, dev):
+        super().__init__()
+        self.qkv_proj = Lin(O.make_weight((4608, 3584), seed=1).to(dev))
+        self.down_proj = Lin(O.make_weight((3584, 2048), seed=2).to(dev))
+
+
+class Mapper:
+    def rollout_map_local_key_to_hf_key(self, n):
+        return n
+
+    def get_unsplited_weight_name(self, n):
+        for p in ("q_proj.", "k_proj.", "v_proj."):
+            if n.startswith(p):
+                return "qkv_proj." + n[len(p):]
+        return n
+
+
+class Rollout(FP8RolloutMixin):
+    def __init__(self, model):
+        self.model = model
+
+    def get_underlying_model(self):
+        return self.model
+
+    def model_param_map(self, mapper):
+        d = {}
+        for name, m in self.model.named_children():
+            d[f"{name}.weight"] = m.weight
+            d[f"{name}.weight_scale"] = m.weight_scale
+        return d
+
+
+def test_weight_sync_end_to_end(dev):
+    """Engine load -> patch -> forward -> a weight sync of the packed qkv weight -> forward."""
+    model = Model(dev)
+    w_qkv = model.qkv_proj.weight.detach().clone()
+    mp.simplify_process_weights_after_loading()
+    for m in model.children():
+        m.quant_method.process_weights_after_loading(m)
+    mp.apply_fp8_linear_patch(model)
+    qo, so = O.quant_rowwise(w_qkv.cpu())
+    assert torch.equal(model.qkv_proj.weight.t().contiguous().view(torch.uint8).cpu(), qo)
+    assert torch.equal(model.qkv_proj.weight_scale.cpu(), so)
+
+    x = O.make_activation(48, 3584, seed=3, chan_outlier_frac=0.005, outlier_mul=30.0)
+    y = model.qkv_proj(x.to(dev))
+    ref = O.fp8_linear_rowwise(x, qo, so, accum=torch.float64)
+    assert y.dtype == torch.bfloat16 and O.rel_frobenius(y.float().cpu(), ref.to(torch.bfloat16).float()) <= 1e-3
+
+    mapper, rollout = Mapper(), Rollout(model)
+    hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
+    view = rollout.post_get_params_for_sync_hook("fp8", mapper, dict(rollout.model_param_map(mapper)), quantized)
+    assert "qkv_proj.weight_scale" not in view
+    recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
+    # first sync: the policy sends the very weights the engine was loaded with -> self check passes
+    hp["qkv_proj.weight"].data.copy_(w_qkv)
+    recv.plan_group(["q_proj.weight", "k_proj.weight", "v_proj.weight"], do_weight_sync_check=True)()
+    # later sync: new weights
+    w_new = O.make_weight((4608, 3584), seed=9, std=0.03)
+    hp["qkv_proj.weight"].data.copy_(w_new.to(dev))
+    assert recv.quantize_full_weight("qkv_proj.weight") is True
+    qn, sn = O.quant_rowwise(w_new)
+    assert torch.equal(model.qkv_proj.weight.t().contiguous().view(torch.uint8).cpu(), qn)
+    assert torch.equal(model.qkv_proj.weight_scale.cpu(), sn)
+    y2 = model.qkv_proj(x.to(dev))
+    ref2 = O.fp8_linear_rowwise(x, qn, sn, accum=torch.float64)
+    assert O.rel_frobenius(y2.float().cpu(), ref2.to(torch.bfloat16).float()) <= 1e-3
+    # a mismatching engine weight fails the first-sync check with the reference's error
+    hp["qkv_proj.weight"].data.mul_(2.0).add_(0.01)
+    with pytest.raises(ValueError, match="FP8 weight doesn't match"):
+        recv.quantize_full_weight("qkv_proj.weight", do_weight_sync_check=True)
+
+
+def test_fp8_quantization_layout(dev):
+    w = O.make_weight((3584, 18944), seed=4).to(dev)
+    qt, s = fp8_quantization(w)
+    assert tuple(qt.shape) == (18944, 3584) and qt.stride() == (1, 18944) and tuple(s.shape) == (3584, 1)
+    param = torch.empty(3584, 18944, dtype=torch.float8_e4m3fn, device=dev).t()
+    param.copy_(qt)                                      # same strides: a flat byte copy
+    assert torch.equal(param.t().contiguous().view(torch.uint8), qt.t().contiguous().view(torch.uint8))
+
+
+def test_float8_linear_recipes(dev):
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = nn.Linear(512, 1024, bias=True)
+            self.lm_head = nn.Linear(512, 256, bias=False)
+
+        def fqn_filter_for_quantization(self):
+            return ["lm_head"]
+
+    x = O.make_activation(40, 512, seed=5)
+    for recipe in ("rowwise", "tensorwise"):
+        torch.manual_seed(0)
+        net = Net().to(dev).to(torch.bfloat16)
+        cfg = SimpleNamespace(train=SimpleNamespace(fp8=fp8_util.FP8Config(enable_fp8=True, quant_recipe=recipe)))
+        fp8_util.FP8ModelConverter(cfg, None).convert_model(net)
+        assert isinstance(net.up, fp8_util.Float8Linear) and type(net.lm_head) is nn.Linear
+        with torch.no_grad():
+            y = net.up(x.to(dev))
+        w, b = net.up.weight.detach().cpu(), net.up.bias.detach().cpu()
+        if recipe == "rowwise":
+            qw, sw = O.quant_rowwise(w)
+            ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
+        else:
+            qw, sw = O.quant_tensorwise(w)
+            qx, sx = O.quant_tensorwise(x)
+            ref = O.scaled_mm_rowwise(qx, sx.expand(40, 1), qw, sw.expand(1024, 1), accum=torch.float64)
+        ref = (ref.to(torch.bfloat16) + b).float()
+        assert y.dtype == torch.bfloat16 and O.rel_frobenius(y.float().cpu(), ref) <= 2e-3
+
+
+def test_ds_group_gemm_strategy(dev):
+    """DSGroupGEMM.arrange_expert_weights + execute against the oracle pipeline
+    (1x128 quant -> grouped gate/up GEMMs -> silu*up -> 1x128 quant -> grouped down GEMM)."""
+    assert group_gemms.DSGroupGEMM.is_available()
+    E, H, I, T, topk = 8, 512, 256, 200, 2
+    g = torch.Generator().manual_seed(11)
+    act = torch.nn.functional.silu
+    strat = group_gemms.DSGroupGEMM(act)
+    mod = nn.Module()
+    weights = {}
+    for name, shape in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+        ws = [O.make_weight(shape, seed=100 + 10 * e + len(name), std=0.05) for e in range(E)]
+        weights[name] = torch.stack(ws)
+        stacked = strat.arrange_expert_weights([w.to(dev) for w in ws], name, mod)
+        mod.register_parameter(f"{name}_weight", nn.Parameter(stacked, requires_grad=False))
+        qo, so = O.quant_block128(weights[name])
+        assert torch.equal(mod.get_parameter(f"{name}_fp8").view(torch.uint8).cpu(), qo)
+        assert torch.equal(mod.get_parameter(f"{name}_scales").cpu(), so)
+    logits = torch.rand(T, E, generator=g)
+    tok, m_idx, m_sizes, m_offsets = O.route_topk_contiguous(logits, topk, 128)
+    x = O.make_activation(T, H, seed=12)
+    xs = torch.zeros(tok.numel(), H, dtype=torch.bfloat16)
+    xs[tok >= 0] = x[tok[tok >= 0]]
+    out = strat.execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+
+    # oracle pipeline; execute() treats every row of a padded group as belonging to that expert
+    full_idx = ops.create_indices_from_offsets_nosync(m_offsets, tok.numel())
+    qx, sx = O.quant_group128(xs)
+    def gmm(name, qa, sa):
+        qb, sb = O.quant_block128(weights[name])
+        return O.grouped_mm_block128(qa, sa, qb, sb, full_idx, accum=torch.float64).to(torch.bfloat16)
+    hidden = act(gmm("gate_proj", qx, sx)) * gmm("up_proj", qx, sx)
+    qh, sh = O.quant_group128(hidden)
+    ref = gmm("down_proj", qh, sh)
+    valid = tok >= 0
+    # bf16 intermediates may differ by an ulp between kernel and oracle, which re-quantisation
+    # can amplify to one e4m3 step on isolated entries: compare in Frobenius norm
+    assert O.rel_frobenius(out[valid].float(), ref[valid].float()) <= 5e-3
+    assert bool((out[~valid] == 0).all())               # zero tokens in, zeros out
