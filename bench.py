@@ -29,6 +29,10 @@ for p in (str(ROOT), str(ROOT / "cosmos-rl_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per cast-kernel launch (average of the 5 launches of a step) measured with
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for a plain
+# 1 GiB copy (x2.000 and x1.000): 2.828e9 read + 1.414e9 written.  Valid for the default workload.
+CAST_TRAFFIC_BYTES_PER_LAUNCH = 4_242_000_000
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 
 QWEN25_7B = [("q_proj", (3584, 3584), 28), ("o_proj", (3584, 3584), 28), ("k_proj", (512, 3584), 28),
@@ -43,6 +47,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three plain 1 GiB device copies, to calibrate HBM traffic counters under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no cross-GPU step on a single "
@@ -133,7 +139,7 @@ def main() -> int:
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(cast_bytes / (cast_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": CAST_TRAFFIC_BYTES_PER_LAUNCH if (n == 197 and launches == 5) else None,
         "bytes_per_launch": cast_bytes // launches,
         "launches_per_step": launches,
         "avg_launch_ms": round(cast_med / launches, 4),
@@ -141,6 +147,14 @@ def main() -> int:
                         "frac": round(2 * numel / (amax_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                         "avg_launch_ms": round(amax_med / launches, 4)},
     }
+
+    if args.copy_probe:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)          # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     del outs
     extra = {}

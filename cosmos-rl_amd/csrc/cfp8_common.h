@@ -182,8 +182,13 @@ __device__ __forceinline__ u32 f32_to_bf16_bits(float f) {
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
     return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
+// two fp32 -> packed bf16 (round to nearest even) with the gfx950 conversion instruction
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ u32 pack_bf16x2(float a, float b) {
-    return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+    f32x2 v;
+    v[0] = a;
+    v[1] = b;
+    return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2_t));
 }
 
 }  // namespace cfp8

@@ -10,10 +10,13 @@
 // (l & 15) and the 32 K-bytes of quarter (l >> 4) for both operands; any
 // permutation of K shared by both operands leaves the dot products unchanged.
 //
-// Tiles: BM x BN x 128 per workgroup, LDS double-buffered.  An LDS tile is
-// [rows][128 bytes]; the 16-byte chunk c of row r is stored at chunk slot
-// c ^ ((r >> 1) & 7), which makes both the 16-byte stores (8 lanes per row) and
-// the MFMA operand reads (16 lanes = 16 rows, same chunk) bank-conflict free.
+// Tiles: BM x BN x 128 per workgroup, LDS double-buffered.  An LDS tile is a
+// sequence of 16-row blocks of 2 KiB; inside a block the 16-byte chunk c (0..7)
+// of row r (0..15) sits at  c * 256 + ((r ^ ((c & 1) << 3)) << 4).  An MFMA
+// operand read (16 consecutive lanes = 16 rows, same chunk) then covers one
+// contiguous 256-byte segment - all 64 banks once - and a staging store (16
+// consecutive lanes = 8 rows x 2 adjacent chunks) does too; measured on gfx950 a
+// row-major tile with an XOR swizzle reads at half the LDS rate.
 //
 // Scaling: fp32 scales cannot ride in the MFMA (its scale operands are E8M0), so
 //   rowwise:  acc over all of K, epilogue acc * sa[m] * sb[n];
@@ -38,11 +41,13 @@ struct GemmArgs {
     int tiles_m, tiles_n;
 };
 
+__device__ __forceinline__ int lds_chunk_offset(int row, int c) {
+    return ((row >> 4) << 11) + (c << 8) + ((((row & 15) ^ ((c & 1) << 3))) << 4);
+}
+
 __device__ __forceinline__ i32x8 lds_frag(const uint8_t* tile, int row, int quarter) {
-    const int sw = (row >> 1) & 7;
-    const uint8_t* base = tile + row * 128;
-    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + (((2 * quarter) ^ sw) << 4));
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + (((2 * quarter + 1) ^ sw) << 4));
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(tile + lds_chunk_offset(row, 2 * quarter));
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(tile + lds_chunk_offset(row, 2 * quarter + 1));
     i32x8 r;
     r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
     r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
@@ -68,12 +73,10 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 }
 
 template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs p) {
+__global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
     constexpr int TM = WTM / 16, TN = WTN / 16;  // MFMA tiles per wave
-    constexpr int A_CH = BM * 8, B_CH = BN * 8;  // 16-byte chunks per K step
-    constexpr int A_IT = (A_CH + NT - 1) / NT, B_IT = (B_CH + NT - 1) / NT;
     static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the MFMA tile");
     static_assert(MODE == kRowwise || WTN <= 128, "a wave's n range must stay inside one 128-block");
 
@@ -101,41 +104,38 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs p) {
     const int lrow = lane & 15, quarter = lane >> 4;
     const int KT = p.K >> 7;
 
-    // global -> register staging of one K step
+    // global -> register staging of one K step.  One wave-wide load covers 8 rows x
+    // 128 bytes (8 full cache lines): lane = pair * 16 + row8 * 2 + half reads chunk
+    // 2 * pair + half of row row8.
+    constexpr int A_BLK = BM / 8, B_BLK = BN / 8, NW = NT / 64;
+    constexpr int A_IT = (A_BLK + NW - 1) / NW, B_IT = (B_BLK + NW - 1) / NW;
+    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
     uint4 ra[A_IT], rb[B_IT];
     auto load_tile = [&](int kt) {
-        const int64_t k = (int64_t)kt << 7;
+        const int64_t k = ((int64_t)kt << 7) + st_c * 16;
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) {
-            const int id = t + NT * i;
-            const int r = id >> 3, c = id & 7;
-            const bool ok = (A_CH % NT == 0 || id < A_CH) && (m0 + r) < p.M;
-            ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + (int64_t)(m0 + r) * p.ld_a + k + c * 16)
-                       : make_uint4(0, 0, 0, 0);
+            const int r = (wave + NW * i) * 8 + st_row8;
+            const bool ok = (A_BLK % NW == 0 || r < BM) && (m0 + r) < p.M;
+            ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + (int64_t)(m0 + r) * p.ld_a + k) : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) {
-            const int id = t + NT * i;
-            const int r = id >> 3, c = id & 7;
-            const bool ok = (B_CH % NT == 0 || id < B_CH) && (n0 + r) < p.N;
-            rb[i] = ok ? *reinterpret_cast<const uint4*>(bptr + (int64_t)(n0 + r) * p.ld_b + k + c * 16)
-                       : make_uint4(0, 0, 0, 0);
+            const int r = (wave + NW * i) * 8 + st_row8;
+            const bool ok = (B_BLK % NW == 0 || r < BN) && (n0 + r) < p.N;
+            rb[i] = ok ? *reinterpret_cast<const uint4*>(bptr + (int64_t)(n0 + r) * p.ld_b + k) : make_uint4(0, 0, 0, 0);
         }
     };
     auto store_tile = [&](int stage) {
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) {
-            const int id = t + NT * i;
-            const int r = id >> 3, c = id & 7;
-            if (A_CH % NT == 0 || id < A_CH)
-                *reinterpret_cast<uint4*>(As(stage) + r * 128 + ((c ^ ((r >> 1) & 7)) << 4)) = ra[i];
+            const int r = (wave + NW * i) * 8 + st_row8;
+            if (A_BLK % NW == 0 || r < BM) *reinterpret_cast<uint4*>(As(stage) + lds_chunk_offset(r, st_c)) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) {
-            const int id = t + NT * i;
-            const int r = id >> 3, c = id & 7;
-            if (B_CH % NT == 0 || id < B_CH)
-                *reinterpret_cast<uint4*>(Bs(stage) + r * 128 + ((c ^ ((r >> 1) & 7)) << 4)) = rb[i];
+            const int r = (wave + NW * i) * 8 + st_row8;
+            if (B_BLK % NW == 0 || r < BN) *reinterpret_cast<uint4*>(Bs(stage) + lds_chunk_offset(r, st_c)) = rb[i];
         }
     };
 
@@ -167,13 +167,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs p) {
         }
 
         // weight fragments stay live for the whole step; activation fragments are
-        // read one 16-row tile at a time to bound register pressure
+        // read one 16-row tile ahead of the MFMAs that consume them
         i32x8 fa[TN];
 #pragma unroll
         for (int i = 0; i < TN; ++i) fa[i] = lds_frag(Bs(cur), wn * WTN + i * 16 + lrow, quarter);
+        i32x8 fb = lds_frag(As(cur), wm * WTM + lrow, quarter);
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
-            const i32x8 fb = lds_frag(As(cur), wm * WTM + j * 16 + lrow, quarter);
+            i32x8 fb_next = fb;
+            if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
             if (MODE == kRowwise) {
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
@@ -188,6 +190,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs p) {
                     for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], s, acc[i][j][e]);
                 }
             }
+            fb = fb_next;
         }
 
         if (kt + 1 < KT) store_tile(cur ^ 1);
