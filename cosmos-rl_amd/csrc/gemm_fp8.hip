@@ -225,6 +225,220 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Rowwise GEMM, large full tiles: 256 x 256 x 128 per workgroup, four wavefronts
+// (one per SIMD, 2 x 2), each owning a 128 x 128 block = 64 accumulators of
+// 16 x 16 (all 256 AGPRs).  With one wave per SIMD nothing hides a stall, so the
+// K step is written as a software pipeline of 32 groups of two MFMAs, each
+// group preceded by at most one global load or LDS store and one fragment read:
+//
+//   S0 (w0,x0): LDS reads x1          + stores of the staged tile kt+1 (first half)
+//   S1 (w0,x1): LDS reads w1          + stores (second half)
+//   -- wait for own LDS traffic, barrier: stage nxt complete, stage cur free --
+//   S2 (w1,x0): LDS reads next w0     + global loads of tile kt+2 (first half) -> registers
+//   S3 (w1,x1): LDS reads next x0     + global loads (second half)
+//
+// so a global load has a full K step (~2048 MFMA cycles) to land before its LDS
+// store, and every fragment is read at least 16 MFMAs before its first use.
+// The epilogue turns each wave's block through LDS so that every global store
+// is 16 bytes per lane and 256 contiguous bytes per output row, non-temporal
+// (the output must not evict operand tiles from L2).
+// Requires M % 256 == 0 and N % 256 == 0 (every address is then a per-lane part
+// plus a wave-uniform part).
+// Measured on config 3, M = 8192: 2.05 PFLOP/s against 1.55 for the 8-wave
+// kernel above; a variant with direct-to-LDS loads (global_load_lds_dwordx4) was
+// correct but slower: each such load holds the wave's issue for > 100 cycles.
+// ---------------------------------------------------------------------------
+#define CFP8_PHASE_END() __builtin_amdgcn_sched_barrier(0)
+#define CFP8_MMA2(wb, wh, xb, xh, g)                                                                   \
+    {                                                                                                  \
+        _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                \
+            const int j = (g) >> 1, i = ((g)&1) * 2 + e;                                               \
+            acc[(wh)*4 + i][(xh)*4 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(            \
+                W[wb][i], X[xb][j], acc[(wh)*4 + i][(xh)*4 + j], 0, 0, 0, 0, 0, 0);                    \
+        }                                                                                              \
+    }
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p) {
+    constexpr int BM = 256, BN = 256;
+    constexpr int STAGE = (BM + BN) * 128;  // 64 KiB
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+
+    // global -> registers -> LDS.  Per K step 64 wave-wide loads of 1 KiB (8 rows x 128 B): wave w
+    // takes u = w, w + 4, ...; u < 32: activation rows u * 8 .., u >= 32: weight rows (u - 32) * 8 ..
+    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
+    const uint8_t* a_base = p.a + (int64_t)m0 * p.ld_a;  // wave-uniform
+    const uint8_t* b_base = p.b + (int64_t)n0 * p.ld_b;
+    const int uodd = wave & 1;  // u & 1 is the same for all of a wave's loads
+    const uint32_t va_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_a + (uint32_t)(st_c * 16);
+    const uint32_t vb_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_b + (uint32_t)(st_c * 16);
+    const int l_lane = lds_chunk_offset(uodd * 8 + st_row8, st_c);
+    i32x4 R[16];  // ext-vector type on purpose: an array of uint4 structs stays in scratch memory
+    auto gload = [&](int kt, int i) {
+        const int u = wave + 4 * i, isB = u >> 5, rb = (u & 31) >> 1;
+        const uint8_t* base = isB ? b_base + (int64_t)rb * 16 * p.ld_b : a_base + (int64_t)rb * 16 * p.ld_a;
+        R[i] = *reinterpret_cast<const i32x4*>(base + ((int64_t)kt << 7) + (isB ? vb_lane : va_lane));
+    };
+    auto lstore = [&](int stage, int i) {
+        const int u = wave + 4 * i, isB = u >> 5, rb = (u & 31) >> 1;
+        *reinterpret_cast<i32x4*>(smem + stage * STAGE + isB * (BM * 128) + rb * 2048 + l_lane) = R[i];
+    };
+
+    f32x4 acc[8][8];  // [n tile][m tile]
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int x_off = lds_chunk_offset(wm * 128 + lrow, 2 * quarter);
+    const int x_off2 = lds_chunk_offset(wm * 128 + lrow, 2 * quarter + 1);
+    const int w_off = BM * 128 + lds_chunk_offset(wn * 128 + lrow, 2 * quarter);
+    const int w_off2 = BM * 128 + lds_chunk_offset(wn * 128 + lrow, 2 * quarter + 1);
+    auto frag = [&](int stage, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage * STAGE + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+    i32x8 W[2][4], X[2][4];  // weight / activation fragments of the two halves of the wave's block
+
+    // prologue: tile 0 -> stage 0 (through registers), tile 1 -> registers
+#pragma unroll
+    for (int i = 0; i < 16; ++i) gload(0, i);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) lstore(0, i);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) gload(KT > 1 ? 1 : 0, i);
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        W[0][g] = frag(0, w_off, w_off2, g);
+        X[0][g] = frag(0, x_off, x_off2, g);
+    }
+    CFP8_PHASE_END();
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1, nxt = cur ^ 1;
+        const int ktl = kt + 2 < KT ? kt + 2 : KT - 1;  // past the end: re-read the last tile, never consumed
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) X[1][g] = frag(cur, x_off, x_off2, 4 + g);
+            lstore(nxt, g);
+            CFP8_MMA2(0, 0, 0, 0, g);
+            CFP8_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) W[1][g] = frag(cur, w_off, w_off2, 4 + g);
+            lstore(nxt, 8 + g);
+            CFP8_MMA2(0, 0, 1, 1, g);
+            CFP8_PHASE_END();
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        CFP8_PHASE_END();
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            gload(ktl, g);
+            if (g < 4) W[0][g] = frag(nxt, w_off, w_off2, g);  // after the last step: stale data, unused
+            CFP8_MMA2(1, 1, 0, 0, g);
+            CFP8_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            gload(ktl, 8 + g);
+            if (g < 4) X[0][g] = frag(nxt, x_off, x_off2, g);
+            CFP8_MMA2(1, 1, 1, 1, g);
+            CFP8_PHASE_END();
+        }
+    }
+
+    float sam[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sam[j] = p.sa[m0 + wm * 128 + j * 16 + lrow];
+    if (OUT_F32) {
+        // a lane already owns 16 contiguous bytes: store directly
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int n = n0 + wn * 128 + i * 16 + quarter * 4;
+            const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int m = m0 + wm * 128 + j * 16 + lrow;
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[e];
+                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: scale, convert, turn the wave's 128 x 128 block through LDS in two halves of 64 rows
+    // (row stride 272 B keeps the 8-byte stores of 16 rows on different banks)
+    __syncthreads();  // all waves are done reading the operand stages
+    constexpr int EST = 272;
+    uint8_t* const ebuf = smem + wave * (64 * EST);
+    f32x4 sbn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(p.sb + n0 + wn * 128 + i * 16 + quarter * 4);
+    const int rd_row = lane >> 4, rd_chunk = lane & 15;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = h * 4 + jj;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
+                *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = r * 4 + rd_row;  // 0..63 within the half
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            const int m = m0 + wm * 128 + h * 64 + row;
+            __builtin_nontemporal_store(
+                d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 128 + rd_chunk * 8));
+        }
+    }
+}
+
+static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 256;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    constexpr size_t lds = (size_t)2 * 512 * 128;
+    static bool raised[2] = {false, false};
+    const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
+    const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256_kernel<true>)
+                       : reinterpret_cast<const void*>(gemm_rowwise_256_kernel<false>);
+    if (!raised[v]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
+        raised[v] = true;
+    }
+    if (v) hipLaunchKernelGGL(gemm_rowwise_256_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL(gemm_rowwise_256_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    return check_launch("gemm");
+}
+
 template <int BM, int BN, int WM, int WN, int MODE>
 static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -256,6 +470,8 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (p.M <= 16) return launch_cfg<16, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
+    if (p.M % 256 == 0 && p.N % 256 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0)
+        return launch_rowwise_256(p, out_dtype, st);
     return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);
 }
 
