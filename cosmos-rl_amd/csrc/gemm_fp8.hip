@@ -439,6 +439,212 @@ static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// ---------------------------------------------------------------------------
+// Rowwise GEMM for M <= 64 (decode-time batches): the 18944 x 3584 weight is read
+// once and nothing else matters, so the kernel is a weight streamer bounded by
+// HBM.  A workgroup of 8 waves owns 64 weight rows; wave (nt, kh) takes the 16
+// rows of n-tile nt and the kh-th half of every 512-byte K chunk, reads its
+// weight fragments straight from global memory into MFMA operand registers
+// (streaming loads, two K steps ahead) and the activation fragments of the
+// chunk from LDS, where the workgroup stages them once per chunk (activations of
+// 64 tokens are as many bytes per chunk as the workgroup's weights, so they must
+// not be re-read per wave).  The two K halves are summed through LDS at the end.
+// ---------------------------------------------------------------------------
+template <int TM, bool OUT_F32>
+__global__ __launch_bounds__(512) void gemm_rowwise_skinny_kernel(const GemmArgs p) {
+    constexpr int KS = 4;                         // K steps (of 128) per chunk
+    constexpr int XSTAGE = KS * TM * 2048;        // bytes of one activation stage
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int nt = wave & 3, kh = wave >> 2;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * 64;
+    const int KT = p.K >> 7;
+    const int chunks = (KT + KS - 1) / KS;
+
+    // activation staging: one wave-wide load = 8 rows x 128 bytes of one K step
+    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
+    i32x4 xr[TM];
+    auto xload = [&](int chunk) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int unit = wave + 8 * i, ks = unit & 3, row = (unit >> 2) * 8 + st_row8;
+            const int kt = chunk * KS + ks;
+            const bool ok = row < p.M && kt < KT;
+            xr[i] = ok ? *reinterpret_cast<const i32x4*>(p.a + (int64_t)row * p.ld_a + ((int64_t)kt << 7) + st_c * 16)
+                       : i32x4{0, 0, 0, 0};
+        }
+    };
+    auto xstore = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int unit = wave + 8 * i, ks = unit & 3, row = (unit >> 2) * 8 + st_row8;
+            *reinterpret_cast<i32x4*>(smem + stage * XSTAGE + (ks * TM + (row >> 4)) * 2048 + lds_chunk_offset(row & 15, st_c)) = xr[i];
+        }
+    };
+    // weight fragments: this wave's two K steps of a chunk, 32 contiguous bytes per lane and step
+    const int wrow = n0 + nt * 16 + lrow;
+    const bool wok = wrow < p.N;
+    const uint8_t* wptr = p.b + (int64_t)(wok ? wrow : 0) * p.ld_b + quarter * 32;
+    i32x8 wf[2];
+    auto wload = [&](int chunk) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int kt = chunk * KS + kh * 2 + h;
+            if (wok && kt < KT) {
+                const u32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7)));
+                const u32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7) + 16));
+                wf[h][0] = lo[0]; wf[h][1] = lo[1]; wf[h][2] = lo[2]; wf[h][3] = lo[3];
+                wf[h][4] = hi[0]; wf[h][5] = hi[1]; wf[h][6] = hi[2]; wf[h][7] = hi[3];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) wf[h][e] = 0;
+            }
+        }
+    };
+
+    f32x4 acc[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    xload(0);
+    wload(0);
+    xstore(0);
+    __syncthreads();
+    for (int c = 0; c < chunks; ++c) {
+        const int cur = c & 1;
+        i32x8 wcur[2] = {wf[0], wf[1]};
+        if (c + 1 < chunks) {
+            xload(c + 1);
+            wload(c + 1);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int ks = kh * 2 + h;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const i32x8 fx = lds_frag(smem + cur * XSTAGE + (ks * TM + j) * 2048, lrow, quarter);
+                acc[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wcur[h], fx, acc[j], 0, 0, 0, 0, 0, 0);
+            }
+        }
+        if (c + 1 < chunks) xstore(cur ^ 1);
+        __syncthreads();
+    }
+
+    // sum the two K halves through LDS (the stages are free now), then scale and store
+    float* red = reinterpret_cast<float*>(smem);
+    if (kh == 1) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) *reinterpret_cast<f32x4*>(red + ((nt * TM + j) * 64 + lane) * 4) = acc[j];
+    }
+    __syncthreads();
+    if (kh == 0) {
+        const int n = n0 + nt * 16 + quarter * 4;
+        if (n < p.N) {
+            const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int m = j * 16 + lrow;
+                if (m >= p.M) continue;
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + ((nt * TM + j) * 64 + lane) * 4);
+                const float sam = p.sa[m];
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (acc[j][e] + o[e]) * sam * sbn[e];
+                if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+                else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                        make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Rowwise GEMM for M <= 16 (single-token decode): no LDS staging and no barrier
+// in the loop.  A workgroup owns 16 weight rows; its four waves split K (wave w
+// takes K steps w, w + 4, ...), each issuing the loads of eight K steps (16 KiB
+// of weights per wave) before the first MFMA.  The few activation rows come
+// straight from global memory (they stay in L2), rows >= M are zero.
+// ---------------------------------------------------------------------------
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_rowwise_gemv_kernel(const GemmArgs p) {
+    __shared__ __attribute__((aligned(16))) float red[3 * 64 * 4];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int KT = p.K >> 7;
+    const int wrow = n0 + lrow;
+    const bool wok = wrow < p.N, xok = lrow < p.M;
+    const uint8_t* wptr = p.b + (int64_t)(wok ? wrow : 0) * p.ld_b + quarter * 32;
+    const uint8_t* xptr = p.a + (int64_t)(xok ? lrow : 0) * p.ld_a + quarter * 32;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = wave; base < KT; base += 32) {
+        u32x4 wl[8], wh[8], xl[8], xh[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int kt = base + 4 * i;
+            const bool in = kt < KT;
+            const int64_t off = (int64_t)(in ? kt : 0) << 7;
+            wl[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + off));
+            wh[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + off + 16));
+            xl[i] = *reinterpret_cast<const u32x4*>(xptr + off);
+            xh[i] = *reinterpret_cast<const u32x4*>(xptr + off + 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool in = base + 4 * i < KT;
+            i32x8 fw, fx;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                fw[e] = (in && wok) ? (int)wl[i][e] : 0;
+                fw[4 + e] = (in && wok) ? (int)wh[i][e] : 0;
+                fx[e] = (in && xok) ? (int)xl[i][e] : 0;
+                fx[4 + e] = (in && xok) ? (int)xh[i][e] : 0;
+            }
+            acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fw, fx, acc, 0, 0, 0, 0, 0, 0);
+        }
+    }
+    if (wave > 0) *reinterpret_cast<f32x4*>(red + ((wave - 1) * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + quarter * 4, m = lrow;
+        if (n < p.N && m < p.M) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) {
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + (w * 64 + lane) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += o[e];
+            }
+            const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
+            const float sam = p.sa[m];
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[e] * sam * sbn[e];
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+    }
+}
+
+static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
+    const int64_t blocks = (p.N + 15) / 16;
+    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(gemm_rowwise_gemv_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(gemm_rowwise_gemv_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, p);
+    return check_launch("gemm");
+}
+
+template <int TM>
+static int launch_rowwise_skinny(GemmArgs& p, int out_dtype, hipStream_t st) {
+    const int64_t blocks = (p.N + 63) / 64;
+    constexpr size_t lds = (size_t)2 * 4 * TM * 2048;   // >= the 4 * TM * 1 KiB of the final reduction
+    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, true>), dim3((unsigned)blocks), dim3(512), lds, st, p);
+    else hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, false>), dim3((unsigned)blocks), dim3(512), lds, st, p);
+    return check_launch("gemm");
+}
+
 template <int BM, int BN, int WM, int WN, int MODE>
 static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -467,6 +673,11 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
 template <int MODE>
 static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
+    if (MODE == kRowwise && p.M <= 64) {
+        if (p.M <= 16) return launch_rowwise_gemv(p, out_dtype, st);
+        if (p.M <= 32) return launch_rowwise_skinny<2>(p, out_dtype, st);
+        return launch_rowwise_skinny<4>(p, out_dtype, st);
+    }
     if (p.M <= 16) return launch_cfg<16, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
