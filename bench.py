@@ -47,6 +47,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--extra-filter", default="", help="run only the secondary kernels whose name contains this text")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 1 GiB device copies, to calibrate HBM traffic counters under rocprofv3 --pmc")
     args = ap.parse_args()
@@ -159,7 +160,7 @@ def main() -> int:
     del outs
     extra = {}
     if not args.no_extra:
-        extra = run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors)
+        extra = run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, args.extra_filter)
     del tensors
     torch.cuda.empty_cache()
 
@@ -204,18 +205,22 @@ def _time_events(torch, fn, warmup, iters, flush=None):
     return statistics.median(ms), min(ms)
 
 
-def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors):
+def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     """Secondary kernels of the path; each entry carries its own roofline fraction."""
     check = _lib.check
     flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=dev)
     out = {}
 
     def hbm(name, bytes_, fn, iters=20):
+        if only and only not in name:
+            return
         med, mn = _time_events(torch, fn, 3, iters, flush)
         out[name] = {"ms": round(med, 4), "GB/s": round(bytes_ / (med * 1e-3) / 1e9, 1),
                      "frac_hbm": round(bytes_ / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     def mfma(name, flops, bytes_, fn, iters=20):
+        if only and only not in name:
+            return
         med, mn = _time_events(torch, fn, 3, iters, flush)
         tf = flops / (med * 1e-3) / 1e12
         gbs = bytes_ / (med * 1e-3) / 1e9
@@ -321,8 +326,9 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors):
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
     mfma("grouped_cfg5_gate_up_down_incl_act_quant", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=10)
-    out["grouped_cfg5_gate_up_down_incl_act_quant"]["routed_rows"] = routed
-    out["grouped_cfg5_gate_up_down_incl_act_quant"]["padded_rows"] = total
+    if "grouped_cfg5_gate_up_down_incl_act_quant" in out:
+        out["grouped_cfg5_gate_up_down_incl_act_quant"]["routed_rows"] = routed
+        out["grouped_cfg5_gate_up_down_incl_act_quant"]["padded_rows"] = total
     return out
 
 

@@ -172,25 +172,41 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int i = 0; i < TN; ++i) fa[i] = lds_frag(Bs(cur), wn * WTN + i * 16 + lrow, quarter);
         i32x8 fb = lds_frag(As(cur), wm * WTM + lrow, quarter);
+        if (MODE == kRowwise) {
 #pragma unroll
-        for (int j = 0; j < TM; ++j) {
-            i32x8 fb_next = fb;
-            if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
-            if (MODE == kRowwise) {
+            for (int j = 0; j < TM; ++j) {
+                i32x8 fb_next = fb;
+                if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, acc[i][j], 0, 0, 0, 0, 0, 0);
-            } else {
-                const float s = s_m[j] * s_n;
+                fb = fb_next;
+            }
+        } else {
+            // block scaling: the products of m-tile j go to `part`; their scaled accumulation runs
+            // one m-tile later, while the matrix pipe works on the next m-tile
+            f32x4 part[TN];
 #pragma unroll
-                for (int i = 0; i < TN; ++i) {
-                    const f32x4 part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        fa[i], fb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            for (int j = 0; j <= TM; ++j) {
+                f32x4 prev[TN];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(part[e], s, acc[i][j][e]);
+                for (int i = 0; i < TN; ++i) prev[i] = part[i];
+                if (j < TM) {
+                    i32x8 fb_next = fb;
+                    if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
+#pragma unroll
+                    for (int i = 0; i < TN; ++i)
+                        part[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+                    fb = fb_next;
+                }
+                if (j > 0) {
+                    const float sc = s_m[j - 1] * s_n;
+#pragma unroll
+                    for (int i = 0; i < TN; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(prev[i][e], sc, acc[i][j - 1][e]);
                 }
             }
-            fb = fb_next;
         }
 
         if (kt + 1 < KT) store_tile(cur ^ 1);
