@@ -62,8 +62,15 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     const int total = tiles_m * tiles_n;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = total >> 3, rem = total & 7;
+#ifdef CFP8_NO_XCD_REMAP
+    const int lin = pid;
+#else
     const int lin = xcd * base + (xcd < rem ? xcd : rem) + local;
-    constexpr int GM = 8;
+#endif
+#ifndef CFP8_GM
+#define CFP8_GM 8
+#endif
+    constexpr int GM = CFP8_GM;
     const int band = GM * tiles_n;
     const int g = lin / band, first = g * GM;
     const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;
@@ -214,6 +221,53 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     }
 
     // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+    if constexpr (!OUT_F32 && BM >= 128) {
+        // bf16, large tiles: scale, convert and turn the wave's block through LDS so that global
+        // stores are 16 bytes per lane, a full row segment of the wave's block at a time, and
+        // non-temporal (the output must not evict operand tiles from L2)
+        constexpr int EST = WTN * 2 + 16;             // LDS row stride in bytes
+        constexpr int LPR = WTN / 8;                  // lanes (16-byte chunks) per row
+        constexpr int RPI = 64 / LPR;                 // rows per wave-wide store
+        constexpr int HR = WTM / 2;                   // the block goes through LDS in two halves of HR rows
+        static_assert(HR % 16 == 0 && WM * WN * HR * EST <= 2 * (BM + BN) * 128, "epilogue buffer must fit the operand stages");
+        __syncthreads();                              // every wave is done reading the operand stages
+        uint8_t* const ebuf = smem + wave * (HR * EST);
+        const int rd_row = lane / LPR, rd_chunk = lane % LPR;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int jj = 0; jj < TM / 2; ++jj) {
+                const int j = h * (TM / 2) + jj;
+                const int m = m0 + wm * WTM + j * 16 + lrow;
+                const float sam = (MODE == kRowwise && m < p.M) ? p.sa[m] : 1.f;
+#pragma unroll
+                for (int i = 0; i < TN; ++i) {
+                    f32x4 v = acc[i][j];
+                    if (MODE == kRowwise) {
+                        const int n = n0 + wn * WTN + i * 16 + quarter * 4;
+                        const f32x4 sbn = n < p.N ? *reinterpret_cast<const f32x4*>(p.sb + n) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = v[e] * sam * sbn[e];
+                    }
+                    *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                        make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                }
+            }
+            // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+            for (int r = 0; r < HR / RPI; ++r) {
+                const int row = r * RPI + rd_row;
+                const int m = m0 + wm * WTM + h * HR + row, n = n0 + wn * WTN + rd_chunk * 8;
+                bool ok = m < p.M && n < p.N;         // N % 16 == 0: an 8-wide chunk is inside or outside as a whole
+                if (MODE == kGrouped && ok) ok = p.m_indices[m] == expert;
+                if (ok) {
+                    const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+                    __builtin_nontemporal_store(d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n));
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + wm * WTM + j * 16 + lrow;
