@@ -79,7 +79,7 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     tn = in / gsz;
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32>
+template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32, bool SCALE_VEC>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
@@ -117,33 +117,91 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     constexpr int A_BLK = BM / 8, B_BLK = BN / 8, NW = NT / 64;
     constexpr int A_IT = (A_BLK + NW - 1) / NW, B_IT = (B_BLK + NW - 1) / NW;
     const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
-    uint4 ra[A_IT], rb[B_IT];
+    // Every load below is unconditional and the K loop has no branch, so that the compiler can
+    // count outstanding loads exactly and wait only for the ones it needs: rows past the edge of
+    // a matrix read the last valid row instead (their products land in outputs that are never
+    // stored), and steps past the end of K re-read the last tile.
+    // Addresses are a wave-uniform 64-bit base plus a 32-bit lane offset (a tile spans fewer
+    // than 2^32 bytes for any leading dimension below 2^24).
+    i32x4 ra[A_IT], rb[B_IT];
+    uint32_t oa[A_IT], ob[B_IT];
+    const uint8_t* const abase = p.a + (int64_t)m0 * p.ld_a;
+    const uint8_t* const bbase = bptr + (int64_t)n0 * p.ld_b;
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) {
+        const int r = (wave + NW * i) * 8 + st_row8;
+        const int rr = (m0 + r) < p.M ? r : (p.M - 1 - m0);
+        oa[i] = (uint32_t)rr * (uint32_t)p.ld_a + st_c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) {
+        const int r = (wave + NW * i) * 8 + st_row8;
+        const int rr = (n0 + r) < p.N ? r : (p.N - 1 - n0);
+        ob[i] = (uint32_t)rr * (uint32_t)p.ld_b + st_c * 16;
+    }
     auto load_tile = [&](int kt) {
-        const int64_t k = ((int64_t)kt << 7) + st_c * 16;
+        const int64_t k = (int64_t)(kt < KT ? kt : KT - 1) << 7;
+        const uint8_t* const ak = abase + k;
+        const uint8_t* const bk = bbase + k;
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const i32x4*>(ak + oa[i]);
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const i32x4*>(bk + ob[i]);
+    };
+    // LDS stores number `first` .. `last`-1 of the A_IT + B_IT that make up one staged tile
+    auto store_part = [&](int stage, int first, int last) {
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) {
             const int r = (wave + NW * i) * 8 + st_row8;
-            const bool ok = (A_BLK % NW == 0 || r < BM) && (m0 + r) < p.M;
-            ra[i] = ok ? *reinterpret_cast<const uint4*>(p.a + (int64_t)(m0 + r) * p.ld_a + k) : make_uint4(0, 0, 0, 0);
+            if (i >= first && i < last && (A_BLK % NW == 0 || r < BM))
+                *reinterpret_cast<i32x4*>(As(stage) + lds_chunk_offset(r, st_c)) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) {
             const int r = (wave + NW * i) * 8 + st_row8;
-            const bool ok = (B_BLK % NW == 0 || r < BN) && (n0 + r) < p.N;
-            rb[i] = ok ? *reinterpret_cast<const uint4*>(bptr + (int64_t)(n0 + r) * p.ld_b + k) : make_uint4(0, 0, 0, 0);
+            if (A_IT + i >= first && A_IT + i < last && (B_BLK % NW == 0 || r < BN))
+                *reinterpret_cast<i32x4*>(Bs(stage) + lds_chunk_offset(r, st_c)) = rb[i];
         }
     };
-    auto store_tile = [&](int stage) {
+    constexpr int ST_ALL = A_IT + B_IT;
+    constexpr int HALF = TM > 1 ? TM / 2 : 1;  // m-tiles over which the LDS stores of the next tile are spread
+
+    // Block scales.  Activation scales are [M, K/128] row-major, so the scales of one K step lie
+    // K/128 floats apart: fetched per step and lane they cost as many cache-line requests as the
+    // operand tile itself.  Instead the workgroup fetches the scales of its BM rows for 8 K steps
+    // at a time, 4 consecutive floats per thread (row = t / 2, half = t % 2), and turns them in LDS
+    // to [K step][row], double buffered by group of 8 steps.  The weight scale is one value per
+    // wave and step, fetched one step ahead.
+    float* const sg_buf = reinterpret_cast<float*>(smem + 2 * STAGE);  // [2][8][BM]
+    const int sg_row = t >> 1, sg_half = t & 1;
+    const float* sg_ptr = p.sa;
+    const float* psb = sbp;
+    if (MODE != kRowwise) {
+        const int r = sg_row < BM ? sg_row : BM - 1;
+        sg_ptr = p.sa + (int64_t)((m0 + r) < p.M ? (m0 + r) : (p.M - 1)) * KT;
+        psb += (int64_t)((n0 + wn * WTN) >> 7) * p.sb_stride_n;
+    }
+    f32x4 sg = {0.f, 0.f, 0.f, 0.f};
+    auto sg_load = [&](int g) {  // scales of K steps 8g + 4 half .. + 3 of this thread's row; steps past K/128 repeat valid ones
+        if (MODE == kRowwise) return;
+        const int k0 = 8 * g + 4 * sg_half;
+        if (SCALE_VEC) {
+            sg = *reinterpret_cast<const f32x4*>(sg_ptr + (k0 + 4 <= KT ? k0 : KT - 4));
+        } else {
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) {
-            const int r = (wave + NW * i) * 8 + st_row8;
-            if (A_BLK % NW == 0 || r < BM) *reinterpret_cast<uint4*>(As(stage) + lds_chunk_offset(r, st_c)) = ra[i];
+            for (int e = 0; e < 4; ++e) sg[e] = sg_ptr[(k0 + e) < KT ? (k0 + e) : (KT - 1)];
         }
+    };
+    auto sg_store = [&](int g) {
+        if (MODE == kRowwise) return;
+        if (NT / 2 <= BM || sg_row < BM) {
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i) {
-            const int r = (wave + NW * i) * 8 + st_row8;
-            if (B_BLK % NW == 0 || r < BN) *reinterpret_cast<uint4*>(Bs(stage) + lds_chunk_offset(r, st_c)) = rb[i];
+            for (int e = 0; e < 4; ++e) sg_buf[((g & 1) * 8 + 4 * sg_half + e) * BM + sg_row] = sg[e];
         }
+    };
+    auto load_sn = [&](int kt) -> float {
+        if (MODE == kRowwise) return 0.f;
+        return psb[(int64_t)(kt < KT ? kt : KT - 1) * p.sb_stride_k];
     };
 
     f32x4 acc[TN][TM];
@@ -152,25 +210,32 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // Pipeline over K steps.  At the top of step kt, LDS stage kt & 1 holds tile kt and the
+    // staging registers hold tile kt+1 (loaded in the second half of step kt-1).  Its LDS stores
+    // into the other stage are spread over the first HALF m-tiles of this step; the global loads
+    // of tile kt+2 are issued right after them, so they have the rest of this step and the
+    // barrier to land.  The last step stores a tile that nobody reads.  The activation scales of
+    // the next group of 8 steps are requested in step 8g+6, right after that step's tile loads,
+    // and stored to LDS in step 8g+7.
     load_tile(0);
-    store_tile(0);
+    sg_load(0);
+    float s_n = load_sn(0);
+    __builtin_amdgcn_sched_barrier(0);  // weight scale before tile kt+1, as in the loop: one wait count fits both
+    store_part(0, 0, ST_ALL);
+    sg_store(0);
+    load_tile(1);
     __syncthreads();
 
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1;
-        if (kt + 1 < KT) load_tile(kt + 1);
-
         float s_m[TM];
-        float s_n = 0.f;
+        const float s_n_cur = s_n;
         if (MODE != kRowwise) {
-            const int KB = KT;
+            const float* const sgk = sg_buf + (((kt >> 3) & 1) * 8 + (kt & 7)) * BM + wm * WTM + lrow;
 #pragma unroll
-            for (int j = 0; j < TM; ++j) {
-                const int m = m0 + wm * WTM + j * 16 + lrow;
-                s_m[j] = m < p.M ? p.sa[(int64_t)m * KB + kt] : 0.f;
-            }
-            const int nb = (n0 + wn * WTN) >> 7;
-            s_n = sbp[(int64_t)nb * p.sb_stride_n + (int64_t)kt * p.sb_stride_k];
+            for (int j = 0; j < TM; ++j) s_m[j] = sgk[j * 16];
+            __builtin_amdgcn_sched_barrier(0);
+            s_n = load_sn(kt + 1);
         }
 
         // weight fragments stay live for the whole step; activation fragments are
@@ -179,44 +244,44 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int i = 0; i < TN; ++i) fa[i] = lds_frag(Bs(cur), wn * WTN + i * 16 + lrow, quarter);
         i32x8 fb = lds_frag(As(cur), wm * WTM + lrow, quarter);
-        if (MODE == kRowwise) {
+        // block scaling: the products of m-tile j go to `part`; their scaled accumulation runs
+        // one m-tile later, while the matrix pipe works on the next m-tile
+        f32x4 part[TN];
 #pragma unroll
-            for (int j = 0; j < TM; ++j) {
-                i32x8 fb_next = fb;
-                if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, acc[i][j], 0, 0, 0, 0, 0, 0);
-                fb = fb_next;
-            }
-        } else {
-            // block scaling: the products of m-tile j go to `part`; their scaled accumulation runs
-            // one m-tile later, while the matrix pipe works on the next m-tile
-            f32x4 part[TN];
-#pragma unroll
-            for (int j = 0; j <= TM; ++j) {
-                f32x4 prev[TN];
+        for (int j = 0; j <= TM; ++j) {
+            f32x4 prev[TN];
+            if (MODE != kRowwise) {
 #pragma unroll
                 for (int i = 0; i < TN; ++i) prev[i] = part[i];
-                if (j < TM) {
-                    i32x8 fb_next = fb;
-                    if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
+            }
+            if (j < TM) {
+                i32x8 fb_next = fb;
+                if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
+                if (j < HALF) store_part(cur ^ 1, ST_ALL * j / HALF, ST_ALL * (j + 1) / HALF);
+                if (MODE != kRowwise && j == HALF - 1 && (kt & 7) == 7) sg_store((kt >> 3) + 1);
 #pragma unroll
-                    for (int i = 0; i < TN; ++i)
+                for (int i = 0; i < TN; ++i) {
+                    if (MODE == kRowwise)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, acc[i][j], 0, 0, 0, 0, 0, 0);
+                    else
                         part[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fa[i], fb, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-                    fb = fb_next;
                 }
-                if (j > 0) {
-                    const float sc = s_m[j - 1] * s_n;
-#pragma unroll
-                    for (int i = 0; i < TN; ++i)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(prev[i][e], sc, acc[i][j - 1][e]);
+                if (j == HALF - 1) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_tile(kt + 2);
+                    if (MODE != kRowwise && (kt & 7) == 6) sg_load((kt >> 3) + 1);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+                fb = fb_next;
+            }
+            if (MODE != kRowwise && j > 0) {
+                const float scj = s_m[j - 1] * s_n_cur;
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j - 1][e] = __builtin_fmaf(prev[i][e], scj, acc[i][j - 1][e]);
             }
         }
-
-        if (kt + 1 < KT) store_tile(cur ^ 1);
         __syncthreads();
     }
 
@@ -722,21 +787,24 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
     constexpr int NT = WM * WN * 64;
-    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
-    auto kf = gemm_kernel<BM, BN, WM, WN, MODE, true>;
-    auto kb = gemm_kernel<BM, BN, WM, WN, MODE, false>;
+    // two operand stages, plus the turned activation scales of two groups of 8 K steps
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128 + (MODE == kRowwise ? 0 : 2 * 8 * BM * sizeof(float));
+    // 16-byte scale loads need every row of the scale matrix 16-byte aligned
+    const bool vec = MODE != kRowwise && (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    using Kern = void (*)(const GemmArgs);
+    const Kern table[2][2] = {{gemm_kernel<BM, BN, WM, WN, MODE, false, false>, gemm_kernel<BM, BN, WM, WN, MODE, true, false>},
+                              {gemm_kernel<BM, BN, WM, WN, MODE, false, MODE != kRowwise>, gemm_kernel<BM, BN, WM, WN, MODE, true, MODE != kRowwise>}};
+    const int f32 = out_dtype == CFP8_OUT_F32;
+    const Kern kern = table[vec][f32];
     if (lds > 64 * 1024) {
-        static bool done_f = false, done_b = false;
-        bool& done = out_dtype == CFP8_OUT_F32 ? done_f : done_b;
-        if (!done) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(out_dtype == CFP8_OUT_F32 ? kf : kb),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        static bool done[2][2] = {{false, false}, {false, false}};
+        if (!done[vec][f32]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
-            done = true;
+            done[vec][f32] = true;
         }
     }
-    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(kf, dim3((unsigned)blocks), dim3(NT), lds, st, p);
-    else hipLaunchKernelGGL(kb, dim3((unsigned)blocks), dim3(NT), lds, st, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds, st, p);
     return check_launch("gemm");
 }
 
