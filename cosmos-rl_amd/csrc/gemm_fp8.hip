@@ -818,6 +818,10 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     }
     if (p.M <= 16) return launch_cfg<16, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
+    // block scaling, large M: one 8-wave workgroup per CU on a 256 x 128 tile reads a quarter fewer operand
+    // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
+    if (MODE == kBlock && p.M > 512 && (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128) >= 384)
+        return launch_cfg<256, 128, 4, 2, kBlock>(p, out_dtype, st);
     if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
     if (p.M % 256 == 0 && p.N % 256 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0)
         return launch_rowwise_256(p, out_dtype, st);

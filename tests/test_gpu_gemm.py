@@ -129,8 +129,10 @@ def block_operands(M, N, K, seed):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 128, 256), (70, 208, 384), (128, 256, 1024), (300, 512, 768),
-                                   (640, 1536, 2048)])
+                                   (640, 1536, 2048), (1000, 12288, 384), (1024, 12288, 512)])
 def test_gemm_block128(dev, M, N, K):
+    # the last two shapes have >= 384 tiles of 256 x 128 and take the 8-wave 256 x 128 kernel: one with a
+    # ragged last tile-row and K/128 not a multiple of 4 (scalar scale loads), one with 16-byte scale loads
     qx, sx, qw, sw = block_operands(M, N, K, seed=M * 3 + N + K)
     ref = O.scaled_mm_block128(qx, sx, qw, sw, accum=torch.float64)
     out32 = torch.empty(M, N, dtype=torch.float32, device=dev)
