@@ -239,6 +239,15 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
             lambda: check(lib.cfp8_quant_rowwise(x.data_ptr(), r, c, c, q.data_ptr(), c, s.data_ptr(), stream)))
         del x, q, s
 
+    # quantise-on-receive straight from an fp32 transfer buffer (cast + quantise + store in one kernel)
+    r, c = 37888, 3584
+    x = torch.empty(r, c, dtype=torch.float32, device=dev).normal_(0, 0.02, generator=gen)
+    q = torch.empty(r, c, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty(r, 1, dtype=torch.float32, device=dev)
+    hbm("rowwise_from_f32_gate_up_37888x3584", 5 * r * c + 4 * r,
+        lambda: check(lib.cfp8_quant_rowwise_from(x.data_ptr(), 2, r, c, c, q.data_ptr(), c, s.data_ptr(), stream)))
+    del x, q, s
+
     # config 4: block quantisation of W [7168, 18432] (transposed fp8 out) + block-scaled GEMM
     K4, N4, M4 = 7168, 18432, 4096
     w4 = torch.empty(K4, N4, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)

@@ -83,6 +83,45 @@ def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+_IN_DTYPE = {torch.bfloat16: _lib.IN_BF16, torch.float16: _lib.IN_F16, torch.float32: _lib.IN_F32}
+
+
+def quant_rowwise_into(recv: torch.Tensor, q_out: torch.Tensor, scale_out: torch.Tensor) -> None:
+    """Rowwise quantisation of ``recv.to(bfloat16)`` written straight into caller-owned storage.
+
+    One kernel for what the reference does in three passes when a received shard holds whole rows of
+    a weight: the dtype cast into the bf16 staging view (cosmos_rl/policy/model/base.py:1053-1069),
+    ``fp8_quantization`` (vllm_rollout.py:989-999) and the copies into the engine's weight and
+    ``weight_scale`` parameters (rollout_control.py:889-898).
+
+    recv       [R, C] bf16 / fp16 / fp32, unit stride along C
+    q_out      fp8 storage of the same logical shape, given row-major: either an [R, C] tensor with
+               unit stride along C, or the engine's transposed parameter ``[C, R]`` with strides
+               ``(1, pitch)`` (the ``.t()`` view of a row-major buffer, monkey_patch_for_fp8.py:52)
+    scale_out  fp32 [R, 1] or [R], contiguous
+    """
+    _need_gpu(recv, q_out, scale_out)
+    if recv.dim() != 2 or recv.dtype not in _IN_DTYPE:
+        raise ValueError(f"expected a 2-D bf16/fp16/fp32 tensor, got {tuple(recv.shape)} {recv.dtype}")
+    if q_out.dtype != FP8_DTYPE or scale_out.dtype != torch.float32:
+        raise ValueError("q_out must be float8_e4m3fn and scale_out float32")
+    rows, cols = recv.shape
+    if q_out.dim() == 2 and tuple(q_out.shape) == (rows, cols) and (q_out.stride(1) == 1 or cols == 1):
+        q_rm = q_out
+    elif q_out.dim() == 2 and tuple(q_out.shape) == (cols, rows) and (q_out.stride(0) == 1 or cols == 1):
+        q_rm = q_out.t()
+    else:
+        raise ValueError(f"q_out {tuple(q_out.shape)} strides {q_out.stride()} is not row-major storage for {tuple(recv.shape)}")
+    if scale_out.numel() != rows or not scale_out.is_contiguous():
+        raise ValueError(f"scale_out must hold {rows} contiguous floats, got {tuple(scale_out.shape)}")
+    if recv.stride(1) != 1 and cols > 1:
+        recv = recv.contiguous()
+    ld_x = recv.stride(0) if rows > 1 else max(cols, 1)
+    ld_q = q_rm.stride(0) if rows > 1 else max(cols, 1)
+    _lib.check(_lib.load().cfp8_quant_rowwise_from(recv.data_ptr(), _IN_DTYPE[recv.dtype], rows, cols, ld_x,
+                                                  q_rm.data_ptr(), ld_q, scale_out.data_ptr(), _stream()))
+
+
 def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Tensor], torch.Tensor]:
     """Tensorwise dynamic quantisation of a list of bf16 tensors in two launches per
     batch.  Returns (list of fp8 tensors shaped like the inputs, fp32 scales [n])."""

@@ -85,3 +85,31 @@ class QuantizedWeightReceiver:
             f"scale_tensor.shape: {scale_tensor.shape}, weight_scale.shape: {weight_scale.shape}")
         scale_tensor.copy_(weight_scale)
         return True
+
+    # -- fused form of base.py:1053-1069 + rollout_control.py:856-898 --------------------------
+    def quantize_received_rows(self, full_weight_name: str, recv_tensor: torch.Tensor, row_start: int = 0) -> bool:
+        """Quantise a received shard that holds whole rows ``[row_start, row_start + n)`` of a weight
+        straight into the engine's fp8 parameter and its ``weight_scale``: no cast into the bf16 staging
+        parameter, no temporary fp8 tensor, no strided copies.  Rowwise scales depend on their own row
+        only, so shards that split a weight along dim 0 (column-parallel layers, q/k/v and gate/up
+        splits, unsharded weights) can each be quantised as they land.  Shards that split rows
+        (row-parallel layers) must go through the staging parameter and ``quantize_full_weight``.
+        The first-sync check of the reference compares old and new bytes and therefore needs the
+        unfused path.  Returns False when the name is not a quantised weight."""
+        from cosmos_rl_amd import ops
+
+        if self.quantization_type != "fp8" or full_weight_name not in self.hp_weight_map:
+            return False
+        model_param_map = self.rollout.model_param_map(self.weight_mapper)
+        native = model_param_map[full_weight_name]                       # [in_dim, out_dim], strides (1, in_dim)
+        scale_tensor = model_param_map[full_weight_name.replace(".weight", ".weight_scale")]
+        out_dim, in_dim = self.hp_weight_map[full_weight_name].shape
+        n = recv_tensor.shape[0]
+        if recv_tensor.dim() != 2 or recv_tensor.shape[1] != in_dim or row_start < 0 or row_start + n > out_dim:
+            raise ValueError(
+                f"received rows [{row_start}, {row_start + n}) x {tuple(recv_tensor.shape[1:])} do not fit "
+                f"{full_weight_name} [{out_dim}, {in_dim}]")
+        assert tuple(scale_tensor.shape) == (out_dim, 1), (
+            f"scale_tensor.shape: {scale_tensor.shape}, weight_scale.shape: {(out_dim, 1)}")
+        ops.quant_rowwise_into(recv_tensor, native[:, row_start:row_start + n], scale_tensor[row_start:row_start + n])
+        return True

@@ -59,6 +59,22 @@ const char* cfp8_last_error(void);
 int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
                        void* q, int64_t ld_q, float* scales, void* stream);
 
+/* Source element types of cfp8_quant_rowwise_from. */
+#define CFP8_IN_BF16 0
+#define CFP8_IN_F16 1
+#define CFP8_IN_F32 2
+
+/* Rowwise quantisation straight from a received weight in its transfer dtype:
+ * q, scales = quant_rowwise(x.to(bfloat16)) with x bf16, fp16 or fp32, written
+ * wherever the caller points q (e.g. the engine's own fp8 parameter, ld_q its row
+ * pitch) and scales.  One kernel in place of the three passes
+ *   recv.to(view.dtype); view.copy_(...)        cosmos_rl/policy/model/base.py:1053-1069
+ *   ops.scaled_fp8_quant(weight, ...)           cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:995-997
+ *   param.copy_(quantized); scale.copy_(scale)  cosmos_rl/rollout/worker/rollout_control.py:889-898
+ * for receives that cover whole rows of a weight.  ld_x in elements of x_dtype. */
+int cfp8_quant_rowwise_from(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld_x,
+                            void* q, int64_t ld_q, float* scales, void* stream);
+
 /* Tensorwise dynamic quantisation of many tensors in two passes (grid amax,
  * then cast), without a host round trip in between.
  * Replaces the torchao tensorwise recipe selected at

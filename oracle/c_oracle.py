@@ -37,6 +37,9 @@ def load() -> ctypes.CDLL:
         lib.fp8ref_e4m3_to_f32.restype = c_float
         lib.fp8ref_e4m3_to_f32.argtypes = [c_uint8]
         lib.fp8ref_quant_rowwise.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+        lib.fp8ref_bf16_from_f32.restype = ctypes.c_uint16
+        lib.fp8ref_bf16_from_f32.argtypes = [c_float]
+        lib.fp8ref_quant_rowwise_f32.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_tensorwise.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_block128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_group128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int]
@@ -49,6 +52,20 @@ def load() -> ctypes.CDLL:
 def _u16(x: np.ndarray) -> np.ndarray:
     assert x.dtype == np.uint16
     return np.ascontiguousarray(x)
+
+
+def bf16_from_f32(v: float) -> int:
+    return int(load().fp8ref_bf16_from_f32(v))
+
+
+def quant_rowwise_f32(x_f32: np.ndarray):
+    assert x_f32.dtype == np.float32
+    x = np.ascontiguousarray(x_f32)
+    R, C = x.shape
+    q = np.empty((R, C), np.uint8)
+    s = np.empty((R, 1), np.float32)
+    load().fp8ref_quant_rowwise_f32(x.ctypes.data, R, C, q.ctypes.data, s.ctypes.data)
+    return q, s
 
 
 def quant_rowwise(x_u16: np.ndarray):

@@ -49,6 +49,9 @@ What pins each function (tests/test_oracle.py, tests/test_c_oracle.py):
   quantizers       invariants: every non-zero set holds a +-0x7E byte, error
                    <= half an e4m3 ulp, idempotent re-quantisation, permutation
                    commutation; C restatement agrees byte for byte
+  transfer dtype   quant_rowwise_from: fp32 -> bf16 rounding of oracle/fp8_ref.c (integer RNE)
+                   against torch's own cast on ties, overflow, NaN, subnormals; then
+                   it is quant_rowwise
   block layout     round trip through weight_dequant (the in-tree inverse)
   1x128 layout     round trip through per_token_cast_back (in-tree)
   GEMMs            fp64 matmul of dequantised operands, one-hot operands,
@@ -121,6 +124,15 @@ def quant_rowwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         torch.zeros(x.shape[0], 1)
     scale = scale_from_amax(amax)
     return _cast_with_scale(x, scale), scale
+
+
+def quant_rowwise_from(recv: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Rowwise quantisation of a received weight in its transfer dtype (bf16 / fp16 / fp32):
+    the three steps ``recv.to(view.dtype)`` + ``view.copy_`` (policy/model/base.py:1053-1069, the
+    staging view is bf16, monkey_patch_for_fp8.py:122-125), ``fp8_quantization``
+    (vllm_rollout.py:989-999) and the copies into the engine's parameters
+    (rollout_control.py:889-898) as one function of the received values."""
+    return quant_rowwise(recv.to(torch.bfloat16))
 
 
 def quant_tensorwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -114,6 +114,40 @@ void fp8ref_quant_rowwise(const uint16_t* x, int64_t R, int64_t C, uint8_t* q, f
     }
 }
 
+/* fp32 -> bf16, round to nearest, ties to even, written as a search over the two neighbouring
+ * bf16 values in double arithmetic (not the usual add-0x7FFF bit trick, so that it checks
+ * torch's cast rather than repeating it); overflow rounds to infinity as IEEE 754 prescribes
+ * (infinity stands for 2^128), NaN -> 0x7FC0.  This is `recv.to(torch.bfloat16)` at
+ * cosmos_rl/policy/model/base.py:1068. */
+uint16_t fp8ref_bf16_from_f32(float f) {
+    if (f != f) return 0x7FC0u;
+    const uint32_t u = f32_bits(f);
+    const uint32_t lo = u & 0xFFFF0000u, hi = lo + 0x10000u;  /* hi is the neighbour farther from zero */
+    if ((lo & 0x7F800000u) == 0x7F800000u) return (uint16_t)(lo >> 16);  /* infinity */
+    const double x = fabs((double)f), a = fabs((double)bits_f32(lo));
+    const double b = ((hi & 0x7FFFFFFFu) == 0x7F800000u) ? ldexp(1.0, 128) : fabs((double)bits_f32(hi));
+    const double da = x - a, db = b - x;
+    if (da < db) return (uint16_t)(lo >> 16);
+    if (da > db) return (uint16_t)(hi >> 16);
+    return (uint16_t)(((lo >> 16) & 1u) ? (hi >> 16) : (lo >> 16));
+}
+
+/* rowwise quantisation of fp32 input rounded to bf16 first (quant_rowwise_from in the torch oracle) */
+void fp8ref_quant_rowwise_f32(const float* x, int64_t R, int64_t C, uint8_t* q, float* s) {
+    for (int64_t r = 0; r < R; ++r) {
+        float amax = 0.0f;
+        int nan = 0;
+        for (int64_t c = 0; c < C; ++c) {
+            float v = fabsf(bf16_to_f32(fp8ref_bf16_from_f32(x[r * C + c])));
+            if (v != v) nan = 1;
+            else if (v > amax) amax = v;
+        }
+        float scale = nan ? bits_f32(0x7FC00000u) : scale_from_amax(amax);
+        s[r] = scale;
+        for (int64_t c = 0; c < C; ++c) q[r * C + c] = cast_one(bf16_to_f32(fp8ref_bf16_from_f32(x[r * C + c])), scale);
+    }
+}
+
 void fp8ref_quant_tensorwise(const uint16_t* x, int64_t n, uint8_t* q, float* s) {
     float sc = scale_from_amax(amax_rect(x, n, 1, n));
     s[0] = sc;

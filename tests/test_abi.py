@@ -36,6 +36,7 @@ def test_header_constants_match_binding():
     assert val("CFP8_OUT_BF16") == _lib.OUT_BF16 and val("CFP8_OUT_F32") == _lib.OUT_F32
     assert val("CFP8_GROUP_MODE_DIV") == _lib.GROUP_MODE_DIV and val("CFP8_GROUP_MODE_DEEPEP") == _lib.GROUP_MODE_DEEPEP
     assert val("CFP8_TENSORWISE_AMAX_SLOTS") == _lib.TENSORWISE_AMAX_SLOTS
+    assert (val("CFP8_IN_BF16"), val("CFP8_IN_F16"), val("CFP8_IN_F32")) == (_lib.IN_BF16, _lib.IN_F16, _lib.IN_F32)
     assert ctypes.sizeof(_lib.TensorDesc) == 32
 
 
@@ -44,6 +45,11 @@ def test_argument_errors_need_no_device():
     # null pointers / bad shapes are rejected before any HIP call
     assert lib.cfp8_quant_rowwise(None, 4, 16, 16, None, 16, None, None) == _lib.EINVAL
     assert "null pointer" in _lib.last_error()
+    assert lib.cfp8_quant_rowwise_from(None, _lib.IN_F32, 4, 16, 16, None, 16, None, None) == _lib.EINVAL
+    assert lib.cfp8_quant_rowwise_from(None, 7, 0, 16, 16, None, 16, None, None) == _lib.EINVAL  # unknown dtype
+    assert lib.cfp8_quant_rowwise_from(None, _lib.IN_F16, 0, 16, 16, None, 16, None, None) == 0  # nothing to do
+    assert lib.cfp8_quant_rowwise_from(None, 7, 4, 16, 16, None, 16, None, None) == _lib.EINVAL
+    assert "unknown source dtype" in _lib.last_error()
     assert lib.cfp8_quant_rowwise(None, -1, 16, 16, None, 16, None, None) == _lib.EINVAL
     assert lib.cfp8_quant_block128(None, 1, 128, 128, None, None, 0, None) == _lib.EINVAL
     assert lib.cfp8_quant_group128(None, 4, 128, 128, None, 128, None, 0, None) == _lib.EINVAL

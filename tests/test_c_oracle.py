@@ -55,6 +55,52 @@ def test_rowwise_and_tensorwise_agree():
     assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
 
 
+def _special_f32():
+    """fp32 patterns that exercise the bf16 rounding: ties both ways, carries into the exponent,
+    overflow to infinity, subnormals, signed zeros, infinities, NaNs, plus random bit patterns."""
+    pats = [0x3F800000, 0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001, 0x3FFF8000, 0x7F7F7FFF, 0x7F7F8000,
+            0x7F7FFFFF, 0x7F800000, 0x7FC00000, 0x7F800001, 0x00000000, 0x00000001, 0x00008000, 0x00018000,
+            0x007F8000, 0x007FFFFF, 0x00800000]
+    pats = pats + [p | 0x80000000 for p in pats]
+    g = torch.Generator().manual_seed(7)
+    rnd = torch.randint(-2**31, 2**31 - 1, (200000,), generator=g, dtype=torch.int64).to(torch.int32)
+    return torch.cat([torch.tensor(pats, dtype=torch.int64).to(torch.int32), rnd]).view(torch.float32)
+
+
+def test_bf16_rounding_matches_torch():
+    """The transfer-dtype cast: the C search over the two neighbouring bf16 values agrees with torch's
+    own fp32 -> bf16 conversion on every special pattern and 200k random bit patterns (NaNs compare as NaN)."""
+    lib = C.load()
+    v = _special_f32()
+    want = v.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([lib.fp8ref_bf16_from_f32(float(x)) for x in v.numpy()], dtype=np.uint16)
+    nan = np.isnan(v.numpy())
+    assert (got[~nan] == want[~nan]).all()
+    assert ((got[nan] & 0x7FFF) > 0x7F80).all() and ((want[nan] & 0x7FFF) > 0x7F80).all()
+    # closed forms: a tie goes to the even mantissa, the largest fp32 rounds to infinity
+    assert lib.fp8ref_bf16_from_f32(float(np.uint32(0x3F808000).view(np.float32))) == 0x3F80
+    assert lib.fp8ref_bf16_from_f32(float(np.uint32(0x3F818000).view(np.float32))) == 0x3F82
+    assert lib.fp8ref_bf16_from_f32(float(np.uint32(0x7F7FFFFF).view(np.float32))) == 0x7F80
+
+
+def test_rowwise_from_fp32_agrees():
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(48, 264, generator=g) * torch.exp(torch.randn(48, 1, generator=g) * 4)
+    w[0] = 0
+    w[1, 3] = float("nan")
+    w[2, 5] = float("inf")
+    w[3] = _special_f32()[:264]
+    w[4] = 3.3e38  # rounds to bf16 infinity
+    q, s = C.quant_rowwise_f32(w.numpy())
+    qo, so = O.quant_rowwise_from(w)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()
+    # bf16 input: the transfer-dtype form is the plain rowwise quantiser
+    wb = w.to(torch.bfloat16)
+    qa, sa = O.quant_rowwise_from(wb)
+    qb, sb = O.quant_rowwise(wb)
+    assert torch.equal(qa, qb) and torch.equal(sa.view(torch.int32), sb.view(torch.int32))
+
+
 def test_block_and_group_agree():
     w = _weights((200, 264), 3)
     q, s = C.quant_block128(u16(w))

@@ -100,6 +100,34 @@ def test_weight_sync_end_to_end(dev):
         recv.quantize_full_weight("qkv_proj.weight", do_weight_sync_check=True)
 
 
+def test_fused_receive_quantises_row_shards_in_place(dev):
+    """q/k/v shards arrive in fp32, each holds whole rows of the packed qkv weight: quantise-on-receive writes
+    the engine's fp8 parameter and weight_scale directly; the result equals the unfused path bit for bit."""
+    model = Model(dev)
+    mp.simplify_process_weights_after_loading()
+    for m in model.children():
+        m.quant_method.process_weights_after_loading(m)
+    mapper, rollout = Mapper(), Rollout(model)
+    hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
+    rollout.post_get_params_for_sync_hook("fp8", mapper, dict(rollout.model_param_map(mapper)), quantized)
+    recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
+    g = torch.Generator().manual_seed(11)
+    w32 = torch.randn(4608, 3584, generator=g) * 0.03                       # transfer dtype fp32
+    for a, b in ((0, 3584), (3584, 4096), (4096, 4608)):                    # q, k, v row ranges
+        assert recv.quantize_received_rows("qkv_proj.weight", w32[a:b].to(dev), row_start=a) is True
+    qo, so = O.quant_rowwise_from(w32)
+    assert torch.equal(model.qkv_proj.weight.t().contiguous().view(torch.uint8).cpu(), qo)
+    assert torch.equal(model.qkv_proj.weight_scale.cpu().view(torch.int32), so.view(torch.int32))
+    # same bytes as the reference's three-pass route through the bf16 staging parameter
+    hp["qkv_proj.weight"].data.copy_(w32.to(dev).to(torch.bfloat16))
+    before = model.qkv_proj.weight.t().contiguous().view(torch.uint8).clone()
+    recv.quantize_full_weight("qkv_proj.weight")
+    assert torch.equal(model.qkv_proj.weight.t().contiguous().view(torch.uint8), before)
+    assert recv.quantize_received_rows("not_quantised.weight", w32[:8].to(dev)) is False
+    with pytest.raises(ValueError, match="do not fit"):
+        recv.quantize_received_rows("qkv_proj.weight", w32[:64].to(dev), row_start=4600)
+
+
 def test_fp8_quantization_layout(dev):
     w = O.make_weight((3584, 18944), seed=4).to(dev)
     qt, s = fp8_quantization(w)

@@ -142,6 +142,60 @@ def test_rowwise_properties_full_size(dev):
     assert torch.equal(qp.view(torch.uint8), qb[perm]) and torch.equal(sp, s[perm])
 
 
+def _recv(rows, cols, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g) * 3)
+    if dtype == torch.float16:
+        w = w.clamp(-6e4, 6e4)
+    w = w.to(dtype)
+    if rows > 4:
+        w[0] = 0
+        w[1, 3] = float("nan")
+        w[2, 5] = float("inf")
+        if dtype == torch.float32:
+            w[3, :8] = torch.tensor([0x3F808000, 0x3F818000, 0x7F7FFFFF, 0x00008000, 0x00018000, 0x80008000, 0x3F807FFF,
+                                     0x3FFF8000], dtype=torch.int64).to(torch.int32).view(torch.float32)
+            w[4] = 3.3e38
+        if dtype == torch.float16:
+            w[3, :4] = torch.tensor([0x0001, 0x03FF, 0x8001, 0x7BFF], dtype=torch.int32).to(torch.int16).view(torch.float16)
+    return w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cols", [8, 136, 896, 3584, 4104, 18944, 40000])
+def test_rowwise_from_transfer_dtype(dev, dtype, cols):
+    """cfp8_quant_rowwise_from: quant_rowwise(recv.to(bf16)) for every source dtype and kernel variant,
+    bytes and scales bit-exact, written straight into caller storage."""
+    rows = 21 if cols < 20000 else 5
+    w = _recv(rows, cols, dtype, seed=cols + 1)
+    q = torch.empty(rows, cols, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty(rows, 1, dtype=torch.float32, device=dev)
+    ops.quant_rowwise_into(w.to(dev), q, s)
+    qo, so = O.quant_rowwise_from(w)
+    assert_scales(s, so, f"{dtype} cols={cols} scales")
+    assert_bytes(q, qo, f"{dtype} cols={cols} bytes")
+
+
+def test_rowwise_from_into_engine_parameter(dev):
+    """Destination = a row range of the engine's transposed fp8 parameter (strides (1, in_dim)) and of its
+    [out, 1] scale parameter; rows outside the range stay untouched."""
+    out_dim, in_dim, a, b = 96, 264, 16, 80
+    w = _recv(b - a, in_dim, torch.float32, seed=3)
+    buf = torch.full((out_dim, in_dim), 0x55, dtype=torch.uint8, device=dev)
+    param = buf.view(torch.float8_e4m3fn).t()                  # [in_dim, out_dim], strides (1, in_dim)
+    scale = torch.full((out_dim, 1), -1.0, dtype=torch.float32, device=dev)
+    ops.quant_rowwise_into(w.to(dev), param[:, a:b], scale[a:b])
+    qo, so = O.quant_rowwise_from(w)
+    assert_bytes(buf[a:b], qo, "rows in range")
+    assert_scales(scale[a:b], so, "scales in range")
+    assert (buf[:a] == 0x55).all() and (buf[b:] == 0x55).all()
+    assert (scale[:a] == -1).all() and (scale[b:] == -1).all()
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_into(w.to(dev), param[:, a:b + 1], scale[a:b])
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_into(w.to(dev).to(torch.float64), param[:, a:b], scale[a:b])
+
+
 # ---------------------------------------------------------------------------- tensorwise
 def test_tensorwise_multi(dev):
     """A Qwen2.5-7B-shaped layer set at reduced width plus ragged extras, in one call."""
