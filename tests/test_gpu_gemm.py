@@ -185,10 +185,11 @@ def test_gemm_block128_cfg4_properties(dev):
 
 
 # ---------------------------------------------------------------------------- grouped
-def test_grouped_gemm(dev):
-    """Ragged groups: top-2 routing of 300 tokens over 6 experts plus an empty expert, groups
-    padded to 128 rows; padding rows (index -1) must be left untouched."""
-    T, E, K, N, topk = 300, 7, 512, 384, 2
+@pytest.mark.parametrize("T,E,K,N,topk", [(300, 7, 512, 384, 2), (2600, 7, 384, 2048, 2)])
+def test_grouped_gemm(dev, T, E, K, N, topk):
+    """Ragged groups: top-2 routing over 6 experts plus an empty expert, groups padded to 128 rows;
+    padding rows (index -1) must be left untouched.  The second shape has >= 384 tiles of 128 x 256
+    (the 8-wave grouped kernel) and K/128 not a multiple of 4."""
     g = torch.Generator().manual_seed(77)
     logits = torch.rand(T, E, generator=g)
     logits[:, 3] = -1.0  # expert 3 gets no token
