@@ -39,7 +39,8 @@ def rowwise_operands(M, N, K, seed, dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 64, 256), (17, 80, 384), (64, 128, 512), (100, 272, 896),
-                                   (128, 128, 128), (300, 1024, 1024), (513, 528, 640), (1024, 768, 3584),
+                                   (128, 128, 128), (200, 272, 384), (256, 512, 256), (300, 1024, 1024), (513, 528, 640),
+                                   (1024, 768, 3584),
                                    # full 256x256 tiles: the four-wave pipelined kernel, K of 1, 3 and 28 steps
                                    (768, 256, 128), (1024, 512, 384), (2048, 1280, 896)])
 def test_scaled_mm_rowwise(dev, M, N, K):
