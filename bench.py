@@ -52,8 +52,9 @@ def main() -> int:
                     help="also run three plain 1 GiB device copies, to calibrate HBM traffic counters under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path has no cross-GPU step on a single "
-              "MI355X; see DESIGN.md for how it shards). Run with --gpus 1.", file=sys.stderr)
+        print("bench.py: this build measures one GPU only: quantisation shards by rows with no exchange, the "
+              "tensorwise recipe needs one all-reduce(max) between its two passes, and that step is not built. "
+              "Run with --gpus 1.", file=sys.stderr)
         return 2
 
     import torch
@@ -211,21 +212,21 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=dev)
     out = {}
 
-    def hbm(name, bytes_, fn, iters=20):
+    def hbm(name, bytes_, fn, iters=50):
         if only and only not in name:
             return
-        med, mn = _time_events(torch, fn, 3, iters, flush)
-        out[name] = {"ms": round(med, 4), "GB/s": round(bytes_ / (med * 1e-3) / 1e9, 1),
+        med, mn = _time_events(torch, fn, 10, iters, flush)
+        out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "GB/s": round(bytes_ / (med * 1e-3) / 1e9, 1),
                      "frac_hbm": round(bytes_ / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
-    def mfma(name, flops, bytes_, fn, iters=20):
+    def mfma(name, flops, bytes_, fn, iters=50):
         if only and only not in name:
             return
-        med, mn = _time_events(torch, fn, 3, iters, flush)
+        med, mn = _time_events(torch, fn, 10, iters, flush)
         tf = flops / (med * 1e-3) / 1e12
         gbs = bytes_ / (med * 1e-3) / 1e9
         bound = "mfma" if flops / bytes_ > FP8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9) else "hbm"
-        out[name] = {"ms": round(med, 4), "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
+        out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
                      "frac": round(tf / FP8_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS, 4)}
 
     # rowwise weight quantisation at the shapes of one weight sync (vLLM packed layers)
@@ -258,6 +259,9 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     q4n = torch.empty(K4, N4, dtype=torch.float8_e4m3fn, device=dev)
     hbm("block128_cfg4_7168x18432", 3 * K4 * N4 + 4 * s4.numel(),
         lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4n.data_ptr(), s4.data_ptr(), 0, stream)))
+    # the inverse: block dequantisation of the same matrix to bf16 (1 B read, 2 B written per element)
+    hbm("dequant_block128_cfg4_7168x18432_bf16", 3 * K4 * N4 + 4 * s4.numel(),
+        lambda: check(lib.cfp8_dequant_block128(q4n.data_ptr(), s4.data_ptr(), K4, N4, w4.data_ptr(), 0, stream)))
     del q4n, w4
     x4 = torch.randn(M4, K4, generator=gen, device=dev).to(torch.bfloat16)
     qx4 = torch.empty(M4, K4, dtype=torch.float8_e4m3fn, device=dev)
@@ -270,7 +274,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         check(lib.cfp8_quant_group128(x4.data_ptr(), M4, K4, K4, qx4.data_ptr(), K4, sx4.data_ptr(), 0, stream))
         check(lib.cfp8_gemm_block128(qx4.data_ptr(), K4, sx4.data_ptr(), q4.data_ptr(), K4, s4.data_ptr(), 1, N4 // 128,
                                      o4.data_ptr(), N4, 0, M4, N4, K4, stream))
-    mfma("gemm_block128_cfg4_4096x18432x7168_incl_act_quant", 2.0 * M4 * N4 * K4, N4 * K4 + M4 * K4 * 2 + M4 * N4 * 2, gemm4, iters=10)
+    mfma("gemm_block128_cfg4_4096x18432x7168_incl_act_quant", 2.0 * M4 * N4 * K4, N4 * K4 + M4 * K4 * 2 + M4 * N4 * 2, gemm4, iters=50)
     del x4, qx4, sx4, o4, q4, s4
 
     # config 3: FP8 linear [M, 3584] x [18944, 3584]^T, per-token activation quant inside the call
@@ -287,7 +291,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
         mfma(f"linear_rowwise_cfg3_M{M}", 2.0 * M * N3 * K3, N3 * K3 + 4 * N3 + M * K3 * 2 + M * N3 * 2,
              lambda: check(lib.cfp8_linear_rowwise(x.data_ptr(), K3, qw3.data_ptr(), K3, sw3.data_ptr(), o.data_ptr(), N3, 0,
-                                                   M, N3, K3, ws.data_ptr(), wsb, stream)), iters=20 if M < 8192 else 10)
+                                                   M, N3, K3, ws.data_ptr(), wsb, stream)), iters=50)
         del x, o, ws
     del qw3, sw3
 
@@ -303,7 +307,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     def quant5():
         check(lib.cfp8_quant_block128(wgu.data_ptr(), E, 2 * I, H, qgu.data_ptr(), sgu.data_ptr(), 0, stream))
         check(lib.cfp8_quant_block128(wd.data_ptr(), E, H, I, qd.data_ptr(), sd.data_ptr(), 0, stream))
-    hbm("block128_cfg5_experts", 3 * (wgu.numel() + wd.numel()) + 4 * (sgu.numel() + sd.numel()), quant5, iters=10)
+    hbm("block128_cfg5_experts", 3 * (wgu.numel() + wd.numel()) + 4 * (sgu.numel() + sd.numel()), quant5, iters=50)
     del wgu, wd
     logits = torch.rand(T, E, generator=gen, device=dev)
     topi = torch.topk(logits, TOPK, dim=1).indices.reshape(-1)
@@ -334,7 +338,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
                                              dn.data_ptr(), H, 0, total, H, I, E, stream))
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
     mfma("grouped_cfg5_gate_up_down_incl_act_quant", flops5,
-         qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=10)
+         qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=50)
     if "grouped_cfg5_gate_up_down_incl_act_quant" in out:
         out["grouped_cfg5_gate_up_down_incl_act_quant"]["routed_rows"] = routed
         out["grouped_cfg5_gate_up_down_incl_act_quant"]["padded_rows"] = total
