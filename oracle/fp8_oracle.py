@@ -276,6 +276,13 @@ def grouped_mm_block128(qa: torch.Tensor, sa: torch.Tensor,
     return out
 
 
+def calc_diff(x: torch.Tensor, y: torch.Tensor) -> float:
+    """The similarity metric of the reference's own FP8 tests (tests/test_deepep.py:62-67):
+    1 - 2<x+1, y+1> / (|x+1|^2 + |y+1|^2) in fp64."""
+    x, y = x.double() + 1, y.double() + 1
+    return float(1 - 2 * (x * y).sum() / (x * x + y * y).sum())
+
+
 def rel_frobenius(got: torch.Tensor, want: torch.Tensor) -> float:
     g, w = got.double(), want.double()
     denom = w.norm().item()

@@ -140,6 +140,7 @@ def test_gemm_block128(dev, M, N, K):
     ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out32)
     err = O.rel_frobenius(out32.cpu(), ref)
     assert err <= TIGHT, f"block fp32 {err:.3e}"
+    assert O.calc_diff(out32.cpu(), ref) < 1e-8  # the reference's own metric (tests/test_deepep.py:62-67)
     out16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out16)
     check_bf16(out16, ref, f"block {M}x{N}x{K}")

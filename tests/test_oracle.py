@@ -266,3 +266,13 @@ def test_routing_helper():
 def test_qwen_shapes_total():
     assert O.qwen25_7b_numel() == 7_070_285_824
     assert sum(n for _, _, n in O.QWEN25_7B_LINEAR_SHAPES) == 197
+
+
+def test_calc_diff_closed_forms():
+    """tests/test_deepep.py:62-67: zero for identical tensors, symmetric, and 1 - 2ab/(a^2+b^2) for constants."""
+    x = torch.tensor([0.5, -2.0, 3.0])
+    assert O.calc_diff(x, x) == 0.0
+    y = torch.tensor([0.25, -1.0, 2.0])
+    assert O.calc_diff(x, y) == O.calc_diff(y, x)
+    a, b = torch.full((4,), 1.0), torch.full((4,), 3.0)     # shifted to 2 and 4
+    assert abs(O.calc_diff(a, b) - (1 - 2 * 2 * 4 / (4 + 16))) < 1e-15
