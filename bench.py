@@ -323,8 +323,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     xs = torch.randn(total, H, generator=gen, device=dev).to(torch.bfloat16)
     qxs = torch.empty(total, H, dtype=torch.float8_e4m3fn, device=dev)
     sxs = torch.empty(total, H // 128, dtype=torch.float32, device=dev)
-    gu = torch.empty(total, 2 * I, dtype=torch.bfloat16, device=dev)
-    hdn = torch.randn(total, I, generator=gen, device=dev).to(torch.bfloat16)
+    gu = torch.zeros(total, 2 * I, dtype=torch.bfloat16, device=dev)  # padding rows are never written by the GEMM
     qh = torch.empty(total, I, dtype=torch.float8_e4m3fn, device=dev)
     sh = torch.empty(total, I // 128, dtype=torch.float32, device=dev)
     dn = torch.empty(total, H, dtype=torch.bfloat16, device=dev)
@@ -333,15 +332,21 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         check(lib.cfp8_quant_group128(xs.data_ptr(), total, H, H, qxs.data_ptr(), H, sxs.data_ptr(), 0, stream))
         check(lib.cfp8_gemm_grouped_block128(qxs.data_ptr(), H, sxs.data_ptr(), qgu.data_ptr(), sgu.data_ptr(), m_idx.data_ptr(),
                                              gu.data_ptr(), 2 * I, 0, total, 2 * I, H, E, stream))
-        check(lib.cfp8_quant_group128(hdn.data_ptr(), total, I, I, qh.data_ptr(), I, sh.data_ptr(), 0, stream))
+        check(lib.cfp8_swiglu_quant_group128(gu.data_ptr(), 2 * I, gu.data_ptr() + I * 2, 2 * I, total, I,
+                                             qh.data_ptr(), I, sh.data_ptr(), stream))
         check(lib.cfp8_gemm_grouped_block128(qh.data_ptr(), I, sh.data_ptr(), qd.data_ptr(), sd.data_ptr(), m_idx.data_ptr(),
                                              dn.data_ptr(), H, 0, total, H, I, E, stream))
+    # SwiGLU + 1x128 requantisation between the two GEMMs, alone: 2 x 2 B read + 1 B written per element
+    moe()
+    hbm("swiglu_quant_cfg5_%dx%d" % (total, I), 5 * total * I + 4 * sh.numel(),
+        lambda: check(lib.cfp8_swiglu_quant_group128(gu.data_ptr(), 2 * I, gu.data_ptr() + I * 2, 2 * I, total, I,
+                                                     qh.data_ptr(), I, sh.data_ptr(), stream)))
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
-    mfma("grouped_cfg5_gate_up_down_incl_act_quant", flops5,
+    mfma("grouped_cfg5_mlp_quant_gateup_swiglu_down", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=50)
-    if "grouped_cfg5_gate_up_down_incl_act_quant" in out:
-        out["grouped_cfg5_gate_up_down_incl_act_quant"]["routed_rows"] = routed
-        out["grouped_cfg5_gate_up_down_incl_act_quant"]["padded_rows"] = total
+    if "grouped_cfg5_mlp_quant_gateup_swiglu_down" in out:
+        out["grouped_cfg5_mlp_quant_gateup_swiglu_down"]["routed_rows"] = routed
+        out["grouped_cfg5_mlp_quant_gateup_swiglu_down"]["padded_rows"] = total
     return out
 
 

@@ -212,6 +212,28 @@ def prepare_fp8_input(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return _group128(x, _lib.GROUP_MODE_DIV)
 
 
+def swiglu_quant(gate: torch.Tensor, up: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``silu(gate) * up`` and the 1x128 quantisation of the product in one kernel; the bf16 product is
+    never written.  Takes the two expert-GEMM outputs of cosmos_rl/policy/kernel/group_gemms.py:194-207
+    (or the two column halves of one fused gate_up output: any row pitch, unit column stride) and returns
+    what ``groupwise_activation_quant(activation(gate) * up)`` returns at :209-218: (fp8 [M, I], fp32 [M, I/128])."""
+    _need_gpu(gate, up)
+    if gate.dtype != torch.bfloat16 or up.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape != up.shape:
+        raise ValueError(f"expected two bf16 [M, I] tensors, got {tuple(gate.shape)} {gate.dtype} and {tuple(up.shape)} {up.dtype}")
+    rows, cols = gate.shape
+    if cols > 1 and gate.stride(1) != 1:
+        gate = gate.contiguous()
+    if cols > 1 and up.stride(1) != 1:
+        up = up.contiguous()
+    q = torch.empty((rows, cols), dtype=FP8_DTYPE, device=gate.device)
+    s = torch.empty((rows, (cols + 127) // 128), dtype=torch.float32, device=gate.device)
+    ldg = gate.stride(0) if rows > 1 else max(cols, 1)
+    ldu = up.stride(0) if rows > 1 else max(cols, 1)
+    _lib.check(_lib.load().cfp8_swiglu_quant_group128(gate.data_ptr(), ldg, up.data_ptr(), ldu, rows, cols,
+                                                     q.data_ptr(), cols, s.data_ptr(), _stream()))
+    return q, s
+
+
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """``per_token_cast_to_fp8`` of the reference's tests/test_deepep.py:75-85, including its
     formula ``x * (448 / amax.clamp(1e-4))`` with scales ``amax / 448``."""

@@ -65,11 +65,21 @@ class TorchBF16GroupGEMM(GroupGEMMStrategy):
 class DSGroupGEMM(GroupGEMMStrategy):
     """FP8 grouped GEMM: block-quantised expert weights, 1x128 activation groups."""
 
-    def __init__(self, custom_activation, use_triton_quant=True):
+    def __init__(self, custom_activation, use_triton_quant=True, fuse_swiglu=True, fuse_gate_up=False):
         # ``use_triton_quant`` selected between two third-party quantisers in the reference
         # (group_gemms.py:188-191); both map to the one HIP group quantiser here.
+        # fuse_swiglu: when the activation is SiLU, ``act(gate) * up`` and the 1x128 quantisation of the
+        # product (group_gemms.py:209-218) run as one kernel and the bf16 product is never written.
+        # fuse_gate_up: the gate and up projections (two GEMMs on the same input, :194-207) run as one
+        # GEMM over the concatenated weights; costs a second copy of those weights.
         self.activation_function = custom_activation
         self.use_triton_quant = use_triton_quant
+        self.fuse_swiglu = fuse_swiglu and self._is_silu(custom_activation)
+        self.fuse_gate_up = fuse_gate_up
+
+    @staticmethod
+    def _is_silu(fn) -> bool:
+        return isinstance(fn, nn.SiLU) or fn is torch.nn.functional.silu
 
     def arrange_expert_weights(self, all_weights, submod_name, module):
         combined_weights = torch.stack(all_weights)
@@ -94,16 +104,29 @@ class DSGroupGEMM(GroupGEMMStrategy):
         hidden_size = module.get_parameter("down_proj_weight").shape[1]
         dev, dt = contig_tokens.device, contig_tokens.dtype
 
-        gate_out = torch.empty((total, intermediate_size), device=dev, dtype=dt)
-        up_out = torch.empty_like(gate_out)
         down_out = torch.empty((total, hidden_size), device=dev, dtype=dt)
-
         gate_up_input = self._quant(valid_tokens)
-        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (gate_fp8, gate_s), gate_out, m_indices)
-        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (up_fp8, up_s), up_out, m_indices)
-        hidden_states = self.activation_function(gate_out) * up_out
-        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(self._quant(hidden_states), (down_fp8, down_s), down_out,
-                                                      m_indices)
+        # padding rows (m_indices < 0) are not written by the GEMMs: start from zeros so that what the
+        # activation reads there is defined
+        if self.fuse_gate_up and intermediate_size % 128 == 0:
+            fused = getattr(module, "_gate_up_fp8_fused", None)
+            if fused is None or fused[2] != (gate_fp8.data_ptr(), up_fp8.data_ptr()):
+                fused = (torch.cat([gate_fp8, up_fp8], dim=1), torch.cat([gate_s, up_s], dim=1),
+                         (gate_fp8.data_ptr(), up_fp8.data_ptr()))
+                module._gate_up_fp8_fused = fused
+            gate_up_out = torch.zeros((total, 2 * intermediate_size), device=dev, dtype=dt)
+            ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (fused[0], fused[1]), gate_up_out, m_indices)
+            gate_out, up_out = gate_up_out[:, :intermediate_size], gate_up_out[:, intermediate_size:]
+        else:
+            gate_out = torch.zeros((total, intermediate_size), device=dev, dtype=dt)
+            up_out = torch.zeros_like(gate_out)
+            ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (gate_fp8, gate_s), gate_out, m_indices)
+            ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (up_fp8, up_s), up_out, m_indices)
+        if self.fuse_swiglu:
+            hidden_quantized = ops.swiglu_quant(gate_out, up_out)
+        else:
+            hidden_quantized = self._quant(self.activation_function(gate_out) * up_out)
+        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(hidden_quantized, (down_fp8, down_s), down_out, m_indices)
         contig_tokens[:total] = down_out
         return contig_tokens
 

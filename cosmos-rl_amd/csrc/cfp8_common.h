@@ -191,4 +191,32 @@ __device__ __forceinline__ u32 pack_bf16x2(float a, float b) {
     return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2_t));
 }
 
+// exp(t) as a fixed sequence of IEEE fp32 operations (range reduction by ln2 in two parts, Taylor
+// polynomial of degree 7 in Horner form with fused multiply-adds, exact scaling): every step is
+// correctly rounded, so a CPU that runs the same sequence gets the same bits.  |error| < 2 ulp.
+// t is clamped to [-104, 89]: below, the result is far under 2^-126 * 2^-24 and 1 + exp(t) == 1
+// anyway; above, it overflows to infinity.  NaN is the caller's business.
+__device__ __forceinline__ float exp32_det(float t) {
+    t = t > 89.0f ? 89.0f : t;
+    t = t < -104.0f ? -104.0f : t;
+    const float n = __builtin_rintf(t * 1.44269502162933349609375f);
+    float r = __builtin_fmaf(n, -0.693145751953125f, t);
+    r = __builtin_fmaf(n, -1.428606765330187045037746429443359375e-06f, r);
+    float p = 1.98412701138295233249664306640625e-04f;               // 1/5040
+    p = __builtin_fmaf(p, r, 1.388888922519981861114501953125e-03f);  // 1/720
+    p = __builtin_fmaf(p, r, 8.3333337679505348205566406250e-03f);    // 1/120
+    p = __builtin_fmaf(p, r, 4.16666679084300994873046875e-02f);      // 1/24
+    p = __builtin_fmaf(p, r, 0.16666667163372039794921875f);          // 1/6
+    p = __builtin_fmaf(p, r, 0.5f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    return __builtin_ldexpf(p, (int)n);
+}
+
+// SiLU of a bf16 value in fp32: x / (1 + exp(-x)), IEEE division; NaN stays NaN
+__device__ __forceinline__ float silu32_det(float x) {
+    if (x != x) return x;
+    return x / (1.0f + exp32_det(-x));
+}
+
 }  // namespace cfp8

@@ -175,6 +175,48 @@ __global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __
     }
 }
 
+// SwiGLU fused with the 1x128 quantiser: h = bf16(bf16(silu(g)) * u) is formed in registers from the
+// two bf16 GEMM outputs and quantised like group128_kernel<DIV> does; h never exists in memory.
+// The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors.
+__device__ __forceinline__ u32 swiglu_pair(u32 g, u32 u) {
+    const float s0 = silu32_det(bf16_lo(g)), s1 = silu32_det(bf16_hi(g));
+    const u32 s = pack_bf16x2(s0, s1);
+    return pack_bf16x2(bf16_lo(s) * bf16_lo(u), bf16_hi(s) * bf16_hi(u));
+}
+
+__global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __restrict__ gate, int64_t ldg,
+                                                              const uint4* __restrict__ up, int64_t ldu, int nvec,
+                                                              int ngroups, uint2* __restrict__ q, int64_t ldq,
+                                                              float* __restrict__ scales, int64_t total_groups) {
+    const int sub = threadIdx.x & 15;
+    const int64_t g0 = ((int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)) * 2;
+    uint4 vg[2], vu[2];
+    int64_t row[2];
+    int gcol[2];
+    bool ok[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int64_t g = g0 + i;
+        row[i] = g / ngroups;
+        gcol[i] = (int)(g - row[i] * ngroups);
+        const int vec = gcol[i] * 16 + sub;
+        ok[i] = g < total_groups && vec < nvec;
+        vg[i] = ok[i] ? ld16<true>(gate + row[i] * ldg + vec) : make_uint4(0, 0, 0, 0);
+        vu[i] = ok[i] ? ld16<true>(up + row[i] * ldu + vec) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint4 h = make_uint4(swiglu_pair(vg[i].x, vu[i].x), swiglu_pair(vg[i].y, vu[i].y),
+                                   swiglu_pair(vg[i].z, vu[i].z), swiglu_pair(vg[i].w, vu[i].w));
+        const u32 m = row16_max(pk_fold(absmax8(0u, h)));
+        const float scale = scale_from_amax(amax_from_bits(m));
+        const Divider d(scale);
+        const uint2 out = cast8(h, d);
+        if (ok[i]) st8<false>(q + row[i] * ldq + gcol[i] * 16 + sub, out);
+        if (sub == 0 && g0 + i < total_groups) scales[row[i] * ngroups + gcol[i]] = scale;
+    }
+}
+
 int launch_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
                           float* scales, int mode, hipStream_t st) {
     const int64_t ngroups = (cols + 127) / 128;
@@ -231,6 +273,26 @@ extern "C" int cfp8_quant_group128(const void* x, int64_t rows, int64_t cols, in
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "quant_group128: misaligned pointer");
     if (int rc = check_device()) return rc;
     return launch_quant_group128(x, rows, cols, ld_x, q, ld_q, scales, mode, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t rows,
+                                          int64_t cols, void* q, int64_t ld_q, float* scales, void* stream) {
+    using namespace cfp8;
+    if (rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "swiglu_quant_group128: negative shape");
+    if (rows == 0 || cols == 0) return CFP8_OK;
+    if (!gate || !up || !q || !scales) return set_error(CFP8_EINVAL, "swiglu_quant_group128: null pointer");
+    if (cols % 8 || ld_gate % 8 || ld_up % 8 || ld_q % 8 || ld_gate < cols || ld_up < cols || ld_q < cols)
+        return set_error(CFP8_EINVAL, "swiglu_quant_group128: cols=%lld ld_gate=%lld ld_up=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
+                         (long long)cols, (long long)ld_gate, (long long)ld_up, (long long)ld_q);
+    if (!aligned16(gate) || !aligned16(up) || (reinterpret_cast<uintptr_t>(q) & 7u))
+        return set_error(CFP8_EINVAL, "swiglu_quant_group128: misaligned pointer");
+    const int64_t ngroups = (cols + 127) / 128, total = rows * ngroups, blocks = (total + 31) / 32;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "swiglu_quant_group128: too many groups for one launch");
+    if (int rc = check_device()) return rc;
+    hipLaunchKernelGGL(swiglu_group128_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(gate), ld_gate / 8, static_cast<const uint4*>(up), ld_up / 8, (int)(cols / 8),
+                       (int)ngroups, static_cast<uint2*>(q), ld_q / 8, scales, total);
+    return check_launch("swiglu_quant_group128");
 }
 
 extern "C" int cfp8_dequant_block128(const void* q, const float* scales, int64_t rows, int64_t cols, void* y,

@@ -130,6 +130,20 @@ int cfp8_quant_block128(const void* x, int64_t batch, int64_t rows, int64_t cols
 int cfp8_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
                         void* q, int64_t ld_q, float* scales, int mode, void* stream);
 
+/* SwiGLU between the expert GEMMs fused with the 1x128 quantisation of its result:
+ *   h = bf16(bf16(silu(gate)) * up),  q, scales = quant_group128(h, CFP8_GROUP_MODE_DIV)
+ * gate, up bf16 [rows, cols] (two GEMM outputs, or the two halves of one fused
+ * gate_up output: up = gate + cols, ld_gate = ld_up = 2 * cols); h is never
+ * written.  Replaces `self.activation_function(gate_proj_out) * up_proj_out`
+ * followed by `groupwise_activation_quant` / `prepare_fp8_input` at
+ * cosmos_rl/policy/kernel/group_gemms.py:209-218 for the SiLU activation.
+ * silu(x) = x / (1 + exp(-x)) in fp32; exp is a fixed sequence of correctly
+ * rounded fp32 operations (two-part ln2 reduction, degree-7 Horner polynomial with
+ * fused multiply-adds, ldexp), so the result is the same bits on any IEEE machine. */
+int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                               int64_t rows, int64_t cols, void* q, int64_t ld_q, float* scales,
+                               void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */

@@ -40,6 +40,11 @@ def load() -> ctypes.CDLL:
         lib.fp8ref_bf16_from_f32.restype = ctypes.c_uint16
         lib.fp8ref_bf16_from_f32.argtypes = [c_float]
         lib.fp8ref_quant_rowwise_f32.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+        lib.fp8ref_exp32.restype = c_float
+        lib.fp8ref_exp32.argtypes = [c_float]
+        lib.fp8ref_silu32.restype = c_float
+        lib.fp8ref_silu32.argtypes = [c_float]
+        lib.fp8ref_swiglu.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
         lib.fp8ref_quant_tensorwise.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_block128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_group128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int]
@@ -66,6 +71,19 @@ def quant_rowwise_f32(x_f32: np.ndarray):
     s = np.empty((R, 1), np.float32)
     load().fp8ref_quant_rowwise_f32(x.ctypes.data, R, C, q.ctypes.data, s.ctypes.data)
     return q, s
+
+
+def swiglu(g_u16: np.ndarray, u_u16: np.ndarray) -> np.ndarray:
+    """bf16(bf16(silu(g)) * u) on uint16 views of bf16 arrays of equal shape."""
+    g, u = _u16(g_u16), _u16(u_u16)
+    assert g.shape == u.shape
+    h = np.empty(g.shape, np.uint16)
+    load().fp8ref_swiglu(g.ctypes.data, u.ctypes.data, g.size, h.ctypes.data)
+    return h
+
+
+def swiglu_quant_group128(g_u16: np.ndarray, u_u16: np.ndarray):
+    return quant_group128(swiglu(g_u16, u_u16), mode=0)
 
 
 def quant_rowwise(x_u16: np.ndarray):

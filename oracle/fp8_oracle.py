@@ -52,6 +52,9 @@ What pins each function (tests/test_oracle.py, tests/test_c_oracle.py):
   transfer dtype   quant_rowwise_from: fp32 -> bf16 rounding of oracle/fp8_ref.c (integer RNE)
                    against torch's own cast on ties, overflow, NaN, subnormals; then
                    it is quant_rowwise
+  SwiGLU + requant exp32 of oracle/fp8_ref.c against fp64 exp (< 2 ulp on a dense grid), closed
+                   forms silu(0) = 0, silu(x) -> x and -> -0 at the ends, hidden state within one
+                   bf16 ulp of torch's silu(g) * u on <= 0.1 % of elements and equal elsewhere
   block layout     round trip through weight_dequant (the in-tree inverse)
   1x128 layout     round trip through per_token_cast_back (in-tree)
   GEMMs            fp64 matmul of dequantised operands, one-hot operands,
@@ -180,6 +183,22 @@ def quant_group128(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     scale = scale_from_amax(g.abs().amax(dim=2))               # [M, kb]
     y = torch.clamp(g / scale[:, :, None], -E4M3_MAX, E4M3_MAX).reshape(M, kb * BLOCK)
     return e4m3_bytes(y[:, :K].contiguous()), scale
+
+
+def swiglu_quant_group128(gate: torch.Tensor, up: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``hidden = activation(gate_out) * up_out`` on bf16 tensors followed by the 1x128 quantiser
+    (cosmos_rl/policy/kernel/group_gemms.py:209-218) for the SiLU activation, with torch's own ops.
+
+    The fused kernel and oracle/fp8_ref.c define exp by a fixed fp32 operation sequence; torch's
+    vectorised exp may differ from it in the last fp32 bit, which moves the bf16 rounding of
+    silu(g) for about one element in 10^4.  Tests therefore hold the kernel bit-exact against the
+    C restatement and within one bf16 ulp of the hidden state (rare) against this function."""
+    h = torch.nn.functional.silu(gate.to(torch.bfloat16)) * up.to(torch.bfloat16)
+    return quant_group128(h)
+
+
+def swiglu_hidden(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    return torch.nn.functional.silu(gate.to(torch.bfloat16)) * up.to(torch.bfloat16)
 
 
 def group128_cast_deepep(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -201,6 +201,40 @@ void fp8ref_quant_group128(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, 
         }
 }
 
+/* exp(t) as the fixed fp32 sequence the SwiGLU kernel uses: two-part ln2 reduction, Taylor
+ * degree 7 in Horner form with fmaf, ldexpf.  Built with -ffp-contract=off, so every operation
+ * below is exactly the one written. */
+float fp8ref_exp32(float t) {
+    t = t > 89.0f ? 89.0f : t;
+    t = t < -104.0f ? -104.0f : t;
+    const float n = rintf(t * 1.44269502162933349609375f);
+    float r = fmaf(n, -0.693145751953125f, t);
+    r = fmaf(n, -1.428606765330187045037746429443359375e-06f, r);
+    float p = 1.98412701138295233249664306640625e-04f;
+    p = fmaf(p, r, 1.388888922519981861114501953125e-03f);
+    p = fmaf(p, r, 8.3333337679505348205566406250e-03f);
+    p = fmaf(p, r, 4.16666679084300994873046875e-02f);
+    p = fmaf(p, r, 0.16666667163372039794921875f);
+    p = fmaf(p, r, 0.5f);
+    p = fmaf(p, r, 1.0f);
+    p = fmaf(p, r, 1.0f);
+    return ldexpf(p, (int)n);
+}
+
+float fp8ref_silu32(float x) {
+    if (x != x) return x;
+    return x / (1.0f + fp8ref_exp32(-x));
+}
+
+/* h = bf16(bf16(silu(g)) * u): `self.activation_function(gate_proj_out) * up_proj_out` on bf16
+ * tensors, cosmos_rl/policy/kernel/group_gemms.py:210 (SiLU), then the 1x128 quantiser of :213-218 */
+void fp8ref_swiglu(const uint16_t* g, const uint16_t* u, int64_t n, uint16_t* h) {
+    for (int64_t i = 0; i < n; ++i) {
+        const uint16_t s = fp8ref_bf16_from_f32(fp8ref_silu32(bf16_to_f32(g[i])));
+        h[i] = fp8ref_bf16_from_f32(bf16_to_f32(s) * bf16_to_f32(u[i]));
+    }
+}
+
 /* Division shortcut used by the kernels: r = 1/s (IEEE), q0 = x*r,
  * e = fma(-q0, s, x), q1 = copysign(fma(e, r, q0), x).  Returns the number of (x, s) pairs,
  * x over all 65536 bf16 patterns with |x| <= amax(s) := 448*s-ish bound lifted

@@ -50,6 +50,8 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_quant_rowwise_from(None, _lib.IN_F16, 0, 16, 16, None, 16, None, None) == 0  # nothing to do
     assert lib.cfp8_quant_rowwise_from(None, 7, 4, 16, 16, None, 16, None, None) == _lib.EINVAL
     assert "unknown source dtype" in _lib.last_error()
+    assert lib.cfp8_swiglu_quant_group128(None, 128, None, 128, 4, 128, None, 128, None, None) == _lib.EINVAL
+    assert lib.cfp8_swiglu_quant_group128(None, 128, None, 128, 0, 128, None, 128, None, None) == 0
     assert lib.cfp8_quant_rowwise(None, -1, 16, 16, None, 16, None, None) == _lib.EINVAL
     assert lib.cfp8_quant_block128(None, 1, 128, 128, None, None, 0, None) == _lib.EINVAL
     assert lib.cfp8_quant_group128(None, 4, 128, 128, None, 128, None, 0, None) == _lib.EINVAL

@@ -129,3 +129,42 @@ def test_division_shortcut_is_exact():
     scales = O.scale_from_amax(amax).numpy()
     bad, soft = C.check_fast_div(scales)
     assert bad == 0 and soft == 0
+
+
+def _swiglu_inputs(M, I, seed):
+    g = torch.Generator().manual_seed(seed)
+    gate = (torch.randn(M, I, generator=g) * 3).to(torch.bfloat16)
+    up = (torch.randn(M, I, generator=g) * 2).to(torch.bfloat16)
+    gate[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 80.0, -80.0, 1e-3, -1e-3]).to(torch.bfloat16)
+    return gate, up
+
+
+def test_exp32_accuracy_and_silu_closed_forms():
+    """The fixed fp32 exp sequence stays within 2 ulp of the fp64 exponential over its whole range, and
+    silu has its closed-form values at 0 and at both ends."""
+    lib = C.load()
+    worst = 0.0
+    for x in np.linspace(-87.0, 88.0, 60001).astype(np.float32):
+        want = np.exp(np.float64(x))
+        worst = max(worst, abs(np.float64(lib.fp8ref_exp32(float(x))) - want) / np.float64(np.spacing(np.float32(want))))
+    assert worst < 2.0
+    assert lib.fp8ref_exp32(0.0) == 1.0
+    assert lib.fp8ref_silu32(0.0) == 0.0 and lib.fp8ref_silu32(40.0) == 40.0
+    assert lib.fp8ref_silu32(-120.0) == 0.0 and np.signbit(np.float32(lib.fp8ref_silu32(-120.0)))
+    assert np.isnan(lib.fp8ref_silu32(float("nan")))
+    assert abs(lib.fp8ref_silu32(1.0) - 1.0 / (1.0 + np.exp(-1.0))) < 1e-7
+
+
+def test_swiglu_restatement_against_torch_ops():
+    """bf16(bf16(silu(g)) * u) of the C restatement against torch's silu(g) * u on bf16 tensors: equal except
+    where torch's exp differs in the last fp32 bit and flips a bf16 rounding - at most 0.1 % of the elements,
+    each by one bf16 ulp - and the quantised result is the 1x128 quantiser applied to that hidden state."""
+    gate, up = _swiglu_inputs(96, 768, 21)
+    h = torch.from_numpy(C.swiglu(u16(gate), u16(up)).view(np.int16)).view(torch.bfloat16)
+    want = O.swiglu_hidden(gate, up)
+    diff = (h.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    assert int(diff.max()) <= 1
+    assert float((diff != 0).float().mean()) <= 1e-3
+    q, s = C.swiglu_quant_group128(u16(gate), u16(up))
+    qo, so = O.quant_group128(h)
+    assert (q == qo.numpy()).all() and (s.view(np.int32) == so.numpy().view(np.int32)).all()

@@ -192,6 +192,16 @@ def test_ds_group_gemm_strategy(dev):
     xs = torch.zeros(tok.numel(), H, dtype=torch.bfloat16)
     xs[tok >= 0] = x[tok[tok >= 0]]
     out = strat.execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+    # the same module through the other kernel choices: one fused gate_up GEMM gives the very same bits as two
+    # GEMMs; the unfused activation (torch silu, mul, then the quantiser) may differ by a bf16 ulp in the hidden state
+    assert strat.fuse_swiglu and not strat.fuse_gate_up
+    out_gu = group_gemms.DSGroupGEMM(act, fuse_gate_up=True).execute(
+        xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+    assert torch.equal(out_gu, out)
+    out_plain = group_gemms.DSGroupGEMM(act, fuse_swiglu=False).execute(
+        xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+    assert O.rel_frobenius(out_plain.float(), out.float()) <= 5e-3
+    assert not group_gemms.DSGroupGEMM(torch.nn.functional.gelu).fuse_swiglu
 
     # oracle pipeline; execute() treats every row of a padded group as belonging to that expert
     full_idx = ops.create_indices_from_offsets_nosync(m_offsets, tok.numel())

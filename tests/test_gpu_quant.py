@@ -334,3 +334,54 @@ def test_group128_edges(dev):
     assert_bytes(q, qo, "group edge bytes")
     q, s = ops.prepare_fp8_input(torch.empty(0, 256, dtype=torch.bfloat16, device=dev))
     assert q.shape == (0, 256) and s.shape == (0, 2)
+
+
+# ---------------------------------------------------------------------------- SwiGLU + 1x128 requantisation
+def _np16(t):
+    import numpy as np
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("M,I", [(1, 128), (37, 200), (300, 768), (129, 1536), (64, 8)])
+def test_swiglu_quant_bit_exact(dev, M, I):
+    """cfp8_swiglu_quant_group128 against the C restatement of the same fp32 operation sequence: bytes and
+    scales bit-exact, including NaN / Inf groups, ragged tail groups and saturating products."""
+    import numpy as np
+    from oracle import c_oracle as C
+    g = torch.Generator().manual_seed(M * 7 + I)
+    gate = (torch.randn(M, I, generator=g) * 4).to(torch.bfloat16)
+    up = (torch.randn(M, I, generator=g) * torch.exp(torch.randn(M, 1, generator=g) * 2)).to(torch.bfloat16)
+    if I >= 8:
+        gate[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 80.0, -80.0, 1e-3, -1e-3]).to(torch.bfloat16)
+    if M > 4:
+        gate[1, 3] = float("nan")
+        up[2, 5] = float("inf")
+        gate[3] = 0
+        up[4] = 0
+    q, s = ops.swiglu_quant(gate.to(dev), up.to(dev))
+    qo, so = C.swiglu_quant_group128(_np16(gate), _np16(up))
+    qo, so = torch.from_numpy(qo), torch.from_numpy(so)
+    nan = torch.isnan(so)
+    assert_scales(s.cpu()[~nan], so[~nan], f"swiglu {M}x{I} scales")
+    assert bool(torch.isnan(s.cpu()[nan]).all())
+    # NaN groups: canonical 0x7F bytes on both sides
+    assert_bytes(q, qo, f"swiglu {M}x{I} bytes")
+
+
+def test_swiglu_quant_fused_gate_up_layout_and_torch_semantics(dev):
+    """gate and up as the two column halves of one [M, 2I] GEMM output (row pitch 2I), and the result
+    against torch's own silu(g) * u followed by the 1x128 quantiser: dequantised values within fp8
+    resolution everywhere, hidden-state flips of one bf16 ulp allowed on at most 0.1 % of the groups."""
+    M, I = 257, 768
+    g = torch.Generator().manual_seed(5)
+    gu = (torch.randn(M, 2 * I, generator=g) * 3).to(torch.bfloat16)
+    gud = gu.to(dev)
+    q, s = ops.swiglu_quant(gud[:, :I], gud[:, I:])
+    q2, s2 = ops.swiglu_quant(gud[:, :I].contiguous(), gud[:, I:].contiguous())
+    assert torch.equal(q.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s, s2)
+    qo, so = O.swiglu_quant_group128(gu[:, :I], gu[:, I:])
+    same_scale = (s.cpu().view(torch.int32) == so.view(torch.int32))
+    assert float((~same_scale).float().mean()) <= 1e-3
+    got = O.group128_dequant(u8(q), s.cpu())
+    want = O.group128_dequant(qo, so)
+    assert O.rel_frobenius(got, want) <= 1e-3
