@@ -844,7 +844,11 @@ static int check_common(const char* who, const void* a, const void* b, const flo
     if (M < 0 || N < 0 || K < 0) return set_error(CFP8_EINVAL, "%s: negative shape", who);
     if (M == 0 || N == 0) return CFP8_OK;  // nothing to compute: pointers may be null
     if (!a || !b || !sa || !sb || !out) return set_error(CFP8_EINVAL, "%s: null pointer", who);
-    if (K % 128 || N % 16) return set_error(CFP8_EINVAL, "%s: K=%lld must be a multiple of 128 and N=%lld of 16", who, (long long)K, (long long)N);
+    if (K == 0 || K % 128 || N % 16)
+        return set_error(CFP8_EINVAL, "%s: K=%lld must be a positive multiple of 128 and N=%lld a multiple of 16", who, (long long)K, (long long)N);
+    // the kernels index rows with 32-bit integers and tile-local byte offsets with 32 bits
+    if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || ld_a >= (1ll << 24) || ld_b >= (1ll << 24))
+        return set_error(CFP8_EINVAL, "%s: shape beyond the supported range (M, N, K < 2^31, leading dimensions < 2^24)", who);
     if (ld_a % 16 || ld_b % 16 || ld_a < K || ld_b < K || ld_out < N || ld_out % 4)
         return set_error(CFP8_EINVAL, "%s: bad leading dimension (ld_a=%lld ld_b=%lld ld_out=%lld)", who, (long long)ld_a, (long long)ld_b, (long long)ld_out);
     if (!aligned16(a) || !aligned16(b) || !aligned16(out) || !aligned16(sb))

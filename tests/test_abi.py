@@ -58,6 +58,13 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert lib.cfp8_gemm_block128(None, 128, None, None, 128, None, 1, 1, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert lib.cfp8_quant_tensorwise_multi(None, 3, None, None) == _lib.EINVAL
+    # shape checks come before any device access: host pointers are never dereferenced here
+    buf = ctypes.create_string_buffer(4096)
+    ptr = (ctypes.addressof(buf) + 255) & ~255
+    assert lib.cfp8_scaled_mm_rowwise(ptr, 128, ptr, ptr, 128, ptr, ptr, 64, 0, 16, 64, 0, None) == _lib.EINVAL   # K = 0
+    assert "positive multiple of 128" in _lib.last_error()
+    assert lib.cfp8_scaled_mm_rowwise(ptr, 1 << 24, ptr, ptr, 128, ptr, ptr, 64, 0, 16, 64, 128, None) == _lib.EINVAL
+    assert "supported range" in _lib.last_error()
     # empty problems succeed without pointers
     assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0
