@@ -144,6 +144,28 @@ int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up
                                int64_t rows, int64_t cols, void* q, int64_t ld_q, float* scales,
                                void* stream);
 
+/* Permutation indices that regroup tokens from (source rank, local expert) order into expert
+ * order with every group padded to a multiple of `alignment` rows (an expert without tokens
+ * still gets `alignment` rows).  tokens_per_expert_group int64 [num_ranks * experts_per_rank],
+ * rank-major.  Outputs: m_sizes, m_offsets int32 [experts_per_rank] (padded group sizes and
+ * their inclusive cumulative sum), start_index_values int64 [num_ranks * experts_per_rank]
+ * (exclusive prefix sum of the counts), permuted_indices int32 [capacity]: source row of every
+ * output row, -1 for padding rows and for rows past sum(m_sizes).  Passing a capacity bound
+ * (e.g. tokens + experts * alignment) keeps the call free of a host read-back.
+ * Replaces generate_permute_indices / fill_indices_wrapper at
+ * cosmos_rl/policy/kernel/moe/indices.py:24-118, 147-220. */
+int cfp8_generate_permute_indices(const int64_t* tokens_per_expert_group, int experts_per_rank,
+                                  int num_ranks, int64_t alignment, int32_t* permuted_indices,
+                                  int64_t capacity, int32_t* m_sizes, int32_t* m_offsets,
+                                  int64_t* start_index_values, void* stream);
+
+/* out[i, :] = x[indices[i], :] for indices[i] >= 0, zeros for -1: the row gather that applies
+ * permuted_indices to the token matrix (the reference indexes with torch:
+ * cosmos_rl/policy/kernel/moe/moe.py token regrouping before group_gemms.py:152-156).
+ * Rows are row_bytes wide (multiple of 16); pitches in bytes. */
+int cfp8_gather_rows(const void* x, int64_t ld_x_bytes, const int32_t* indices, int64_t rows_out,
+                     int64_t row_bytes, void* out, int64_t ld_out_bytes, void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */
