@@ -98,6 +98,25 @@ def test_fp8_linear_cfg3_shapes(dev, M):
         assert torch.equal(o3.view(M, N), out16 + bias.to(dev))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (2, 272, 896), (3, 1024, 3584), (4, 48, 8320), (4, 18944, 3584)])
+def test_fp8_linear_small_m(dev, M, N, K):
+    """Decode shapes: cfp8_linear_rowwise equals cfp8_scaled_mm_rowwise on separately quantised activations bit
+    for bit; K > 4096 walks the K loop of the M <= 16 kernel more than once; a NaN token stays a NaN row and
+    leaves the others alone."""
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=99 + M + N, dev=dev)
+    y = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)
+    qxd, sxd = ops.quant_rowwise(x.to(dev))
+    y2 = ops.scaled_mm(qxd, f8(qw, dev).t(), sxd, sw.to(dev).t(), out_dtype=torch.float32)
+    assert torch.equal(y, y2)
+    ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
+    assert O.rel_frobenius(y.cpu(), ref) <= TIGHT
+    if M > 1:
+        xn = x.clone()
+        xn[0, 5] = float("nan")
+        yn = ops.fp8_linear(xn.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)
+        assert bool(torch.isnan(yn[0]).all()) and torch.equal(yn[1:], y[1:])
+
+
 def test_fp8_linear_full_cfg3_properties(dev):
     """Full Qwen2.5-7B MLP shape [8192, 3584] x [18944, 3584]^T on the GPU only.  Linearity in the
     weight scales (doubling sw doubles the fp32 output exactly), row-subset consistency with an
