@@ -122,14 +122,12 @@ def main() -> int:
     reps = max(3, args.steps)
     amax_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_amax_multi(descs, n, amax_ws.data_ptr(), stream)), reps)
     cast_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_cast_multi(descs, n, amax_ws.data_ptr(), stream)), reps)
-    # launches per pass: batches of <= 48 tensors (and <= CFP8_TW_BATCH_MB of bf16 if that knob is set)
-    budget = (int(os.environ.get("CFP8_TW_BATCH_MB", "0")) or (1 << 40)) << 20
-    launches, cnt, by = 0, 0, 0
+    # launches per pass: batches of <= 48 tensors
+    launches, cnt = 0, 0
     for t in tensors:
-        b = t.numel() * 2
-        if cnt and (cnt == 48 or by + b > budget):
-            launches, cnt, by = launches + 1, 0, 0
-        cnt, by = cnt + 1, by + b
+        if cnt == 48:
+            launches, cnt = launches + 1, 0
+        cnt += 1
     launches += 1
     cast_med = statistics.median(cast_ms)
     amax_med = statistics.median(amax_ms)

@@ -12,7 +12,6 @@
 //                  the tensor's slots and forms the scale on its own.
 // The table of tensors travels in the kernel arguments (scalar loads), so the
 // library needs no device-side descriptor buffer.
-#include <stdlib.h>
 
 #include "cfp8_common.h"
 
@@ -108,27 +107,6 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
     }
 }
 
-// bf16 bytes per batch; CFP8_TW_BATCH_MB overrides the default (read once)
-static int64_t batch_bytes() {
-    static int64_t v = [] {
-        const char* e = getenv("CFP8_TW_BATCH_MB");
-        long mb = e ? atol(e) : 0;
-        if (mb <= 0) return (int64_t)1 << 60;  // default: no byte limit, 48 tensors per launch
-        return (int64_t)mb << 20;
-    }();
-    return v;
-}
-
-// Access policy, CFP8_TW_MODE overrides (read once).  bit 0: pass 1 loads stream past the
-// caches; bit 1: pass 2 loads do; bit 2: pass 2 stores do.
-static int access_mode() {
-    static int v = [] {
-        const char* e = getenv("CFP8_TW_MODE");
-        return e ? atoi(e) : 7;
-    }();
-    return v;
-}
-
 enum : int { kPhaseAmax = 1, kPhaseCast = 2 };
 
 static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream, int phases) {
@@ -152,25 +130,23 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
         const int64_t per = 64 * 1024;
         hipLaunchKernelGGL(tensorwise_zero_kernel, dim3((unsigned)((total + per - 1) / per)), dim3(64), 0, st, slots, total);
     }
-    // Tensors are taken in batches of at most kMaxBatch entries (and batch_bytes() of
-    // bf16 when that tuning knob is set); with both phases requested each batch runs
-    // pass 1 then pass 2 back to back.  Measured on MI355X: few large launches with
-    // streaming accesses beat small batches that would let pass 2 hit the 256 MiB
-    // memory-side cache, because every launch pays a ramp-up and a tail.
-    const int64_t budget_vecs = batch_bytes() / 16;
+    // Tensors are taken in batches of at most kMaxBatch entries; with both phases requested each
+    // batch runs pass 1 then pass 2 back to back.  Every access streams past the caches (non-temporal
+    // loads in both passes, non-temporal stores).  Measured on MI355X: few large launches with
+    // streaming accesses beat small batches that would let pass 2 hit the 256 MiB memory-side cache,
+    // because every launch pays a ramp-up and a tail.
     int64_t i = 0;
     while (i < n) {
         TensorTable tb;
         tb.n = 0;
         unsigned blocks = 0;
-        int64_t vecs = 0;
         while (i < n && tb.n < kMaxBatch) {
             const cfp8_tensor_desc& d = descs[i];
             int64_t nvec = d.numel / 8;
             // a tensor with no element still owns one workgroup: it writes the scale
             unsigned nb = (unsigned)((nvec + kChunkVecs - 1) / kChunkVecs);
             if (nb == 0) nb = 1;
-            if (tb.n > 0 && ((uint64_t)blocks + nb > 0x7FFFFFFFull || vecs + nvec > budget_vecs)) break;
+            if (tb.n > 0 && (uint64_t)blocks + nb > 0x7FFFFFFFull) break;
             tb.x[tb.n] = static_cast<const uint4*>(d.x);
             tb.q[tb.n] = static_cast<uint2*>(d.q);
             tb.scale[tb.n] = d.scale;
@@ -178,24 +154,12 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
             tb.amax[tb.n] = slots + i * kAmaxSlots;
             tb.first_block[tb.n] = blocks;
             blocks += nb;
-            vecs += nvec;
             ++tb.n;
             ++i;
         }
         tb.first_block[tb.n] = blocks;
-        const int mode = access_mode();
-        if (phases & kPhaseAmax) {
-            if (mode & 1) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
-            else hipLaunchKernelGGL(tensorwise_amax_kernel<false>, dim3(blocks), dim3(256), 0, st, tb);
-        }
-        if (phases & kPhaseCast) {
-            switch ((mode >> 1) & 3) {
-                case 0: hipLaunchKernelGGL((tensorwise_cast_kernel<false, false>), dim3(blocks), dim3(256), 0, st, tb); break;
-                case 1: hipLaunchKernelGGL((tensorwise_cast_kernel<true, false>), dim3(blocks), dim3(256), 0, st, tb); break;
-                case 2: hipLaunchKernelGGL((tensorwise_cast_kernel<false, true>), dim3(blocks), dim3(256), 0, st, tb); break;
-                default: hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb); break;
-            }
-        }
+        if (phases & kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
+        if (phases & kPhaseCast) hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
     }
     return check_launch("quant_tensorwise");
 }
