@@ -1,4 +1,5 @@
 // Version, error reporting and device check of libcosmosfp8.
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -24,26 +25,23 @@ int check_launch(const char* what) {
 }
 
 int check_device() {
-    // one flag per device ordinal; -1 unknown, 0 bad, 1 good
-    static int8_t cache[64];
-    static bool init = false;
-    if (!init) {
-        memset(cache, -1, sizeof(cache));
-        init = true;
-    }
+    // one flag per device ordinal: 0 unknown, 1 good, 2 bad.  Relaxed atomics: two threads that race on
+    // the first call both query the device and store the same answer.
+    static std::atomic<int8_t> cache[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {
         (void)hipGetLastError();
         return set_error(CFP8_EARCH, "no HIP device is current");
     }
-    if (dev >= 0 && dev < 64 && cache[dev] == 1) return CFP8_OK;
+    const bool cached = dev >= 0 && dev < 64;
+    if (cached && cache[dev].load(std::memory_order_relaxed) == 1) return CFP8_OK;
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
         (void)hipGetLastError();
         return set_error(CFP8_EARCH, "cannot query device %d", dev);
     }
-    bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-    if (dev >= 0 && dev < 64) cache[dev] = ok ? 1 : 0;
+    const bool ok = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    if (cached) cache[dev].store(ok ? 1 : 2, std::memory_order_relaxed);
     if (!ok) return set_error(CFP8_EARCH, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
     return CFP8_OK;
 }

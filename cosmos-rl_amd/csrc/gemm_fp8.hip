@@ -22,6 +22,8 @@
 //   rowwise:  acc over all of K, epilogue acc * sa[m] * sb[n];
 //   block:    every K step is one 128-block; its MFMA result is folded into the
 //             running sum as acc += part * (sa[m, kb] * sb[n / 128, kb]).
+#include <atomic>
+
 #include "cfp8_common.h"
 
 namespace cfp8 {
@@ -555,20 +557,33 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     }
 }
 
+// Kernels that use more than 64 KiB of LDS need the limit raised once per device and function.
+// `flag` is that (device, function) pair's once-flag; a race on the first call raises it twice, harmlessly.
+static int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag) {
+    if (flag.load(std::memory_order_relaxed)) return CFP8_OK;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    flag.store(true, std::memory_order_relaxed);
+    return CFP8_OK;
+}
+static int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached) beyond
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 64;
+    return dev >= 0 && dev < 64 ? dev : 64;
+}
+
 static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 256;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     constexpr size_t lds = (size_t)2 * 512 * 128;
-    static bool raised[2] = {false, false};
+    static std::atomic<bool> raised[65][2];  // zero-initialised
     const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
     const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256_kernel<true>)
                        : reinterpret_cast<const void*>(gemm_rowwise_256_kernel<false>);
-    if (!raised[v]) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
-        raised[v] = true;
-    }
+    const int slot = device_slot();
+    if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
     if (v) hipLaunchKernelGGL(gemm_rowwise_256_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_256_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm");
@@ -797,12 +812,10 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int f32 = out_dtype == CFP8_OUT_F32;
     const Kern kern = table[vec][f32];
     if (lds > 64 * 1024) {
-        static bool done[2][2] = {{false, false}, {false, false}};
-        if (!done[vec][f32]) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
-            done[vec][f32] = true;
-        }
+        static std::atomic<bool> done[65][2][2];  // zero-initialised
+        const int slot = device_slot();
+        if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
+        if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds, done[slot][vec][f32])) return rc;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds, st, p);
     return check_launch("gemm");

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
 // group-rows so that four loads are in flight per lane.
 // ---------------------------------------------------------------------------
 template <int MODE>
-__global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__ x, int64_t rows, int nvec,
+__global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__ x, int nvec,
                                                        int ngroups, int64_t ldx, uint2* __restrict__ q, int64_t ldq,
                                                        float* __restrict__ scales, int64_t total_groups) {
     const int sub = threadIdx.x & 15;
@@ -226,11 +226,11 @@ int launch_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_
     const uint4* xv = static_cast<const uint4*>(x);
     uint2* qv = static_cast<uint2*>(q);
     if (mode == CFP8_GROUP_MODE_DIV)
-        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DIV>, dim3((unsigned)blocks), dim3(256), 0, st, xv, rows,
+        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DIV>, dim3((unsigned)blocks), dim3(256), 0, st, xv,
                            (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
     else
         hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DEEPEP>, dim3((unsigned)blocks), dim3(256), 0, st, xv,
-                           rows, (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
+                           (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
     return check_launch("quant_group128");
 }
 
