@@ -413,17 +413,25 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     // global -> registers -> LDS.  Per K step 64 wave-wide loads of 1 KiB (8 rows x 128 B): wave w
     // takes u = w, w + 4, ...; u < 32: activation rows u * 8 .., u >= 32: weight rows (u - 32) * 8 ..
     const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
-    const uint8_t* a_base = p.a + (int64_t)m0 * p.ld_a;  // wave-uniform
-    const uint8_t* b_base = p.b + (int64_t)n0 * p.ld_b;
+    // Wave-uniform bases and strides of this wave's row blocks (u >> 1 = (wave >> 1) + 2 i).  They pass
+    // through an empty asm so that the compiler keeps them in SGPRs for the whole K loop: left alone it
+    // re-reads the kernel arguments inside the loop, and every scalar load has to be waited for with
+    // lgkmcnt(0), which drains the LDS queue of the fragment reads in flight.
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_b;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, b_step = 32u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
+    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));
     const int uodd = wave & 1;  // u & 1 is the same for all of a wave's loads
     const uint32_t va_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_a + (uint32_t)(st_c * 16);
     const uint32_t vb_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_b + (uint32_t)(st_c * 16);
     const int l_lane = lds_chunk_offset(uodd * 8 + st_row8, st_c);
     i32x4 R[16];  // ext-vector type on purpose: an array of uint4 structs stays in scratch memory
-    auto gload = [&](int kt, int i) {
-        const int u = wave + 4 * i, isB = u >> 5, rb = (u & 31) >> 1;
-        const uint8_t* base = isB ? b_base + (int64_t)rb * 16 * p.ld_b : a_base + (int64_t)rb * 16 * p.ld_a;
-        R[i] = *reinterpret_cast<const i32x4*>(base + ((int64_t)kt << 7) + (isB ? vb_lane : va_lane));
+    auto gload = [&](int kt, int i) {  // i < 8: activation rows, i >= 8: weight rows (wave < 4)
+        const uint64_t base = (i < 8 ? a_wave + (uint64_t)i * a_step : b_wave + (uint64_t)(i - 8) * b_step) + ((uint64_t)kt << 7);
+        // an address built from an integer must be told that it is global memory (else: flat loads)
+        typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+        typedef const __attribute__((address_space(1))) i32x4* gvec_t;
+        R[i] = *(gvec_t)((gptr_t)base + (i < 8 ? va_lane : vb_lane));
     };
     auto lstore = [&](int stage, int i) {
         const int u = wave + 4 * i, isB = u >> 5, rb = (u & 31) >> 1;
