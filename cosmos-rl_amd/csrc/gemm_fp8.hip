@@ -459,13 +459,19 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     };
     i32x8 W[2][4], X[2][4];  // weight / activation fragments of the two halves of the wave's block
 
-    // prologue: tile 0 -> stage 0 (through registers), tile 1 -> registers
+    // prologue: tile 0 -> stage 0 (through registers); tile 1: activation half -> stage 1, weight half stays
+    // in registers 8..15; activation half of tile 2 -> registers 0..7
+    const int last = KT - 1;
 #pragma unroll
     for (int i = 0; i < 16; ++i) gload(0, i);
 #pragma unroll
     for (int i = 0; i < 16; ++i) lstore(0, i);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) gload(KT > 1 ? 1 : 0, i);
+    for (int i = 0; i < 16; ++i) gload(1 < last ? 1 : last, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lstore(1, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) gload(2 < last ? 2 : last, i);
     __syncthreads();
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -476,18 +482,22 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1, nxt = cur ^ 1;
-        const int ktl = kt + 2 < KT ? kt + 2 : KT - 1;  // past the end: re-read the last tile, never consumed
+        // past the end: re-read the last tile, never consumed
+        const int kb = kt + 2 < last ? kt + 2 : last;  // weight half, loaded in S0/S1
+        const int ka = kt + 3 < last ? kt + 3 : last;  // activation half, loaded in S2/S3
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
             if (g < 4) X[1][g] = frag(cur, x_off, x_off2, 4 + g);
-            lstore(nxt, g);
+            if (g & 1) gload(kb, 8 + (g >> 1));
+            else lstore(nxt, 8 + (g >> 1));
             CFP8_MMA2(0, 0, 0, 0, g);
             CFP8_PHASE_END();
         }
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
             if (g < 4) W[1][g] = frag(cur, w_off, w_off2, 4 + g);
-            lstore(nxt, 8 + g);
+            if (g & 1) gload(kb, 12 + (g >> 1));
+            else lstore(nxt, 12 + (g >> 1));
             CFP8_MMA2(0, 0, 1, 1, g);
             CFP8_PHASE_END();
         }
@@ -496,15 +506,17 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
         CFP8_PHASE_END();
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            gload(ktl, g);
             if (g < 4) W[0][g] = frag(nxt, w_off, w_off2, g);  // after the last step: stale data, unused
+            if (g & 1) gload(ka, g >> 1);
+            else lstore(cur, g >> 1);
             CFP8_MMA2(1, 1, 0, 0, g);
             CFP8_PHASE_END();
         }
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            gload(ktl, 8 + g);
             if (g < 4) X[0][g] = frag(nxt, x_off, x_off2, g);
+            if (g & 1) gload(ka, 4 + (g >> 1));
+            else lstore(cur, 4 + (g >> 1));
             CFP8_MMA2(1, 1, 1, 1, g);
             CFP8_PHASE_END();
         }
