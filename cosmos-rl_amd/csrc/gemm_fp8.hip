@@ -866,8 +866,25 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kRowwise && p.M > 128 && p.M <= 256) return launch_cfg<256, 128, 4, 2, kRowwise>(p, out_dtype, st);
     if (MODE == kRowwise && p.M > 256 && p.M <= 512) return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);
     if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
-    if (p.M % 256 == 0 && p.N % 256 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0)
+    if (p.M % 256 == 0 && p.N % 256 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0) {
+        // One workgroup per CU and equal tiles: the launch runs in rounds of 256 tiles, and a last round that is
+        // at most half full costs a whole round.  Then the last tile-columns go to a second launch on 256 x 128
+        // tiles (half the work per workgroup, 8 waves) and the first launch ends on a full round.
+        const int64_t tm = p.M / 256, tn = p.N / 256, rem = (tm * tn) % 256;
+        const int64_t cut = (rem + tm - 1) / tm;  // tile-columns that hold the partial round
+        if (tm * tn > 256 && rem > 0 && rem <= 128 && cut < tn) {
+            GemmArgs head = p;
+            head.N = (int)((tn - cut) * 256);
+            if (int rc = launch_rowwise_256(head, out_dtype, st)) return rc;
+            GemmArgs tail = p;
+            tail.N = (int)(cut * 256);
+            tail.b = p.b + (int64_t)head.N * p.ld_b;
+            tail.sb = p.sb + head.N;
+            tail.out = static_cast<uint8_t*>(p.out) + (int64_t)head.N * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+            return launch_cfg<256, 128, 4, 2, kRowwise>(tail, out_dtype, st);
+        }
         return launch_rowwise_256(p, out_dtype, st);
+    }
     return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);
 }
 
