@@ -462,12 +462,33 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     // prologue: tile 0 -> stage 0 (through registers); tile 1: activation half -> stage 1, weight half stays
     // in registers 8..15; activation half of tile 2 -> registers 0..7
     const int last = KT - 1;
+    // The tile's 256 activation scales and 256 weight scales go to LDS behind the two stages now, so that the
+    // epilogue does not start with a global round trip.
+    float* const scale_lds = reinterpret_cast<float*>(smem + 2 * STAGE);  // [0, 256): sa, [256, 512): sb
+    {
+        const float s_a = p.sa[m0 + t], s_b = p.sb[n0 + t];
+        scale_lds[t] = s_a;
+        scale_lds[256 + t] = s_b;
+    }
+    // (tiles 0 and 1 are requested together: the fragment registers are still free to hold tile 0)
+    {
+        i32x4 T0[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) gload(0, i);
+        for (int i = 0; i < 16; ++i) {
+            gload(0, i);
+            T0[i] = R[i];
+        }
 #pragma unroll
-    for (int i = 0; i < 16; ++i) lstore(0, i);
+        for (int i = 0; i < 16; ++i) gload(1 < last ? 1 : last, i);
+        CFP8_PHASE_END();
 #pragma unroll
-    for (int i = 0; i < 16; ++i) gload(1 < last ? 1 : last, i);
+        for (int i = 0; i < 16; ++i) {
+            const i32x4 keep = R[i];
+            R[i] = T0[i];
+            lstore(0, i);
+            R[i] = keep;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) lstore(1, i);
 #pragma unroll
@@ -524,13 +545,13 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 
     float sam[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) sam[j] = p.sa[m0 + wm * 128 + j * 16 + lrow];
+    for (int j = 0; j < 8; ++j) sam[j] = scale_lds[wm * 128 + j * 16 + lrow];
     if (OUT_F32) {
         // a lane already owns 16 contiguous bytes: store directly
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int n = n0 + wn * 128 + i * 16 + quarter * 4;
-            const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
+            const f32x4 sbn = *reinterpret_cast<const f32x4*>(scale_lds + 256 + wn * 128 + i * 16 + quarter * 4);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int m = m0 + wm * 128 + j * 16 + lrow;
@@ -544,12 +565,12 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     }
     // bf16: scale, convert, turn the wave's 128 x 128 block through LDS in two halves of 64 rows
     // (row stride 272 B keeps the 8-byte stores of 16 rows on different banks)
+    f32x4 sbn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(scale_lds + 256 + wn * 128 + i * 16 + quarter * 4);
     __syncthreads();  // all waves are done reading the operand stages
     constexpr int EST = 272;
     uint8_t* const ebuf = smem + wave * (64 * EST);
-    f32x4 sbn[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(p.sb + n0 + wn * 128 + i * 16 + quarter * 4);
     const int rd_row = lane >> 4, rd_chunk = lane & 15;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -596,7 +617,7 @@ static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 256;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
-    constexpr size_t lds = (size_t)2 * 512 * 128;
+    constexpr size_t lds = (size_t)2 * 512 * 128 + 2 * 256 * sizeof(float);  // two operand stages + the tile's scales
     static std::atomic<bool> raised[65][2];  // zero-initialised
     const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
     const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256_kernel<true>)
