@@ -887,7 +887,21 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kRowwise && p.M > 128 && p.M <= 256) return launch_cfg<256, 128, 4, 2, kRowwise>(p, out_dtype, st);
     if (MODE == kRowwise && p.M > 256 && p.M <= 512) return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);
     if (p.M <= 512 || MODE != kRowwise) return launch_cfg<128, 128, 2, 2, MODE>(p, out_dtype, st);
-    if (p.M % 256 == 0 && p.N % 256 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0) {
+    const bool out16 = (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0;
+    if (p.M % 256 != 0 && p.N % 256 == 0 && out16) {
+        // any number of tokens: the first M / 256 * 256 rows take the 256 x 256 kernel, the last < 256 rows are
+        // a small problem of their own (rows are independent, so the split changes no result)
+        GemmArgs body = p;
+        body.M = p.M / 256 * 256;
+        if (int rc = launch_gemm<MODE>(body, out_dtype, st)) return rc;
+        GemmArgs rest = p;
+        rest.M = p.M - body.M;
+        rest.a = p.a + (int64_t)body.M * p.ld_a;
+        rest.sa = p.sa + body.M;
+        rest.out = static_cast<uint8_t*>(p.out) + (int64_t)body.M * p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+        return launch_gemm<MODE>(rest, out_dtype, st);
+    }
+    if (p.M % 256 == 0 && p.N % 256 == 0 && out16) {
         // One workgroup per CU and equal tiles: the launch runs in rounds of 256 tiles, and a last round that is
         // at most half full costs a whole round.  Then the last tile-columns go to a second launch on 256 x 128
         // tiles (half the work per workgroup, 8 waves) and the first launch ends on a full round.

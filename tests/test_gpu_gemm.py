@@ -44,7 +44,9 @@ def rowwise_operands(M, N, K, seed, dev):
                                    # full 256x256 tiles: the four-wave pipelined kernel, K of 1, 3 and 28 steps
                                    (768, 256, 128), (1024, 512, 384), (2048, 1280, 896),
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
-                                   (2048, 8448, 256)])
+                                   (2048, 8448, 256),
+                                   # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
+                                   (1000, 512, 384), (520, 256, 256)])
 def test_scaled_mm_rowwise(dev, M, N, K):
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
     ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
