@@ -249,6 +249,38 @@ def test_grouped_gemm(dev, T, E, K, N, topk):
     assert torch.equal(out2.cpu()[rows0], out[perm])
 
 
+def test_random_shapes_all_dispatch_paths(dev):
+    """Seeded sweep over row counts on both sides of every dispatch threshold (16, 32, 64, 128, 256, 512, multiples of
+    256 and not), N a multiple of 16 or 256, K 1..9 steps: rowwise mm, fused linear and block-scaled mm."""
+    import random
+    rnd = random.Random(2024)
+    Ms = [1, 5, 16, 17, 33, 64, 65, 127, 129, 255, 257, 300, 511, 513, 600, 768, 1000, 1030, 1279]
+    for it in range(24):
+        M = rnd.choice(Ms)
+        N = 256 * rnd.randint(1, 4) if rnd.random() < 0.4 else 16 * rnd.randint(1, 60)
+        K = 128 * rnd.randint(1, 9)
+        mode = rnd.choice(["row", "lin", "blk"])
+        g = torch.Generator().manual_seed(it)
+        x = (torch.randn(M, K, generator=g) * 2).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16)
+        if mode == "blk":
+            qx, sx = O.quant_group128(x)
+            qw, sw = O.quant_block128(w)
+            ref = O.scaled_mm_block128(qx, sx, qw, sw, accum=torch.float64)
+            out = torch.empty(M, N, dtype=torch.float32, device=dev)
+            ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out)
+        else:
+            qw, sw = O.quant_rowwise(w)
+            ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
+            if mode == "lin":
+                out = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)
+            else:
+                qx, sx = O.quant_rowwise(x)
+                out = ops.scaled_mm(f8(qx, dev), f8(qw, dev).t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+        err = O.rel_frobenius(out.cpu(), ref)
+        assert err <= TIGHT, f"{mode} M={M} N={N} K={K}: {err:.3e}"
+
+
 def test_gemm_errors(dev):
     a = torch.zeros(16, 100, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
     b = torch.zeros(32, 100, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
