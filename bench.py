@@ -342,6 +342,18 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
     mfma("grouped_cfg5_mlp_quant_gateup_swiglu_down", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=50)
+    # weighted combine of the expert rows back into token order (bf16 rounding at every step)
+    e_sorted, order = torch.sort(topi, stable=True)
+    first = torch.cumsum(counts, 0) - counts
+    row_of_slot = torch.empty(T * TOPK, dtype=torch.int64, device=dev)
+    row_of_slot[order] = start[e_sorted] + torch.arange(T * TOPK, device=dev) - first[e_sorted]
+    slot_order = torch.argsort(topi.view(T, TOPK), dim=1, stable=True)
+    row_map = torch.gather(row_of_slot.view(T, TOPK), 1, slot_order).to(torch.int32).contiguous()
+    probs = torch.rand(T, TOPK, generator=gen, device=dev).to(torch.bfloat16)
+    yt = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    hbm("combine_rows_cfg5_%dx%d_top%d" % (T, H, TOPK), T * TOPK * (2 * H + 6) + T * H * 2,
+        lambda: check(lib.cfp8_combine_rows(dn.data_ptr(), H, total, row_map.data_ptr(), probs.data_ptr(), 0, T, TOPK, H, 0,
+                                            yt.data_ptr(), H, stream)))
     if "grouped_cfg5_mlp_quant_gateup_swiglu_down" in out:
         out["grouped_cfg5_mlp_quant_gateup_swiglu_down"]["routed_rows"] = routed
         out["grouped_cfg5_mlp_quant_gateup_swiglu_down"]["padded_rows"] = total

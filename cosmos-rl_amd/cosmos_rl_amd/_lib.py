@@ -17,6 +17,7 @@ GROUP_MODE_DIV = 0
 GROUP_MODE_DEEPEP = 1
 TENSORWISE_AMAX_SLOTS = 64
 IN_BF16, IN_F16, IN_F32 = 0, 1, 2
+COMBINE_BF16_STEPS, COMBINE_F32 = 0, 1
 
 EINVAL, EARCH, ELAUNCH, EWORKSPACE = -1, -2, -3, -4
 
@@ -40,6 +41,8 @@ SIGNATURES = {
     "cfp8_swiglu_quant_group128": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_generate_permute_indices": (c_int, [c_void_p, c_int, c_int, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "cfp8_gather_rows": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
+    "cfp8_combine_rows": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_int,
+                                  c_void_p, c_int64, c_void_p]),
     "cfp8_dequant_block128": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "cfp8_scaled_mm_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                        c_int, c_int64, c_int64, c_int64, c_void_p]),

@@ -108,6 +108,64 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint4* __restric
     }
 }
 
+// Weighted combine of expert outputs back into token order: one wavefront per (token, 64 x 16-byte
+// chunk of the row).  Lane s first fetches slot s of the token's row map and weight; the slots are
+// then walked in order with lane-to-scalar reads, so every load of the walk has a uniform base.
+// A slot whose row is negative (or not below num_rows) contributes an exact zero.
+//   STEPS: every product and every partial sum is rounded to bf16, the arithmetic of
+//          `y.scatter_add_(0, idx, expert_out * weights[idx, top, None])` on bf16 tensors;
+//   else:  fp32 accumulator acc = fma(row, weight, acc), rounded to bf16 once.
+template <bool STEPS, bool W32>
+__global__ __launch_bounds__(256) void combine_rows_kernel(const uint4* __restrict__ rows, int64_t ldr,
+                                                           int64_t num_rows, const int32_t* __restrict__ row_map,
+                                                           const void* __restrict__ weights, int64_t tokens, int topk, int nvec, int chunks,
+                                                           uint4* __restrict__ out, int64_t ldo) {
+    const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (unit >= tokens * chunks) return;  // whole wavefronts leave
+    const int64_t t = unit / chunks;
+    const int lane = threadIdx.x & 63;
+    const int v = (int)(unit - t * chunks) * 64 + lane;
+    const int vv = v < nvec ? v : nvec - 1;  // lanes past the row end re-read its last vector and store nothing
+    int32_t src = -1;
+    float w = 0.f;
+    if (lane < topk) {
+        src = row_map[t * topk + lane];
+        if (W32) w = static_cast<const float*>(weights)[t * topk + lane];
+        else w = __uint_as_float((u32) static_cast<const uint16_t*>(weights)[t * topk + lane] << 16);
+    }
+    if (src < 0 || src >= num_rows) {  // padding slot, or an index no source row has
+        src = -1;
+        w = 0.f;
+    }
+    u32 y[4] = {0u, 0u, 0u, 0u};
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int s = 0; s < topk; ++s) {
+        const int32_t r = __builtin_amdgcn_readlane(src, s);
+        const float ws = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(w), s));
+        uint4 d = ld16<true>(rows + (int64_t)(r < 0 ? 0 : r) * ldr + vv);
+        if (r < 0) d = make_uint4(0, 0, 0, 0);
+        const u32 x[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float lo = __uint_as_float(x[e] << 16), hi = __uint_as_float(x[e] & 0xFFFF0000u);
+            if (STEPS) {
+                const u32 p = pack_bf16x2(lo * ws, hi * ws);
+                y[e] = pack_bf16x2(__uint_as_float(y[e] << 16) + __uint_as_float(p << 16),
+                                   __uint_as_float(y[e] & 0xFFFF0000u) + __uint_as_float(p & 0xFFFF0000u));
+            } else {
+                acc[2 * e] = __builtin_fmaf(lo, ws, acc[2 * e]);
+                acc[2 * e + 1] = __builtin_fmaf(hi, ws, acc[2 * e + 1]);
+            }
+        }
+    }
+    if (!STEPS) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = pack_bf16x2(acc[2 * e], acc[2 * e + 1]);
+    }
+    if (v < nvec) st16<true>(out + t * ldo + v, make_uint4(y[0], y[1], y[2], y[3]));
+}
+
 }  // namespace cfp8
 
 extern "C" int cfp8_generate_permute_indices(const int64_t* tokens_per_expert_group, int experts_per_rank, int num_ranks,
@@ -152,4 +210,38 @@ extern "C" int cfp8_gather_rows(const void* x, int64_t ld_x_bytes, const int32_t
                        static_cast<const uint4*>(x), ld_x_bytes / 16, indices, rows_out, (int)(row_bytes / 16),
                        static_cast<uint4*>(out), ld_out_bytes / 16);
     return check_launch("gather_rows");
+}
+
+extern "C" int cfp8_combine_rows(const void* rows, int64_t ld_rows, int64_t num_rows, const int32_t* row_map,
+                                 const void* weights, int weights_dtype, int64_t tokens, int topk, int64_t hidden,
+                                 int mode, void* out, int64_t ld_out, void* stream) {
+    using namespace cfp8;
+    if (tokens < 0 || hidden < 0 || num_rows < 0) return set_error(CFP8_EINVAL, "combine_rows: negative shape");
+    if (topk < 0 || topk > 64) return set_error(CFP8_EINVAL, "combine_rows: topk=%d must be in [0, 64]", topk);
+    if (mode != CFP8_COMBINE_BF16_STEPS && mode != CFP8_COMBINE_F32) return set_error(CFP8_EINVAL, "combine_rows: unknown mode %d", mode);
+    if (weights_dtype != CFP8_IN_BF16 && weights_dtype != CFP8_IN_F32)
+        return set_error(CFP8_EINVAL, "combine_rows: weights must be bf16 or fp32");
+    if (mode == CFP8_COMBINE_BF16_STEPS && weights_dtype != CFP8_IN_BF16)
+        return set_error(CFP8_EINVAL, "combine_rows: the bf16-steps mode takes bf16 weights");
+    if (tokens == 0 || hidden == 0) return CFP8_OK;
+    if (!out || (topk > 0 && (!rows || !row_map || !weights))) return set_error(CFP8_EINVAL, "combine_rows: null pointer");
+    if (topk > 0 && num_rows == 0) return set_error(CFP8_EINVAL, "combine_rows: no source rows");
+    if (hidden % 8 || ld_rows % 8 || ld_out % 8 || ld_rows < hidden || ld_out < hidden)
+        return set_error(CFP8_EINVAL, "combine_rows: hidden=%lld and the row pitches must be multiples of 8 with pitch >= hidden", (long long)hidden);
+    if (!aligned16(rows) || !aligned16(out)) return set_error(CFP8_EINVAL, "combine_rows: misaligned pointer");
+    const int64_t nvec = hidden / 8, chunks = (nvec + 63) / 64;
+    if (nvec > 0x7FFFFFFFll || tokens > 0x7FFFFFFFFFFFll / chunks || (tokens * chunks + 3) / 4 > 0x7FFFFFFFll)
+        return set_error(CFP8_EINVAL, "combine_rows: too large for one launch");
+    if (int rc = check_device()) return rc;
+    const dim3 grid((unsigned)((tokens * chunks + 3) / 4)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint4* r = static_cast<const uint4*>(rows);
+    uint4* o = static_cast<uint4*>(out);
+    if (mode == CFP8_COMBINE_BF16_STEPS)
+        hipLaunchKernelGGL((combine_rows_kernel<true, false>), grid, block, 0, st, r, ld_rows / 8, num_rows, row_map, weights, tokens, topk, (int)nvec, (int)chunks, o, ld_out / 8);
+    else if (weights_dtype == CFP8_IN_F32)
+        hipLaunchKernelGGL((combine_rows_kernel<false, true>), grid, block, 0, st, r, ld_rows / 8, num_rows, row_map, weights, tokens, topk, (int)nvec, (int)chunks, o, ld_out / 8);
+    else
+        hipLaunchKernelGGL((combine_rows_kernel<false, false>), grid, block, 0, st, r, ld_rows / 8, num_rows, row_map, weights, tokens, topk, (int)nvec, (int)chunks, o, ld_out / 8);
+    return check_launch("combine_rows");
 }

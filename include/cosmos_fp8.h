@@ -166,6 +166,25 @@ int cfp8_generate_permute_indices(const int64_t* tokens_per_expert_group, int ex
 int cfp8_gather_rows(const void* x, int64_t ld_x_bytes, const int32_t* indices, int64_t rows_out,
                      int64_t row_bytes, void* out, int64_t ld_out_bytes, void* stream);
 
+/* Weighted combine of expert outputs back into token order (bf16 in, bf16 out):
+ *   out[t, :] = sum over slots s = 0 .. topk-1, in that order, of weights[t, s] * rows[row_map[t, s], :]
+ * row_map int32 [tokens, topk]; a slot with row_map < 0 or >= num_rows contributes nothing.
+ * topk <= 64, hidden % 8 == 0, pitches in elements.
+ *   CFP8_COMBINE_BF16_STEPS (weights bf16): every product and every partial sum is rounded to
+ *     bf16, starting from +0 -- bit for bit what GroupedExperts.forward accumulates with
+ *     `expert_out * weights[idx, top, None]` and `y.scatter_add_` on bf16 tensors when the slots
+ *     of a token are ordered by ascending expert id (the order of its loop over experts):
+ *     cosmos_rl/policy/kernel/moe/moe.py:240-262.
+ *   CFP8_COMBINE_F32 (weights bf16 or fp32): fp32 accumulator acc = fma(row, weight, acc), one
+ *     rounding at the end -- the arithmetic of the vendored Triton kernel
+ *     cosmos_rl/policy/kernel/megatron_moe/permutation.py:336-428 (whether its multiply and add
+ *     contract into an fma is the Triton compiler's choice; fma is assumed here). */
+#define CFP8_COMBINE_BF16_STEPS 0
+#define CFP8_COMBINE_F32 1
+int cfp8_combine_rows(const void* rows, int64_t ld_rows, int64_t num_rows, const int32_t* row_map,
+                      const void* weights, int weights_dtype, int64_t tokens, int topk, int64_t hidden,
+                      int mode, void* out, int64_t ld_out, void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */

@@ -45,6 +45,8 @@ def load() -> ctypes.CDLL:
         lib.fp8ref_silu32.restype = c_float
         lib.fp8ref_silu32.argtypes = [c_float]
         lib.fp8ref_swiglu.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
+        lib.fp8ref_combine_rows.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]
+        lib.fp8ref_combine_rows.restype = None
         lib.fp8ref_quant_tensorwise.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_block128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p]
         lib.fp8ref_quant_group128.argtypes = [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int]
@@ -84,6 +86,21 @@ def swiglu(g_u16: np.ndarray, u_u16: np.ndarray) -> np.ndarray:
 
 def swiglu_quant_group128(g_u16: np.ndarray, u_u16: np.ndarray):
     return quant_group128(swiglu(g_u16, u_u16), mode=0)
+
+
+def combine_rows(rows_u16: np.ndarray, row_map: np.ndarray, weights: np.ndarray, mode: int = 0) -> np.ndarray:
+    """out[t] = sum_s weights[t, s] * rows[row_map[t, s]] (slot order; < 0 skipped).  weights: uint16 view
+    of bf16, or float32 (mode 1 only).  mode 0: bf16 rounding at every step; 1: fp32 fma accumulator."""
+    rows = _u16(rows_u16)
+    rm = np.ascontiguousarray(row_map, dtype=np.int32)
+    T, topk = rm.shape
+    w = np.ascontiguousarray(weights)
+    assert w.shape == rm.shape and w.dtype in (np.uint16, np.float32)
+    out = np.empty((T, rows.shape[1]), np.uint16)
+    w16 = w.ctypes.data if w.dtype == np.uint16 else None
+    w32 = w.ctypes.data if w.dtype == np.float32 else None
+    load().fp8ref_combine_rows(rows.ctypes.data, rows.shape[1], rm.ctypes.data, w16, w32, T, topk, mode, out.ctypes.data)
+    return out
 
 
 def quant_rowwise(x_u16: np.ndarray):

@@ -235,6 +235,34 @@ void fp8ref_swiglu(const uint16_t* g, const uint16_t* u, int64_t n, uint16_t* h)
     }
 }
 
+/* Weighted combine of expert outputs into token order with bf16 rounding after every product and
+ * every partial sum, starting from +0: `y = zeros_like(x)`, then per expert (ascending)
+ * `y.scatter_add_(0, idx, expert_out * weights[idx, top, None])` on bf16 tensors,
+ * cosmos_rl/policy/kernel/moe/moe.py:240-262.  row_map [T, topk] lists each token's source rows in
+ * accumulation order (< 0: nothing).  mode 1: fp32 accumulator acc = fma(row, w, acc), one rounding
+ * (cosmos_rl/policy/kernel/megatron_moe/permutation.py:370-424; w is fp32 there). */
+void fp8ref_combine_rows(const uint16_t* rows, int64_t H, const int32_t* row_map, const uint16_t* w16, const float* w32,
+                         int64_t T, int64_t topk, int mode, uint16_t* out) {
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h) {
+            uint16_t y = 0;
+            float acc = 0.0f;
+            for (int64_t s = 0; s < topk; ++s) {
+                const int32_t r = row_map[t * topk + s];
+                if (r < 0) continue;
+                const float x = bf16_to_f32(rows[(int64_t)r * H + h]);
+                const float w = w32 ? w32[t * topk + s] : bf16_to_f32(w16[t * topk + s]);
+                if (mode == 0) {
+                    const uint16_t p = fp8ref_bf16_from_f32(x * w);
+                    y = fp8ref_bf16_from_f32(bf16_to_f32(y) + bf16_to_f32(p));
+                } else {
+                    acc = fmaf(x, w, acc);
+                }
+            }
+            out[t * H + h] = mode == 0 ? y : fp8ref_bf16_from_f32(acc);
+        }
+}
+
 /* Division shortcut used by the kernels: r = 1/s (IEEE), q0 = x*r,
  * e = fma(-q0, s, x), q1 = copysign(fma(e, r, q0), x).  Returns the number of (x, s) pairs,
  * x over all 65536 bf16 patterns with |x| <= amax(s) := 448*s-ish bound lifted

@@ -7,6 +7,11 @@ cases the reference's own self-tests use (:225-261 all counts 4, alignment 32; :
 [4,0,2,3,1,0,0,5], alignment 8, with their assertions: sizes are multiples of the alignment, an expert
 without tokens gets `alignment` slots all -1), by the worked example of the docstring (:166-171), and
 by ``brute_force`` below, which builds the same answer from explicit python lists with no prefix sums.
+
+``grouped_experts_combine`` restates the output side of ``GroupedExperts.forward``
+(cosmos_rl/policy/kernel/moe/moe.py:240-262) with the expert MLP replaced by given rows; it is pinned
+by the scalar C restatement ``fp8ref_combine_rows`` (explicit bf16 rounding of every product and partial
+sum, rounding by neighbour search in double arithmetic) in tests/test_moe_indices.py.
 """
 from __future__ import annotations
 
@@ -56,3 +61,20 @@ def brute_force(counts: List[int], experts_per_rank: int, num_ranks: int, alignm
         n = -(-n // alignment) * alignment
         out.extend(rows_of_expert[e] + [-1] * (n - len(rows_of_expert[e])))
     return out
+
+
+def grouped_experts_combine(expert_rows: List[torch.Tensor], token_mask: torch.Tensor, weights: torch.Tensor,
+                            indices: torch.Tensor, hidden: int) -> torch.Tensor:
+    """y [T, hidden] as GroupedExperts.forward builds it (moe.py:240-262), where expert_rows[i] stands for
+    ``swiglu(x_idx, ...)`` of expert i: one row per token routed to it, tokens in ascending order."""
+    T = indices.shape[0]
+    y = torch.zeros(T, hidden, dtype=expert_rows[0].dtype if expert_rows else weights.dtype)  # :240
+    for i in range(len(expert_rows)):                                                       # :243
+        indices_mask = torch.logical_and(indices == i, token_mask.unsqueeze(-1))           # :244
+        idx, top = torch.where(indices_mask)                                                # :245
+        if idx.numel() == 0:                                                                # :247
+            continue
+        idx_b = idx[:, None].expand(-1, hidden)                                             # :256
+        expert_out = expert_rows[i] * weights[idx, top, None]                               # :259-261
+        y.scatter_add_(dim=0, index=idx_b, src=expert_out)                                  # :263
+    return y

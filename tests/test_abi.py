@@ -37,6 +37,7 @@ def test_header_constants_match_binding():
     assert val("CFP8_GROUP_MODE_DIV") == _lib.GROUP_MODE_DIV and val("CFP8_GROUP_MODE_DEEPEP") == _lib.GROUP_MODE_DEEPEP
     assert val("CFP8_TENSORWISE_AMAX_SLOTS") == _lib.TENSORWISE_AMAX_SLOTS
     assert (val("CFP8_IN_BF16"), val("CFP8_IN_F16"), val("CFP8_IN_F32")) == (_lib.IN_BF16, _lib.IN_F16, _lib.IN_F32)
+    assert (val("CFP8_COMBINE_BF16_STEPS"), val("CFP8_COMBINE_F32")) == (_lib.COMBINE_BF16_STEPS, _lib.COMBINE_F32)
     assert ctypes.sizeof(_lib.TensorDesc) == 32
 
 
@@ -65,6 +66,15 @@ def test_argument_errors_need_no_device():
     assert "positive multiple of 128" in _lib.last_error()
     assert lib.cfp8_scaled_mm_rowwise(ptr, 1 << 24, ptr, ptr, 128, ptr, ptr, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert "supported range" in _lib.last_error()
+    # weighted combine: topk range, mode / dtype pairing, row width
+    assert lib.cfp8_combine_rows(ptr, 64, 4, ptr, ptr, _lib.IN_BF16, 4, 65, 64, 0, ptr, 64, None) == _lib.EINVAL
+    assert "topk" in _lib.last_error()
+    assert lib.cfp8_combine_rows(ptr, 64, 4, ptr, ptr, _lib.IN_F32, 4, 2, 64, _lib.COMBINE_BF16_STEPS, ptr, 64, None) == _lib.EINVAL
+    assert lib.cfp8_combine_rows(ptr, 64, 4, ptr, ptr, _lib.IN_F16, 4, 2, 64, _lib.COMBINE_F32, ptr, 64, None) == _lib.EINVAL
+    assert lib.cfp8_combine_rows(ptr, 60, 4, ptr, ptr, _lib.IN_BF16, 4, 2, 60, 0, ptr, 60, None) == _lib.EINVAL
+    assert lib.cfp8_combine_rows(ptr, 64, 4, ptr, ptr, _lib.IN_BF16, 4, 2, 64, 2, ptr, 64, None) == _lib.EINVAL
+    assert lib.cfp8_combine_rows(None, 64, 4, None, None, _lib.IN_BF16, 4, 2, 64, 0, None, 64, None) == _lib.EINVAL
+    assert lib.cfp8_combine_rows(None, 64, 0, None, None, _lib.IN_BF16, 0, 2, 64, 0, None, 64, None) == 0
     # empty problems succeed without pointers
     assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0

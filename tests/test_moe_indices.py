@@ -78,3 +78,167 @@ def test_permute_tokens_feeds_the_grouped_layout(dev):
     want = torch.zeros(want_idx.numel(), H, dtype=torch.bfloat16)
     want[want_idx >= 0] = x[want_idx[want_idx >= 0].long()]
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+# ---------------------------------------------------------------------------------------------
+# weighted combine of expert outputs (the output side of GroupedExperts.forward)
+# ---------------------------------------------------------------------------------------------
+def _same_bf16(a, b):
+    """bit-equal, except that a NaN matches any NaN: inf - inf has an unspecified sign and payload (x86 gives a
+    negative quiet NaN, the GPU a positive one, and torch's vector and scalar casts disagree as well)"""
+    a, b = a.cpu(), b.cpu()
+    na, nb = torch.isnan(a), torch.isnan(b)
+    return bool((na == nb).all()) and torch.equal(a.view(torch.int16)[~na], b.view(torch.int16)[~nb])
+
+
+def _routing_case(seed, T, K, E, H, mask_p=0.2):
+    g = torch.Generator().manual_seed(seed)
+    indices = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])      # distinct experts per token
+    token_mask = torch.rand(T, generator=g) >= mask_p
+    weights = torch.rand(T, K, generator=g).to(torch.bfloat16)
+    expert_rows = []
+    for i in range(E):
+        n = int(((indices == i) & token_mask[:, None]).sum())
+        r = torch.randn(n, H, generator=g)
+        r[torch.rand(n, H, generator=g) < 0.01] *= 1e-39                               # bf16 subnormals
+        r[torch.rand(n, H, generator=g) < 0.01] *= 3e38                                # overflow to infinity
+        expert_rows.append(r.to(torch.bfloat16))
+    return indices, token_mask, weights, expert_rows
+
+
+def _row_map_by_loops(indices, token_mask, expert_rows):
+    """rows of all experts stacked in expert order; row_map[t] = the token's rows by ascending expert, -1 filled"""
+    T, K = indices.shape
+    starts, n = [], 0
+    for r in expert_rows:
+        starts.append(n)
+        n += r.shape[0]
+    seen = [0] * len(expert_rows)
+    row_of = {}
+    for t in range(T):                      # tokens ascending inside an expert: the order torch.where gives
+        if not token_mask[t]:
+            continue
+        for k in range(K):
+            e = int(indices[t, k])
+            row_of[(t, k)] = starts[e] + seen[e]
+            seen[e] += 1
+    row_map = torch.full((T, K), -1, dtype=torch.int32)
+    w_order = torch.zeros((T, K), dtype=torch.int64)
+    for t in range(T):
+        slots = sorted(range(K), key=lambda k: int(indices[t, k]))
+        for j, k in enumerate(slots):
+            row_map[t, j] = row_of.get((t, k), -1)
+            w_order[t, j] = k
+    return torch.cat(expert_rows) if expert_rows else None, row_map, w_order
+
+
+def test_combine_oracle_pinned_by_scalar_restatement():
+    from oracle import c_oracle as CO
+    for seed, (T, K, E, H) in enumerate([(40, 4, 8, 16), (17, 8, 16, 24), (5, 1, 3, 8), (30, 2, 2, 8)]):
+        indices, token_mask, weights, expert_rows = _routing_case(seed, T, K, E, H)
+        want = MO.grouped_experts_combine(expert_rows, token_mask, weights, indices, H)
+        rows, row_map, w_order = _row_map_by_loops(indices, token_mask, expert_rows)
+        w = torch.gather(weights, 1, w_order)
+        got = CO.combine_rows(rows.view(torch.int16).numpy().view("uint16"), row_map.numpy(),
+                              w.view(torch.int16).numpy().view("uint16"), mode=0)
+        assert _same_bf16(torch.from_numpy(got.view("int16")).view(torch.bfloat16), want), seed
+
+
+def test_combine_closed_forms():
+    from oracle import c_oracle as CO
+    bf = lambda v: torch.tensor(v, dtype=torch.float32).to(torch.bfloat16)
+    one = bf([[1.0] * 8])
+    # one expert, weight 1: the row itself
+    rows = torch.randn(3, 8, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    y = MO.grouped_experts_combine([rows], torch.ones(3, dtype=torch.bool), torch.ones(3, 1, dtype=torch.bfloat16),
+                                   torch.zeros(3, 1, dtype=torch.int64), 8)
+    assert torch.equal(y, rows)
+    # the order of accumulation is the expert order: 1 + 2^-8 ties to 1 (twice), 2^-8 + 2^-8 + 1 = 1 + 2^-7
+    small = bf([[2.0 ** -8] * 8])
+    idx = torch.tensor([[0, 1, 2]])
+    m, w = torch.ones(1, dtype=torch.bool), torch.ones(1, 3, dtype=torch.bfloat16)
+    assert MO.grouped_experts_combine([one, small, small], m, w, idx, 8)[0, 0].item() == 1.0
+    assert MO.grouped_experts_combine([small, small, one], m, w, idx, 8)[0, 0].item() == 1.0 + 2.0 ** -7
+    # and the slot order of `indices` does not matter, only the expert ids do
+    assert MO.grouped_experts_combine([small, small, one], m, w, torch.tensor([[2, 0, 1]]), 8)[0, 0].item() == 1.0 + 2.0 ** -7
+    # the product is rounded before it is added: 1.5 * (1 + 2^-7) = 1.51171875 -> bf16 1.5078125 (tie to even)... checked in C
+    r = CO.combine_rows(bf([[1.0 + 2.0 ** -7] * 8]).view(torch.int16).numpy().view("uint16"), torch.tensor([[0]], dtype=torch.int32).numpy(),
+                        bf([[1.5]]).view(torch.int16).numpy().view("uint16"), mode=0)
+    want = (bf([1.0 + 2.0 ** -7]) * bf([1.5]))
+    assert int(r[0, 0]) == int(want.view(torch.int16).item()) & 0xFFFF
+    # fp32 mode: nothing is rounded until the end -> 1 + 2^-8 + 2^-8 = 1 + 2^-7 whatever the order
+    rows3 = torch.cat([one, small, small]).view(torch.int16).numpy().view("uint16")
+    r = CO.combine_rows(rows3, torch.tensor([[0, 1, 2]], dtype=torch.int32).numpy(),
+                        torch.ones(1, 3, dtype=torch.float32).numpy(), mode=1)
+    assert r[0, 0] == int(bf([1.0 + 2.0 ** -7]).view(torch.int16).item())
+    # a masked token stays zero
+    y = MO.grouped_experts_combine([one[:0], one[:0]], torch.zeros(1, dtype=torch.bool), torch.ones(1, 2, dtype=torch.bfloat16),
+                                   torch.tensor([[0, 1]]), 8)
+    assert torch.equal(y, torch.zeros(1, 8, dtype=torch.bfloat16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,K,E,H", [(300, 8, 16, 2048), (77, 4, 32, 264), (1, 1, 1, 8), (513, 6, 64, 7168), (64, 8, 8, 520)])
+def test_combine_rows_gpu_bit_exact(dev, T, K, E, H):
+    from oracle import c_oracle as CO
+    from cosmos_rl_amd.policy.kernel.moe.moe import TokenRouting, combine_expert_outputs
+    indices, token_mask, weights, expert_rows = _routing_case(T + H, T, K, E, H)
+    want = MO.grouped_experts_combine(expert_rows, token_mask, weights, indices, H)
+    rows, row_map, w_order = _row_map_by_loops(indices, token_mask, expert_rows)
+    routing = TokenRouting(None, row_map.to(dev), w_order.to(dev), None, None)
+    got = combine_expert_outputs(rows.to(dev), routing, weights.to(dev))
+    assert _same_bf16(got, want) and bool(torch.isnan(want).any()) == (H >= 264)  # the big cases do hit inf - inf
+    # fp32 accumulation, against the scalar restatement (small cases) and an fp64 sum (all)
+    for w in (weights, weights.float() * 1.37):
+        got32 = combine_expert_outputs(rows.to(dev), routing, w.to(dev), accumulate="fp32").cpu()
+        ws = torch.gather(w, 1, w_order)
+        if T * H <= 300 * 2048:
+            wn = ws.numpy() if ws.dtype == torch.float32 else ws.view(torch.int16).numpy().view("uint16")
+            ref = CO.combine_rows(rows.view(torch.int16).numpy().view("uint16"), row_map.numpy(), wn, mode=1)
+            assert _same_bf16(got32, torch.from_numpy(ref.view("int16")).view(torch.bfloat16))
+        safe = row_map.clamp_min(0).long()
+        terms = rows.double()[safe] * ws.double()[:, :, None] * (row_map >= 0)[:, :, None]
+        exact = terms.nan_to_num(0.0, 0.0, 0.0).sum(1)
+        fin = torch.isfinite(got32.double()) & torch.isfinite(terms).all(1) & (exact.abs() < 1e30)
+        err = (got32.double() - exact).abs()[fin]
+        assert bool((err <= exact.abs()[fin] * 2.0 ** -8 + terms.nan_to_num(0.0, 0.0, 0.0).abs().sum(1)[fin] * 2.0 ** -22).all())
+
+
+@pytest.mark.gpu
+def test_grouped_experts_forward_routes_and_combines(dev):
+    from cosmos_rl_amd.policy.kernel.moe.moe import grouped_experts_forward, route_tokens
+    T, K, E, H, al = 500, 4, 12, 256, 32
+    indices, token_mask, weights, _ = _routing_case(9, T, K, E, 8)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+
+    class PerExpertScale:  # stands for the expert MLP: expert e multiplies its rows by (e + 2) / 4
+        def execute(self, contig, m_sizes, m_offsets, module):
+            ends = m_offsets.cpu().tolist()
+            out = contig.clone()
+            for e in range(E):
+                s = ends[e] - int(m_sizes[e])
+                out[s:ends[e]] = contig[s:ends[e]] * ((e + 2) / 4)
+            return out
+
+    got = grouped_experts_forward(x.to(dev), token_mask.to(dev), weights.to(dev), indices.to(dev), PerExpertScale(), None, E, al)
+    expert_rows = []
+    for e in range(E):
+        idx, _top = torch.where((indices == e) & token_mask[:, None])
+        expert_rows.append(x[idx] * ((e + 2) / 4))
+    want = MO.grouped_experts_combine(expert_rows, token_mask, weights, indices, H)
+    assert torch.equal(got.cpu().view(torch.int16), want.view(torch.int16))
+    # the layout itself: every routed (token, expert) pair owns exactly one row of the expert's group
+    r = route_tokens(indices.to(dev), token_mask.to(dev), E, al)
+    ends = r.m_offsets.cpu().tolist()
+    sizes = r.m_sizes.cpu().tolist()
+    rt = r.row_tokens.cpu()
+    for e in range(E):
+        grp = rt[ends[e] - sizes[e]:ends[e]]
+        idx, _ = torch.where((indices == e) & token_mask[:, None])
+        assert grp[:idx.numel()].tolist() == idx.tolist() and bool((grp[idx.numel():] == -1).all())
+        assert sizes[e] % al == 0 and sizes[e] >= al
+    assert bool((rt[ends[-1]:] == -1).all())
+    # nobody routed: zeros
+    none = grouped_experts_forward(x.to(dev), torch.zeros(T, dtype=torch.bool, device=dev), weights.to(dev), indices.to(dev),
+                                   PerExpertScale(), None, E, al)
+    assert not bool(none.any())
