@@ -293,6 +293,15 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         del x, o, ws
     del qw3, sw3
 
+    # MXFP4 quantisation of the gate_up expert weights of GPT-OSS-20B: [32 experts x 5760, 2880]
+    RX, KX = 32 * 5760, 2880
+    wx = torch.empty(RX, KX, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+    qx = torch.empty(RX, KX // 2, dtype=torch.uint8, device=dev)
+    sx = torch.empty(RX, KX // 32, dtype=torch.uint8, device=dev)
+    hbm("mxfp4_gptoss20b_gate_up_%dx%d" % (RX, KX), RX * KX * 2 + RX * KX // 2 + RX * KX // 32,
+        lambda: check(lib.cfp8_quant_mxfp4(wx.data_ptr(), RX, KX, KX, qx.data_ptr(), KX // 2, sx.data_ptr(), KX // 32, stream)))
+    del wx, qx, sx
+
     # config 5: Qwen3-30B-A3B experts, 8192 tokens routed top-8 over 128 experts
     E, H, I, T, TOPK = 128, 2048, 768, 8192, 8
     wgu = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)

@@ -234,6 +234,21 @@ def swiglu_quant(gate: torch.Tensor, up: torch.Tensor) -> Tuple[torch.Tensor, to
     return q, s
 
 
+def quant_mxfp4(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """MXFP4 along the last axis of a bf16 tensor [..., K], K % 32 == 0: (uint8 [..., K/2] with two e2m1
+    codes per byte, even element low; uint8 [..., K/32] e8m0 scales)."""
+    _need_gpu(w)
+    if w.dtype != torch.bfloat16 or w.dim() < 1 or w.shape[-1] % 32:
+        raise ValueError(f"expected a bf16 tensor whose last dimension is a multiple of 32, got {tuple(w.shape)} {w.dtype}")
+    w = w.contiguous()
+    K = w.shape[-1]
+    rows = w.numel() // K if K else 0
+    q = torch.empty((*w.shape[:-1], K // 2), dtype=torch.uint8, device=w.device)
+    s = torch.empty((*w.shape[:-1], K // 32), dtype=torch.uint8, device=w.device)
+    _lib.check(_lib.load().cfp8_quant_mxfp4(w.data_ptr(), rows, K, K, q.data_ptr(), K // 2, s.data_ptr(), K // 32, _stream()))
+    return q, s
+
+
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """``per_token_cast_to_fp8`` of the reference's tests/test_deepep.py:75-85, including its
     formula ``x * (448 / amax.clamp(1e-4))`` with scales ``amax / 448``."""

@@ -185,6 +185,19 @@ int cfp8_combine_rows(const void* rows, int64_t ld_rows, int64_t num_rows, const
                       const void* weights, int weights_dtype, int64_t tokens, int topk, int64_t hidden,
                       int mode, void* out, int64_t ld_out, void* stream);
 
+/* MXFP4 quantisation of bf16 rows: every block of 32 consecutive elements of a row gets one
+ * e8m0 scale byte 2^ceil(log2(amax / 6)) and 32 e2m1 codes (round to nearest, ties away from zero),
+ * two per byte, even element in the low nibble.  q uint8 [rows, cols / 2] (pitch ld_q bytes,
+ * multiple of 4), scales uint8 [rows, cols / 32] (pitch ld_scales bytes), cols % 32 == 0, ld_x in
+ * elements (multiple of 8).  NaN / infinity inputs give unspecified codes.
+ * Replaces quantize_mx4 = triton_kernels' downcast_to_mxfp(w, torch.uint8, axis=1) at
+ * cosmos_rl/rollout/vllm_rollout/monkey_patch_for_mxfp4.py:18-24 together with the two transposes
+ * around it at cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:1018-1029 (blocks along the last
+ * axis of the [experts * out, in] weight); the engine-specific swizzle that follows there
+ * (:1037-1045) is not part of this call. */
+int cfp8_quant_mxfp4(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
+                     void* scales, int64_t ld_scales, void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */

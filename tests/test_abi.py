@@ -75,6 +75,11 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_combine_rows(ptr, 64, 4, ptr, ptr, _lib.IN_BF16, 4, 2, 64, 2, ptr, 64, None) == _lib.EINVAL
     assert lib.cfp8_combine_rows(None, 64, 4, None, None, _lib.IN_BF16, 4, 2, 64, 0, None, 64, None) == _lib.EINVAL
     assert lib.cfp8_combine_rows(None, 64, 0, None, None, _lib.IN_BF16, 0, 2, 64, 0, None, 64, None) == 0
+    assert lib.cfp8_quant_mxfp4(ptr, 4, 48, 48, ptr, 24, ptr, 2, None) == _lib.EINVAL     # cols % 32
+    assert "multiple of 32" in _lib.last_error()
+    assert lib.cfp8_quant_mxfp4(ptr, 4, 64, 64, ptr, 30, ptr, 2, None) == _lib.EINVAL     # q pitch
+    assert lib.cfp8_quant_mxfp4(None, 4, 64, 64, None, 32, None, 2, None) == _lib.EINVAL
+    assert lib.cfp8_quant_mxfp4(None, 0, 64, 64, None, 32, None, 2, None) == 0
     # empty problems succeed without pointers
     assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0
