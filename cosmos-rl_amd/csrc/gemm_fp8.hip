@@ -633,56 +633,60 @@ static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
 // ---------------------------------------------------------------------------
 // Rowwise GEMM for M <= 64 (decode-time batches): the 18944 x 3584 weight is read
 // once and nothing else matters, so the kernel is a weight streamer bounded by
-// HBM.  A workgroup of 8 waves owns 64 weight rows; wave (nt, kh) takes the 16
-// rows of n-tile nt and the kh-th half of every 512-byte K chunk, reads its
+// HBM.  A workgroup of 2 NTL waves owns 16 NTL weight rows; wave (nt, kh) takes the 16
+// rows of n-tile nt and the kh-th half of every chunk of KS K steps, reads its
 // weight fragments straight from global memory into MFMA operand registers
-// (streaming loads, two K steps ahead) and the activation fragments of the
+// (streaming loads, one chunk ahead) and the activation fragments of the
 // chunk from LDS, where the workgroup stages them once per chunk (activations of
 // 64 tokens are as many bytes per chunk as the workgroup's weights, so they must
 // not be re-read per wave).  The two K halves are summed through LDS at the end.
 // ---------------------------------------------------------------------------
-template <int TM, bool OUT_F32>
-__global__ __launch_bounds__(512) void gemm_rowwise_skinny_kernel(const GemmArgs p) {
-    constexpr int KS = 4;                         // K steps (of 128) per chunk
+template <int TM, int NTL, int KS, bool OUT_F32>
+__global__ __launch_bounds__(NTL * 128) void gemm_rowwise_skinny_kernel(const GemmArgs p) {
+    constexpr int NW = NTL * 2;                   // waves: NTL n-tiles x 2 K halves
+    constexpr int HS = KS / 2;                    // K steps per wave and chunk
+    constexpr int XU = KS * TM * 2;               // wave-wide loads that stage one chunk of activations
+    constexpr int XI = (XU + NW - 1) / NW;
     constexpr int XSTAGE = KS * TM * 2048;        // bytes of one activation stage
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int nt = wave & 3, kh = wave >> 2;
+    const int nt = wave % NTL, kh = wave / NTL;
     const int lrow = lane & 15, quarter = lane >> 4;
-    const int n0 = blockIdx.x * 64;
+    const int n0 = blockIdx.x * (NTL * 16);
     const int KT = p.K >> 7;
     const int chunks = (KT + KS - 1) / KS;
 
     // activation staging: one wave-wide load = 8 rows x 128 bytes of one K step
     const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
-    i32x4 xr[TM];
+    i32x4 xr[XI];
     auto xload = [&](int chunk) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int unit = wave + 8 * i, ks = unit & 3, row = (unit >> 2) * 8 + st_row8;
+        for (int i = 0; i < XI; ++i) {
+            const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
             const int kt = chunk * KS + ks;
-            const bool ok = row < p.M && kt < KT;
+            const bool ok = unit < XU && row < p.M && kt < KT;
             xr[i] = ok ? *reinterpret_cast<const i32x4*>(p.a + (int64_t)row * p.ld_a + ((int64_t)kt << 7) + st_c * 16)
                        : i32x4{0, 0, 0, 0};
         }
     };
     auto xstore = [&](int stage) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int unit = wave + 8 * i, ks = unit & 3, row = (unit >> 2) * 8 + st_row8;
-            *reinterpret_cast<i32x4*>(smem + stage * XSTAGE + (ks * TM + (row >> 4)) * 2048 + lds_chunk_offset(row & 15, st_c)) = xr[i];
+        for (int i = 0; i < XI; ++i) {
+            const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
+            if (XU % NW == 0 || unit < XU)
+                *reinterpret_cast<i32x4*>(smem + stage * XSTAGE + (ks * TM + (row >> 4)) * 2048 + lds_chunk_offset(row & 15, st_c)) = xr[i];
         }
     };
     // weight fragments: this wave's two K steps of a chunk, 32 contiguous bytes per lane and step
     const int wrow = n0 + nt * 16 + lrow;
     const bool wok = wrow < p.N;
     const uint8_t* wptr = p.b + (int64_t)(wok ? wrow : 0) * p.ld_b + quarter * 32;
-    i32x8 wf[2];
+    i32x8 wf[HS];
     auto wload = [&](int chunk) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int kt = chunk * KS + kh * 2 + h;
+        for (int h = 0; h < HS; ++h) {
+            const int kt = chunk * KS + kh * HS + h;
             if (wok && kt < KT) {
                 const u32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7)));
                 const u32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7) + 16));
@@ -705,14 +709,16 @@ __global__ __launch_bounds__(512) void gemm_rowwise_skinny_kernel(const GemmArgs
     __syncthreads();
     for (int c = 0; c < chunks; ++c) {
         const int cur = c & 1;
-        i32x8 wcur[2] = {wf[0], wf[1]};
+        i32x8 wcur[HS];
+#pragma unroll
+        for (int h = 0; h < HS; ++h) wcur[h] = wf[h];
         if (c + 1 < chunks) {
             xload(c + 1);
             wload(c + 1);
         }
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int ks = kh * 2 + h;
+        for (int h = 0; h < HS; ++h) {
+            const int ks = kh * HS + h;
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
                 const i32x8 fx = lds_frag(smem + cur * XSTAGE + (ks * TM + j) * 2048, lrow, quarter);
@@ -827,13 +833,39 @@ static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+template <int TM, int NTL>
+static int launch_rowwise_skinny_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
+    constexpr int KS = 8;
+    const int64_t blocks = (p.N + NTL * 16 - 1) / (NTL * 16);
+    constexpr size_t lds = (size_t)2 * KS * TM * 2048;   // >= the NTL * TM * 1 KiB of the final reduction
+    static_assert(lds >= (size_t)NTL * TM * 1024 && lds <= 160 * 1024, "skinny kernel LDS");
+    static std::atomic<bool> raised[65][2];
+    const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
+    const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_skinny_kernel<TM, NTL, KS, true>)
+                       : reinterpret_cast<const void*>(gemm_rowwise_skinny_kernel<TM, NTL, KS, false>);
+    const int slot = device_slot();
+    if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (v) hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, true>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
+    else hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, false>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
+    return check_launch("gemm");
+}
+
+// Rows of the weight per workgroup.  The kernel is bound by memory latency: a workgroup has one chunk of
+// 1 KiB per weight row in flight, so what counts is that all weight rows are resident at once - one
+// workgroup per CU (its two activation stages take most of the LDS), as close to 256 workgroups as the
+// row count allows.  Measured for 64 tokens on the 18944 x 3584 weight: 80 rows (237 workgroups) 24 us,
+// 64 rows (296, a second round on 40 CUs) 36 us, 96 rows (198) 26 us; on 3584 x 3584: 32 rows 15.5 us,
+// 80 rows 19.5 us.
 template <int TM>
 static int launch_rowwise_skinny(GemmArgs& p, int out_dtype, hipStream_t st) {
-    const int64_t blocks = (p.N + 63) / 64;
-    constexpr size_t lds = (size_t)2 * 4 * TM * 2048;   // >= the 4 * TM * 1 KiB of the final reduction
-    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, true>), dim3((unsigned)blocks), dim3(512), lds, st, p);
-    else hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, false>), dim3((unsigned)blocks), dim3(512), lds, st, p);
-    return check_launch("gemm");
+    const int64_t ntiles = (p.N + 15) / 16, per = (ntiles + 255) / 256;
+    if (per <= 2) return launch_rowwise_skinny_cfg<TM, 2>(p, out_dtype, st);
+    if (per == 3) return launch_rowwise_skinny_cfg<TM, 3>(p, out_dtype, st);
+    if (per == 4) return launch_rowwise_skinny_cfg<TM, 4>(p, out_dtype, st);
+    if (per == 6) return launch_rowwise_skinny_cfg<TM, 6>(p, out_dtype, st);
+    if (per == 7 || per == 8) return launch_rowwise_skinny_cfg<TM, 8>(p, out_dtype, st);
+    return launch_rowwise_skinny_cfg<TM, 5>(p, out_dtype, st);  // 5, and everything that takes several rounds anyway
 }
 
 template <int BM, int BN, int WM, int WN, int MODE>

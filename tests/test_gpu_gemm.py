@@ -46,7 +46,11 @@ def rowwise_operands(M, N, K, seed, dev):
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
                                    (2048, 8448, 256),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
-                                   (1000, 512, 384), (520, 256, 256)])
+                                   (1000, 512, 384), (520, 256, 256),
+                                   # 17..64 tokens: the weight streamer with 32, 48, 64, 80, 96 and 128 weight rows per
+                                   # workgroup (chosen from N), ragged last workgroup, K of 1, 3, 8 and 9 steps
+                                   (40, 528, 1152), (20, 8208, 128), (64, 12272, 384), (33, 16400, 1024), (64, 20016, 128),
+                                   (18, 24592, 256), (50, 28688, 128), (32, 40976, 128)])
 def test_scaled_mm_rowwise(dev, M, N, K):
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
     ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
