@@ -48,6 +48,7 @@ SIGNATURES = {
     "cfp8_scaled_mm_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                        c_int, c_int64, c_int64, c_int64, c_void_p]),
     "cfp8_linear_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "cfp8_linear_workspace_bytes_split": (c_size_t, [c_int64, c_int64, c_int64]),
     "cfp8_linear_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int,
                                     c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "cfp8_gemm_block128": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64,

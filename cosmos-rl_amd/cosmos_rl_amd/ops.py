@@ -329,7 +329,8 @@ def fp8_linear(x: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor
     lib = _lib.load()
     need = lib.cfp8_linear_workspace_bytes(M, K)
     if workspace is None or workspace.numel() * workspace.element_size() < need:
-        workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=x.device)
+        # the larger size lets the library split K where that pays (few weight rows, long K, 17..64 tokens)
+        workspace = torch.empty(max(lib.cfp8_linear_workspace_bytes_split(M, N, K), 256), dtype=torch.uint8, device=x.device)
     sw = weight_scale.reshape(-1)
     if sw.dtype != torch.float32 or not sw.is_contiguous():
         sw = sw.contiguous().float()

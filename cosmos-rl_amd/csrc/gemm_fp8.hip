@@ -41,6 +41,10 @@ struct GemmArgs {
     int64_t sb_stride_n, sb_stride_k, sb_stride_e;
     int M, N, K;
     int tiles_m, tiles_n;
+    // split-K (rowwise, at most 64 tokens): fp32 partial sums [k_slices, M, N] in caller-provided memory
+    float* partial;
+    size_t partial_bytes;
+    int k_slices, slice_steps;
 };
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int c) {
@@ -653,9 +657,12 @@ __global__ __launch_bounds__(NTL * 128) void gemm_rowwise_skinny_kernel(const Ge
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int nt = wave % NTL, kh = wave / NTL;
     const int lrow = lane & 15, quarter = lane >> 4;
-    const int n0 = blockIdx.x * (NTL * 16);
-    const int KT = p.K >> 7;
-    const int chunks = (KT + KS - 1) / KS;
+    // K slices of one n-block are neighbours in the grid; slice s covers K steps [kt0, KT)
+    const int slice = p.k_slices > 1 ? (int)(blockIdx.x % (unsigned)p.k_slices) : 0;
+    const int n0 = (p.k_slices > 1 ? (int)(blockIdx.x / (unsigned)p.k_slices) : (int)blockIdx.x) * (NTL * 16);
+    const int kt0 = slice * p.slice_steps;
+    const int KT = p.k_slices > 1 ? ((p.K >> 7) < kt0 + p.slice_steps ? (p.K >> 7) : kt0 + p.slice_steps) : (p.K >> 7);
+    const int chunks = (KT - kt0 + KS - 1) / KS;
 
     // activation staging: one wave-wide load = 8 rows x 128 bytes of one K step
     const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
@@ -664,7 +671,7 @@ __global__ __launch_bounds__(NTL * 128) void gemm_rowwise_skinny_kernel(const Ge
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
-            const int kt = chunk * KS + ks;
+            const int kt = kt0 + chunk * KS + ks;
             const bool ok = unit < XU && row < p.M && kt < KT;
             xr[i] = ok ? *reinterpret_cast<const i32x4*>(p.a + (int64_t)row * p.ld_a + ((int64_t)kt << 7) + st_c * 16)
                        : i32x4{0, 0, 0, 0};
@@ -686,7 +693,7 @@ __global__ __launch_bounds__(NTL * 128) void gemm_rowwise_skinny_kernel(const Ge
     auto wload = [&](int chunk) {
 #pragma unroll
         for (int h = 0; h < HS; ++h) {
-            const int kt = chunk * KS + kh * HS + h;
+            const int kt = kt0 + chunk * KS + kh * HS + h;
             if (wok && kt < KT) {
                 const u32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7)));
                 const u32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + ((int64_t)kt << 7) + 16));
@@ -738,7 +745,20 @@ __global__ __launch_bounds__(NTL * 128) void gemm_rowwise_skinny_kernel(const Ge
     __syncthreads();
     if (kh == 0) {
         const int n = n0 + nt * 16 + quarter * 4;
-        if (n < p.N) {
+        if (n < p.N && p.k_slices > 1) {
+            // a K slice: the unscaled sums go to this slice's plane of the partial buffer
+            float* const plane = p.partial + (int64_t)slice * p.M * p.N;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int m = j * 16 + lrow;
+                if (m >= p.M) continue;
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + ((nt * TM + j) * 64 + lane) * 4);
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[j][e] + o[e];
+                *reinterpret_cast<f32x4*>(plane + (int64_t)m * p.N + n) = v;
+            }
+        } else if (n < p.N) {
             const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
@@ -833,10 +853,34 @@ static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// Sum of the K slices in slice order, scales, conversion: out[m, n] = (sum_s partial[s, m, n]) * sa[m] * sb[n]
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int M, int N,
+                                                            const float* __restrict__ sa, const float* __restrict__ sb,
+                                                            void* __restrict__ out, int64_t ld_out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one thread per 4 consecutive columns
+    const int nq = N >> 2;
+    if (i >= (int64_t)M * nq) return;
+    const int m = (int)(i / nq), n = (int)(i - (int64_t)m * nq) * 4;
+    f32x4 v = *reinterpret_cast<const f32x4*>(partial + (int64_t)m * N + n);
+    for (int s = 1; s < slices; ++s) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(partial + ((int64_t)s * M + m) * N + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += o[e];
+    }
+    const float sam = sa[m];
+    const f32x4 sbn = *reinterpret_cast<const f32x4*>(sb + n);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = v[e] * sam * sbn[e];
+    if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(out) + (int64_t)m * ld_out + n) = v;
+    else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(out) + (int64_t)m * ld_out + n) =
+            make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+}
+
 template <int TM, int NTL>
 static int launch_rowwise_skinny_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     constexpr int KS = 8;
-    const int64_t blocks = (p.N + NTL * 16 - 1) / (NTL * 16);
+    const int64_t blocks = (p.N + NTL * 16 - 1) / (NTL * 16) * (p.k_slices > 1 ? p.k_slices : 1);
     constexpr size_t lds = (size_t)2 * KS * TM * 2048;   // >= the NTL * TM * 1 KiB of the final reduction
     static_assert(lds >= (size_t)NTL * TM * 1024 && lds <= 160 * 1024, "skinny kernel LDS");
     static std::atomic<bool> raised[65][2];
@@ -848,7 +892,28 @@ static int launch_rowwise_skinny_cfg(GemmArgs& p, int out_dtype, hipStream_t st)
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
     if (v) hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, true>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
     else hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, false>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
+    if (p.k_slices > 1) {
+        const unsigned rb = (unsigned)(((int64_t)p.M * (p.N >> 2) + 255) / 256);
+        if (v) hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3(rb), dim3(256), 0, st, p.partial, p.k_slices, p.M, p.N, p.sa, p.sb, p.out, p.ld_out);
+        else hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3(rb), dim3(256), 0, st, p.partial, p.k_slices, p.M, p.N, p.sa, p.sb, p.out, p.ld_out);
+    }
     return check_launch("gemm");
+}
+
+// K slices for a weight with few rows and a long K (e.g. a down projection): with at most 256 n-tiles there
+// are too few workgroups to pull the weight at memory speed, so K is cut into up to kMaxSlices slices of at
+// least 7 steps, each slice a workgroup, as many as fit one round of 256.  Needs room for the partial sums.
+constexpr int kMaxSlices = 8;
+static int pick_k_slices(const GemmArgs& p, int ntl) {
+    const int64_t ntiles = (p.N + 15) / 16;
+    if (!p.partial || ntiles > 256 || p.N % 4) return 1;
+    const int64_t nb = (ntiles + ntl - 1) / ntl;
+    const int kt = p.K >> 7;
+    int64_t s = 256 / nb;
+    if (s > kt / 7) s = kt / 7;
+    if (s > kMaxSlices) s = kMaxSlices;
+    if (s < 2 || (size_t)s * (size_t)p.M * (size_t)p.N * 4 > p.partial_bytes) return 1;
+    return (int)s;
 }
 
 // Rows of the weight per workgroup.  The kernel is bound by memory latency: a workgroup has one chunk of
@@ -860,6 +925,12 @@ static int launch_rowwise_skinny_cfg(GemmArgs& p, int out_dtype, hipStream_t st)
 template <int TM>
 static int launch_rowwise_skinny(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int64_t ntiles = (p.N + 15) / 16, per = (ntiles + 255) / 256;
+    p.k_slices = pick_k_slices(p, 4);
+    if (p.k_slices > 1) {
+        const int kt = p.K >> 7;
+        p.slice_steps = (kt + p.k_slices - 1) / p.k_slices;
+        return launch_rowwise_skinny_cfg<TM, 4>(p, out_dtype, st);
+    }
     if (per <= 2) return launch_rowwise_skinny_cfg<TM, 2>(p, out_dtype, st);
     if (per == 3) return launch_rowwise_skinny_cfg<TM, 3>(p, out_dtype, st);
     if (per == 4) return launch_rowwise_skinny_cfg<TM, 4>(p, out_dtype, st);
@@ -1005,6 +1076,12 @@ extern "C" size_t cfp8_linear_workspace_bytes(int64_t M, int64_t K) {
     return q + (((size_t)M * 4 + 255) & ~(size_t)255);
 }
 
+extern "C" size_t cfp8_linear_workspace_bytes_split(int64_t M, int64_t N, int64_t K) {
+    const size_t base = cfp8_linear_workspace_bytes(M, K);
+    if (base == 0 || N <= 0 || M <= 16 || M > 64 || (N + 15) / 16 > 256 || N % 4 || (K >> 7) < 14) return base;
+    return base + (size_t)cfp8::kMaxSlices * (size_t)M * (size_t)N * 4;
+}
+
 extern "C" int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, int64_t ld_w, const float* w_scale,
                                    void* out, int64_t ld_out, int out_dtype, int64_t M, int64_t N, int64_t K,
                                    void* workspace, size_t workspace_bytes, void* stream) {
@@ -1029,6 +1106,10 @@ extern "C" int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, i
     p.out = out;
     p.ld_a = K; p.ld_b = ld_w; p.ld_out = ld_out;
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    // what the workspace holds beyond the quantised activation is room for split-K partial sums
+    const size_t base = cfp8_linear_workspace_bytes(M, K);
+    p.partial = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + base);
+    p.partial_bytes = workspace_bytes - base;
     return launch_gemm<kRowwise>(p, out_dtype, st);
 }
 

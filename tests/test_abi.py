@@ -95,6 +95,11 @@ def test_linear_workspace_bytes():
     assert lib.cfp8_linear_workspace_bytes(0, 128) == 0
     n = lib.cfp8_linear_workspace_bytes(64, 3584)
     assert n >= 64 * 3584 + 64 * 4 and n % 256 == 0
+    # the split-K size adds room for partial sums only where the library would split: 17..64 tokens, at most
+    # 4096 weight rows, K of at least 14 steps
+    assert lib.cfp8_linear_workspace_bytes_split(64, 3584, 18944) == lib.cfp8_linear_workspace_bytes(64, 18944) + 8 * 64 * 3584 * 4
+    for M, N, K in [(16, 3584, 18944), (65, 3584, 18944), (64, 18944, 3584), (64, 3584, 1024), (0, 64, 128)]:
+        assert lib.cfp8_linear_workspace_bytes_split(M, N, K) == lib.cfp8_linear_workspace_bytes(M, K)
     # too small a workspace is an error code of its own
     rc = lib.cfp8_linear_rowwise(None, 3584, None, 3584, None, None, 64, 0, 64, 64, 3584, None, 0, None)
     assert rc == _lib.EWORKSPACE

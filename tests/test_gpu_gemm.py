@@ -106,6 +106,28 @@ def test_fp8_linear_cfg3_shapes(dev, M):
         assert torch.equal(o3.view(M, N), out16 + bias.to(dev))
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 3584, 18944), (17, 4096, 1792), (40, 528, 7168), (33, 2064, 3584), (64, 1024, 896)])
+def test_fp8_linear_split_k(dev, M, N, K):
+    """Few weight rows, long K, 17..64 tokens: with the larger workspace the call cuts K into slices (fp32 partial
+    sums, summed in slice order by a second launch); with the minimal workspace it does not.  Both meet the GEMM
+    bar, and they agree to fp32 summation order."""
+    from cosmos_rl_amd import _lib
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=7 + M + N, dev=dev)
+    ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
+    lib = _lib.load()
+    small = torch.empty(lib.cfp8_linear_workspace_bytes(M, K), dtype=torch.uint8, device=dev)
+    big_n = lib.cfp8_linear_workspace_bytes_split(M, N, K)
+    assert (big_n > small.numel()) == (K >= 1792)
+    y_split = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)          # allocates the larger one
+    y_plain = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32, workspace=small)
+    for y in (y_split, y_plain):
+        assert O.rel_frobenius(y.cpu(), ref) <= TIGHT
+    assert O.rel_frobenius(y_split.cpu(), y_plain.cpu()) <= 1e-6
+    if K >= 1792:
+        assert not torch.equal(y_split, y_plain) or K == 1792   # a different summation order shows in the last bits
+    check_bf16(ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev)), ref, f"split-K linear {M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (2, 272, 896), (3, 1024, 3584), (4, 48, 8320), (4, 18944, 3584)])
 def test_fp8_linear_small_m(dev, M, N, K):
     """Decode shapes: cfp8_linear_rowwise equals cfp8_scaled_mm_rowwise on separately quantised activations bit
