@@ -45,7 +45,8 @@ def route_tokens(indices: torch.Tensor, token_mask: Optional[torch.Tensor], n_ex
         idx64 = torch.where(token_mask.to(torch.bool).unsqueeze(-1), idx64, torch.full_like(idx64, n_experts))
     key = idx64.reshape(-1)                                   # masked slots fall into a bin past the last expert
     order = torch.argsort(key, stable=True)
-    counts = torch.bincount(key, minlength=n_experts + 1)[:n_experts]
+    # (torch.bincount reads its result size back from the device; a scatter-add does not, so this can be graph-captured)
+    counts = torch.zeros(n_experts + 1, dtype=torch.int64, device=dev).scatter_add_(0, key, torch.ones_like(key))[:n_experts]
     capacity = int(max_rows) if max_rows is not None else T * K + n_experts * alignment
     permuted, m_sizes, m_offsets = generate_permute_indices(counts, n_experts, 1, alignment, max_len=capacity)
     valid_row = permuted >= 0
@@ -54,7 +55,7 @@ def route_tokens(indices: torch.Tensor, token_mask: Optional[torch.Tensor], n_ex
     row_of_slot = torch.full((T * K + 1,), -1, dtype=torch.int32, device=dev)
     row_of_slot.scatter_(0, torch.where(valid_row, src_slot, torch.full_like(src_slot, T * K)),
                          torch.arange(capacity, dtype=torch.int32, device=dev))
-    row_of_slot[T * K] = -1
+    row_of_slot[T * K:].fill_(-1)                             # the slot that caught the padding rows
     _, slot_order = torch.sort(idx64, dim=1, stable=True)
     row_map = torch.gather(row_of_slot[:T * K].view(T, K), 1, slot_order).contiguous()
     return TokenRouting(row_tokens, row_map, slot_order, m_sizes, m_offsets)
