@@ -187,9 +187,21 @@ def main() -> int:
     return 0
 
 
+WARM_SECONDS = 0.15
+
+
 def _time_events(torch, fn, warmup, iters, flush=None):
-    for _ in range(warmup):
+    # The GPU raises its shader clock over the first ~25 ms of sustained load (an MFMA-bound kernel runs 20 %
+    # slower at the start of that ramp), so warm up for a stretch of wall time, not just a count of calls,
+    # with the same call / flush pattern as the timed loop.
+    t0, n = time.perf_counter(), 0
+    while n < warmup or time.perf_counter() - t0 < WARM_SECONDS:
+        if flush is not None:
+            flush.add_(1)
         fn()
+        n += 1
+        if n % 10 == 0:
+            torch.cuda.synchronize()
     times = []
     for _ in range(iters):
         if flush is not None:
