@@ -602,6 +602,280 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Block-scaled and grouped GEMM, full tiles: 256 x 128 (block) or 128 x 256 (grouped, whose groups are
+// 128 rows) x 128 per workgroup, eight wavefronts (two per SIMD), each a 64 x 64 block = 4 x tiles
+// times 4 w tiles.  One wave keeps only one LDS instruction in progress at a time, so the K step is
+// laid out around its LDS queue:
+//
+//   group 0: read x2 | 3 LDS stores of tile kt+1 | per w tile i: rescale of last step's (i, x2), MFMA (i, x0)
+//   group 1: read x3 | 3 LDS stores, 3 global loads of tile kt+2 | per i: rescale of last step's (i, x3), MFMA (i, x1)
+//   wait for own LDS traffic, barrier: stage nxt complete, stage cur free
+//   tail:    next step's x0 | 3 global loads | per i: rescale of (i, x0), (i, x1), MFMAs (i, x2), (i, x3),
+//            then next step's w tile i into the registers those MFMAs just consumed; next step's x1 and scales
+//
+// No MFMA after the barrier waits for LDS, every rescale (acc += products * s_m * s_n, VALU) reads MFMA
+// results issued at least five MFMAs earlier, and the first MFMAs of a step find their fragments read
+// during the previous tail.  Activation scales reach LDS eight K steps at a time (turned to [step][row]),
+// the tile's weight scales once in the prologue.  Requires M % BM == 0, N % BN == 0 and
+// K / 128 * (BN / 128) <= kMaxTileWeightScales.
+// ---------------------------------------------------------------------------
+constexpr int kMaxTileWeightScales = 2048;
+
+template <int BM, int BN, int MODE, bool OUT_F32, bool SCALE_VEC>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8_kernel(const GemmArgs p) {
+    static_assert((BM == 256 && BN == 128) || (BM == 128 && BN == 256), "eight 64 x 64 wave tiles");
+    static_assert(MODE == kBlock || MODE == kGrouped, "block-scaled modes only");
+    constexpr int WM = BM / 64;
+    constexpr int STAGE = (BM + BN) * 128;  // 48 KiB
+    constexpr int A_IT = BM / 64, B_IT = BN / 64;  // wave-wide loads (8 rows x 128 B) per wave and K step: 4 + 2 or 2 + 4
+    constexpr int NB = BN / 128;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const uint8_t* bptr = p.b;
+    const float* sbp = p.sb;
+    int expert = 0;
+    if (MODE == kGrouped) {
+        expert = p.m_indices[m0];  // groups start on multiples of 128 = BM rows
+        if (expert < 0) return;    // a tile of padding (uniform for the workgroup)
+        bptr += (int64_t)expert * p.N * p.ld_b;
+        sbp += (int64_t)expert * p.sb_stride_e;
+    }
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+
+    // global -> registers -> LDS: wave w takes the 16-row blocks (w >> 1) + 4 i of each operand, the half (w & 1) of them
+    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_b;
+    uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
+    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));  // keep them in SGPRs for the whole loop
+    const uint32_t va_lane = (uint32_t)((wave & 1) * 8 + st_row8) * (uint32_t)p.ld_a + (uint32_t)(st_c * 16);
+    const uint32_t vb_lane = (uint32_t)((wave & 1) * 8 + st_row8) * (uint32_t)p.ld_b + (uint32_t)(st_c * 16);
+    const int l_lane = lds_chunk_offset((wave & 1) * 8 + st_row8, st_c) + (wave >> 1) * 2048;
+    i32x4 R[6];
+    auto gload = [&](int kt, int i) {
+        const uint64_t base = (i < A_IT ? a_wave + (uint64_t)i * a_step : b_wave + (uint64_t)(i - A_IT) * b_step) + ((uint64_t)kt << 7);
+        typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+        typedef const __attribute__((address_space(1))) i32x4* gvec_t;
+        R[i] = *(gvec_t)((gptr_t)base + (i < A_IT ? va_lane : vb_lane));
+    };
+    auto lstore = [&](int stage, int i) {
+        *reinterpret_cast<i32x4*>(smem + stage * STAGE + (i < A_IT ? i * 8192 : BM * 128 + (i - A_IT) * 8192) + l_lane) = R[i];
+    };
+
+    // activation scales: 8 K steps of this tile's rows per fetch, 4 consecutive floats per thread
+    float* const sg_buf = reinterpret_cast<float*>(smem + 2 * STAGE);  // [2][8][BM]
+    float* const sn_lds = sg_buf + 2 * 8 * BM;                         // [KT][NB]
+    const int sg_row = t >> 1, sg_half = t & 1;
+    const float* const sg_ptr = p.sa + (int64_t)(m0 + (sg_row < BM ? sg_row : BM - 1)) * KT;
+    f32x4 sg = {0.f, 0.f, 0.f, 0.f};
+    auto sg_load = [&](int g) {
+        const int k0 = 8 * g + 4 * sg_half;
+        if (SCALE_VEC) {
+            sg = *reinterpret_cast<const f32x4*>(sg_ptr + (k0 + 4 <= KT ? k0 : KT - 4));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sg[e] = sg_ptr[(k0 + e) < KT ? (k0 + e) : (KT - 1)];
+        }
+    };
+    auto sg_store = [&](int g) {
+        if (BM == 256 || sg_row < BM) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sg_buf[((g & 1) * 8 + 4 * sg_half + e) * BM + sg_row] = sg[e];
+        }
+    };
+
+    f32x4 acc[4][4], P[2][4];  // [w tile][x tile]; raw products of two x tiles
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        P[0][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        P[1][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int x_off = lds_chunk_offset(wm * 64 + lrow, 2 * quarter);
+    const int x_off2 = lds_chunk_offset(wm * 64 + lrow, 2 * quarter + 1);
+    const int w_off = BM * 128 + lds_chunk_offset(wn * 64 + lrow, 2 * quarter);
+    const int w_off2 = BM * 128 + lds_chunk_offset(wn * 64 + lrow, 2 * quarter + 1);
+    auto frag = [&](int stage, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage * STAGE + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+    i32x8 W[4], X[4];
+    float sm[4], s_n;
+    auto read_scales = [&](int kt) {  // s_m of this wave's four x tiles and s_n of its weight block for K step kt
+        const int k = kt < last ? kt : last;
+        const float* const sgk = sg_buf + (((k >> 3) & 1) * 8 + (k & 7)) * BM + wm * 64 + lrow;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sm[j] = sgk[j * 16];
+        s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
+    };
+
+    // prologue: scales, then tiles 0 and 1 requested together; tile 0 goes to stage 0, tile 1 stays in R
+    sg_load(0);
+    for (int idx = t; idx < KT * NB; idx += 512) {
+        const int k = idx / NB, nb = idx - k * NB;
+        sn_lds[idx] = sbp[(int64_t)((n0 >> 7) + nb) * p.sb_stride_n + (int64_t)k * p.sb_stride_k];
+    }
+    {
+        i32x4 T0[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            gload(0, i);
+            T0[i] = R[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 6; ++i) gload(1 < last ? 1 : last, i);
+        CFP8_PHASE_END();
+        sg_store(0);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            const i32x4 keep = R[i];
+            R[i] = T0[i];
+            lstore(0, i);
+            R[i] = keep;
+        }
+    }
+    __syncthreads();
+    // (the same order as in the loop's tail: the compiler merges both when it counts outstanding reads at the loop head)
+    X[0] = frag(0, x_off, x_off2, 0);
+    CFP8_PHASE_END();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        W[i] = frag(0, w_off, w_off2, i);
+        CFP8_PHASE_END();
+    }
+    X[1] = frag(0, x_off, x_off2, 1);
+    read_scales(0);
+    CFP8_PHASE_END();
+    float sc2p = 0.f, sc3p = 0.f;  // scales of the products still waiting in P from the previous step
+
+#define CFP8_RESCALE(i, j, pj, sc)                                                                   \
+    _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(P[pj][i][e], sc, acc[i][j][e])
+#define CFP8_PRODUCT(i, j, pj) \
+    P[pj][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[j], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0)
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1, nxt = cur ^ 1;
+        const int kl = kt + 2 < last ? kt + 2 : last;  // past the end: re-read the last tile, never consumed
+        // group 0
+        X[2] = frag(cur, x_off, x_off2, 2);
+        lstore(nxt, 0);
+        lstore(nxt, 1);
+        lstore(nxt, 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            CFP8_RESCALE(i, 2, 0, sc2p);
+            CFP8_PRODUCT(i, 0, 0);
+        }
+        CFP8_PHASE_END();
+        // group 1
+        X[3] = frag(cur, x_off, x_off2, 3);
+        lstore(nxt, 3);
+        lstore(nxt, 4);
+        lstore(nxt, 5);
+        gload(kl, 0);
+        gload(kl, 1);
+        gload(kl, 2);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            CFP8_RESCALE(i, 3, 1, sc3p);
+            CFP8_PRODUCT(i, 1, 1);
+        }
+        if ((kt & 7) == 7) sg_store((kt >> 3) + 1);
+        CFP8_PHASE_END();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        CFP8_PHASE_END();
+        // tail
+        const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
+        sc2p = sm[2] * s_n;
+        sc3p = sm[3] * s_n;
+        X[0] = frag(nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
+        gload(kl, 3);
+        gload(kl, 4);
+        gload(kl, 5);
+        if ((kt & 7) == 6) sg_load((kt >> 3) + 1);
+        CFP8_PHASE_END();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            CFP8_RESCALE(i, 0, 0, sc0);
+            CFP8_RESCALE(i, 1, 1, sc1);
+            CFP8_PRODUCT(i, 2, 0);
+            CFP8_PRODUCT(i, 3, 1);
+            CFP8_PHASE_END();
+            W[i] = frag(nxt, w_off, w_off2, i);
+            CFP8_PHASE_END();
+        }
+        X[1] = frag(nxt, x_off, x_off2, 1);
+        read_scales(kt + 1);
+        CFP8_PHASE_END();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        CFP8_RESCALE(i, 2, 0, sc2p);
+        CFP8_RESCALE(i, 3, 1, sc3p);
+    }
+#undef CFP8_RESCALE
+#undef CFP8_PRODUCT
+
+    // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+    if (OUT_F32) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + wm * 64 + j * 16 + lrow;
+            if (MODE == kGrouped && p.m_indices[m] != expert) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + wn * 64 + i * 16 + quarter * 4;
+                __builtin_nontemporal_store(acc[i][j], reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: turn the wave's 64 x 64 block through LDS in two halves of 32 rows (row stride 144 B), so that
+    // global stores are 16 bytes per lane and 128 contiguous bytes per row, non-temporal
+    __syncthreads();  // all waves are done reading the operand stages
+    constexpr int EST = 144;
+    uint8_t* const ebuf = smem + wave * (32 * EST);
+    const int rd_row = lane >> 3, rd_chunk = lane & 7;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = h * 2 + jj;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 v = acc[i][j];
+                *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = r * 8 + rd_row;  // 0..31 within the half
+            const int m = m0 + wm * 64 + h * 32 + row;
+            if (MODE == kGrouped && p.m_indices[m] != expert) continue;
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            __builtin_nontemporal_store(
+                d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
+        }
+    }
+}
+
 // Kernels that use more than 64 KiB of LDS need the limit raised once per device and function.
 // `flag` is that (device, function) pair's once-flag; a race on the first call raises it twice, harmlessly.
 static int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag) {
@@ -965,11 +1239,37 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+template <int BM, int BN, int MODE>
+static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / BM;
+    p.tiles_n = p.N / BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    // two operand stages, the turned activation scales of two groups of 8 K steps, the tile's weight scales
+    const size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
+    const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    using Kern = void (*)(const GemmArgs);
+    const Kern table[2][2] = {{gemm_block_w8_kernel<BM, BN, MODE, false, false>, gemm_block_w8_kernel<BM, BN, MODE, true, false>},
+                              {gemm_block_w8_kernel<BM, BN, MODE, false, true>, gemm_block_w8_kernel<BM, BN, MODE, true, true>}};
+    const int f32 = out_dtype == CFP8_OUT_F32;
+    const Kern kern = table[vec][f32];
+    // the limit is raised to the largest size this kernel can ask for, once per device and instantiation
+    constexpr size_t lds_max = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
+    static std::atomic<bool> done[65][2][2];  // zero-initialised
+    const int slot = device_slot();
+    if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec][f32])) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
+    return check_launch("gemm");
+}
+
 template <int MODE>
 static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) {
         // groups are 128-row aligned, so a tile is 128 rows; 256 columns per workgroup (8 waves) read a
         // quarter fewer operand bytes per flop than 128
+        if (p.M % 128 == 0 && p.N % 256 == 0 && (int64_t)(p.M / 128) * (p.N / 256) >= 384 && (p.K >> 7) * 2 <= kMaxTileWeightScales)
+            return launch_block_w8<128, 256, kGrouped>(p, out_dtype, st);
         if (p.N % 256 == 0 && (int64_t)((p.M + 127) / 128) * (p.N / 256) >= 384)
             return launch_cfg<128, 256, 2, 4, kGrouped>(p, out_dtype, st);
         return launch_cfg<128, 128, 2, 2, kGrouped>(p, out_dtype, st);
@@ -983,6 +1283,9 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     // block scaling, large M: one 8-wave workgroup per CU on a 256 x 128 tile reads a quarter fewer operand
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
+    if (MODE == kBlock && p.M > 512 && p.M % 256 == 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
+        (p.K >> 7) <= kMaxTileWeightScales)
+        return launch_block_w8<256, 128, kBlock>(p, out_dtype, st);
     if (MODE == kBlock && p.M > 512 && (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128) >= 384)
         return launch_cfg<256, 128, 4, 2, kBlock>(p, out_dtype, st);
     // measured on config 3 (N = 18944, K = 3584): 129..256 rows run 10 % faster as one 256 x 128 tile-row,

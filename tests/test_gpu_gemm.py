@@ -179,7 +179,9 @@ def block_operands(M, N, K, seed):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 128, 256), (70, 208, 384), (128, 256, 1024), (300, 512, 768),
-                                   (640, 1536, 2048), (1000, 12288, 384), (1024, 12288, 512)])
+                                   (640, 1536, 2048), (1000, 12288, 384), (1024, 12288, 512),
+                                   # full 256 x 128 tiles, >= 384 of them (the eight-wave kernel): K of 5, 1, 9 and 17 steps
+                                   (1024, 12288, 640), (768, 16384, 128), (1024, 12416, 1152), (1280, 10240, 2176)])
 def test_gemm_block128(dev, M, N, K):
     # the last two shapes have >= 384 tiles of 256 x 128 and take the 8-wave 256 x 128 kernel: one with a
     # ragged last tile-row and K/128 not a multiple of 4 (scalar scale loads), one with 16-byte scale loads
@@ -236,11 +238,13 @@ def test_gemm_block128_cfg4_properties(dev):
 
 
 # ---------------------------------------------------------------------------- grouped
-@pytest.mark.parametrize("T,E,K,N,topk", [(300, 7, 512, 384, 2), (2600, 7, 384, 2048, 2)])
+@pytest.mark.parametrize("T,E,K,N,topk", [(300, 7, 512, 384, 2), (2600, 7, 384, 2048, 2), (3300, 7, 1152, 2048, 2), (3300, 7, 1024, 1792, 2),
+                                          (3300, 7, 128, 2048, 2)])
 def test_grouped_gemm(dev, T, E, K, N, topk):
     """Ragged groups: top-2 routing over 6 experts plus an empty expert, groups padded to 128 rows;
-    padding rows (index -1) must be left untouched.  The second shape has >= 384 tiles of 128 x 256
-    (the 8-wave grouped kernel) and K/128 not a multiple of 4."""
+    padding rows (index -1) must be left untouched.  The shapes with 3300 tokens have >= 384 tiles of
+    128 x 256 (the eight-wave kernel): K of 9 steps (more than one group of 8 activation-scale steps, scalar
+    scale loads), 8 steps (16-byte scale loads) with N = 7 * 256, and a single step."""
     g = torch.Generator().manual_seed(77)
     logits = torch.rand(T, E, generator=g)
     logits[:, 3] = -1.0  # expert 3 gets no token
