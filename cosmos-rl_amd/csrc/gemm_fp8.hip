@@ -1309,8 +1309,8 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     }
     if (p.M % 256 == 0 && p.N % 256 == 0 && out16) {
         // One workgroup per CU and equal tiles: the launch runs in rounds of 256 tiles, and a last round that is
-        // at most half full costs a whole round.  Then the last tile-columns go to a second launch on 256 x 128
-        // tiles (half the work per workgroup, 8 waves) and the first launch ends on a full round.
+        // at most half full costs a whole round.  Then the last tile-columns go to a second launch on smaller
+        // tiles and the first launch ends on a full round.
         const int64_t tm = p.M / 256, tn = p.N / 256, rem = (tm * tn) % 256;
         const int64_t cut = (rem + tm - 1) / tm;  // tile-columns that hold the partial round
         if (tm * tn > 256 && rem > 0 && rem <= 128 && cut < tn) {
@@ -1322,6 +1322,10 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
             tail.b = p.b + (int64_t)head.N * p.ld_b;
             tail.sb = p.sb + head.N;
             tail.out = static_cast<uint8_t*>(p.out) + (int64_t)head.N * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+            // few tail tiles: 128 x 128 tiles (4 waves, two workgroups per CU) spread them over more CUs
+            // (M = 1024: 40 tile-columns' worth as 160 workgroups 72 us in all, as 80 of 256 x 128 78 us;
+            // M = 2048: 320 against 160 workgroups, 125 against 122 us)
+            if (cut * tm * 4 <= 256) return launch_cfg<128, 128, 2, 2, kRowwise>(tail, out_dtype, st);
             return launch_cfg<256, 128, 4, 2, kRowwise>(tail, out_dtype, st);
         }
         return launch_rowwise_256(p, out_dtype, st);
