@@ -242,3 +242,33 @@ def test_grouped_experts_forward_routes_and_combines(dev):
     none = grouped_experts_forward(x.to(dev), torch.zeros(T, dtype=torch.bool, device=dev), weights.to(dev), indices.to(dev),
                                    PerExpertScale(), None, E, al)
     assert not bool(none.any())
+
+
+@pytest.mark.gpu
+def test_combine_rows_slot_limits(dev):
+    """64 slots per token (the most the kernel takes), no slot at all (zeros), and indices no source row has"""
+    from cosmos_rl_amd import _lib
+    from cosmos_rl_amd.policy.kernel.moe.moe import TokenRouting, combine_expert_outputs
+    from oracle import c_oracle as CO
+    g = torch.Generator().manual_seed(5)
+    T, K, H, R = 9, 64, 72, 700
+    rows = torch.randn(R, H, generator=g).to(torch.bfloat16)
+    row_map = torch.randint(-1, R, (T, K), generator=g, dtype=torch.int32)
+    w = torch.rand(T, K, generator=g).to(torch.bfloat16)
+    order = torch.arange(K).expand(T, K).contiguous()
+    want = CO.combine_rows(rows.view(torch.int16).numpy().view("uint16"), row_map.numpy(), w.view(torch.int16).numpy().view("uint16"), 0)
+    got = combine_expert_outputs(rows.to(dev), TokenRouting(None, row_map.to(dev), order.to(dev), None, None), w.to(dev))
+    assert _same_bf16(got, torch.from_numpy(want.view("int16")).view(torch.bfloat16))
+    # rows >= the number of source rows count as padding
+    rm2 = row_map.clone()
+    rm2[0, :5] = R + 3
+    want2 = row_map.clone()
+    want2[0, :5] = -1
+    ref2 = CO.combine_rows(rows.view(torch.int16).numpy().view("uint16"), want2.numpy(), w.view(torch.int16).numpy().view("uint16"), 0)
+    got2 = combine_expert_outputs(rows.to(dev), TokenRouting(None, rm2.to(dev), order.to(dev), None, None), w.to(dev))
+    assert _same_bf16(got2, torch.from_numpy(ref2.view("int16")).view(torch.bfloat16))
+    # no slot: zeros, and no pointer is needed for what is not read
+    out = torch.full((T, H), 3.0, dtype=torch.bfloat16, device=dev)
+    _lib.check(_lib.load().cfp8_combine_rows(None, H, 0, None, None, _lib.IN_BF16, T, 0, H, 0, out.data_ptr(), H,
+                                             torch.cuda.current_stream().cuda_stream))
+    assert not bool(out.any())
