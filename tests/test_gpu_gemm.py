@@ -128,11 +128,13 @@ def test_fp8_linear_split_k(dev, M, N, K):
     check_bf16(ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev)), ref, f"split-K linear {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (2, 272, 896), (3, 1024, 3584), (4, 48, 8320), (4, 18944, 3584)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (2, 272, 896), (3, 1024, 3584), (4, 48, 8320), (4, 18944, 3584), (1, 18944, 3584),
+                                   (2, 528, 4096), (4, 64, 4224), (5, 272, 896), (1, 16, 2048)])
 def test_fp8_linear_small_m(dev, M, N, K):
     """Decode shapes: cfp8_linear_rowwise equals cfp8_scaled_mm_rowwise on separately quantised activations bit
-    for bit; K > 4096 walks the K loop of the M <= 16 kernel more than once; a NaN token stays a NaN row and
-    leaves the others alone."""
+    for bit - up to 4 tokens and K <= 4096 it is one launch that quantises the tokens inside the GEMM kernel,
+    otherwise two; K > 4096 walks the K loop of the M <= 16 kernel more than once; a NaN token stays a NaN row
+    and leaves the others alone."""
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=99 + M + N, dev=dev)
     y = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32)
     qxd, sxd = ops.quant_rowwise(x.to(dev))
@@ -140,6 +142,12 @@ def test_fp8_linear_small_m(dev, M, N, K):
     assert torch.equal(y, y2)
     ref = O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)
     assert O.rel_frobenius(y.cpu(), ref) <= TIGHT
+    # a row pitch larger than K, and the bf16 epilogue
+    xp = torch.zeros(M, K + 64, dtype=torch.bfloat16, device=dev)
+    xp[:, :K] = x.to(dev)
+    assert torch.equal(ops.fp8_linear(xp[:, :K], f8(qw, dev).t(), sw.to(dev), out_dtype=torch.float32), y)
+    y16 = ops.fp8_linear(x.to(dev), f8(qw, dev).t(), sw.to(dev))
+    assert torch.equal(y16, ops.scaled_mm(qxd, f8(qw, dev).t(), sxd, sw.to(dev).t(), out_dtype=torch.bfloat16))
     if M > 1:
         xn = x.clone()
         xn[0, 5] = float("nan")
