@@ -246,6 +246,70 @@ def test_gemm_block128_cfg4_properties(dev):
 
 
 # ---------------------------------------------------------------------------- grouped
+def test_grouped_cfg5_full_size_properties(dev):
+    """Config 5 at full size: 8192 tokens routed top-8 over 128 experts (65536 rows, groups padded to 128), expert MLP
+    shapes [1536, 2048] and [2048, 768], through the host path of the reference (route -> gather -> DSGroupGEMM-style
+    chain -> combine).  Size-independent checks: padding rows stay untouched, sampled rows of both GEMMs against
+    the fp64 dequantised product, the fused SwiGLU quantiser against the unfused torch chain's bytes on a slice,
+    permuting the tokens of one expert permutes its output rows, and the combined output of a token whose 8 weights
+    are zero except one equals that expert's row times the weight."""
+    from cosmos_rl_amd.policy.kernel.moe.indices import permute_tokens
+    from cosmos_rl_amd.policy.kernel.moe.moe import combine_expert_outputs, route_tokens
+    E, T, TOPK, H, I = 128, 8192, 8, 2048, 768
+    g = torch.Generator(device=dev).manual_seed(55)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    wgu = (torch.randn(E, 2 * I, H, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    wd = (torch.randn(E, H, I, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    qgu, sgu = ops.per_block_cast_to_fp8(wgu)
+    qd, sd = ops.per_block_cast_to_fp8(wd)
+    top = torch.topk(torch.rand(T, E, generator=g, device=dev), TOPK, dim=1)
+    r = route_tokens(top.indices.to(torch.int32), None, E, 128)
+    total = int(r.m_offsets[-1])
+    assert total % 128 == 0 and int((r.row_tokens >= 0).sum()) == T * TOPK
+    contig = permute_tokens(x, r.row_tokens)[:total]
+    m_idx = ops.create_indices_from_offsets_nosync(r.m_offsets, total)
+    m_idx = torch.where(r.row_tokens[:total] >= 0, m_idx, torch.full_like(m_idx, -1))
+    qx, sx = ops.groupwise_activation_quant(contig)
+    gu = torch.full((total, 2 * I), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qgu, sgu), gu, m_idx)
+    pad = m_idx < 0
+    assert bool(pad.any()) and bool((gu[pad] == 7.0).all()), "padding rows were written"
+    rows = (~pad).nonzero().flatten()[::977][:40]
+
+    def ref_rows(qa, sa, qb, sb, rows_):
+        e = m_idx[rows_].long()
+        a = qa[rows_].double() * sa[rows_].double().repeat_interleave(128, dim=1)
+        b = qb[e].double() * sb[e].double().repeat_interleave(128, dim=1).repeat_interleave(128, dim=2)[:, :qb.shape[1]]
+        return torch.einsum("rk,rnk->rn", a, b)
+
+    check_bf16(gu[rows], ref_rows(qx, sx, qgu, sgu, rows).float().cpu(), "cfg5 gate_up rows")
+    gu[pad] = 0
+    qh, sh = ops.swiglu_quant(gu[:, :I], gu[:, I:])
+    sl = slice(0, 4096)
+    h = torch.nn.functional.silu(gu[sl, :I]) * gu[sl, I:]
+    qh2, sh2 = ops.groupwise_activation_quant(h)
+    same = (qh[sl].view(torch.uint8) == qh2.view(torch.uint8)).float().mean().item()
+    assert same > 0.99, same  # torch's silu differs from the library's fixed exp sequence by a bf16 ulp on a few elements
+    dn = torch.zeros(total, H, dtype=torch.bfloat16, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qh, sh), (qd, sd), dn, m_idx)
+    check_bf16(dn[rows], ref_rows(qh, sh, qd, sd, rows).float().cpu(), "cfg5 down rows")
+    # permutation inside expert 3's group
+    rows3 = (m_idx == 3).nonzero().flatten()
+    perm = rows3[torch.randperm(rows3.numel(), generator=torch.Generator().manual_seed(1)).to(dev)]
+    qh_p, sh_p = qh.clone(), sh.clone()
+    qh_p[rows3], sh_p[rows3] = qh[perm], sh[perm]
+    dn_p = torch.zeros_like(dn)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qh_p, sh_p), (qd, sd), dn_p, m_idx)
+    assert torch.equal(dn_p[rows3], dn[perm])
+    # combine: one-hot weights pick one expert row, scaled
+    wts = torch.zeros(T, TOPK, dtype=torch.bfloat16, device=dev)
+    wts[:, 2] = 0.5
+    y = combine_expert_outputs(dn, r, wts)
+    slot_pos = (r.slot_order == 2).float().argmax(dim=1)
+    src = r.row_map.gather(1, slot_pos[:, None]).flatten().long()
+    assert torch.equal(y, (dn[src].float() * 0.5).to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("T,E,K,N,topk", [(300, 7, 512, 384, 2), (2600, 7, 384, 2048, 2), (3300, 7, 1152, 2048, 2), (3300, 7, 1024, 1792, 2),
                                           (3300, 7, 128, 2048, 2)])
 def test_grouped_gemm(dev, T, E, K, N, topk):
