@@ -237,7 +237,8 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         gbs = bytes_ / (med * 1e-3) / 1e9
         bound = "mfma" if flops / bytes_ > FP8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9) else "hbm"
         out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
-                     "frac": round(tf / FP8_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS, 4)}
+                     "frac": round(tf / FP8_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS, 4),
+                     "frac_mfma": round(tf / FP8_PEAK_TFLOPS, 4), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
 
     # rowwise weight quantisation at the shapes of one weight sync (vLLM packed layers)
     for nm, (r, c) in [("rowwise_cfg1_4864x896", (4864, 896)), ("rowwise_qkv_4608x3584", (4608, 3584)),
@@ -355,6 +356,16 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
                                              qh.data_ptr(), I, sh.data_ptr(), stream))
         check(lib.cfp8_gemm_grouped_block128(qh.data_ptr(), I, sh.data_ptr(), qd.data_ptr(), sd.data_ptr(), m_idx.data_ptr(),
                                              dn.data_ptr(), H, 0, total, H, I, E, stream))
+    # the same MLP with SwiGLU + requantisation as the epilogue of the gate_up GEMM (gate and up weights interleaved
+    # in blocks of 128 rows): three launches, the bf16 gate_up product never reaches memory
+    qgi, sgi = ops.interleave_gate_up((qgu[:, :I], sgu[:, :I // 128]), (qgu[:, I:], sgu[:, I // 128:]))
+
+    def moe_fused():
+        check(lib.cfp8_quant_group128(xs.data_ptr(), total, H, H, qxs.data_ptr(), H, sxs.data_ptr(), 0, stream))
+        check(lib.cfp8_gemm_grouped_swiglu_quant(qxs.data_ptr(), H, sxs.data_ptr(), qgi.data_ptr(), sgi.data_ptr(), m_idx.data_ptr(),
+                                                 qh.data_ptr(), I, sh.data_ptr(), total, I, H, E, stream))
+        check(lib.cfp8_gemm_grouped_block128(qh.data_ptr(), I, sh.data_ptr(), qd.data_ptr(), sd.data_ptr(), m_idx.data_ptr(),
+                                             dn.data_ptr(), H, 0, total, H, I, E, stream))
     # SwiGLU + 1x128 requantisation between the two GEMMs, alone: 2 x 2 B read + 1 B written per element
     moe()
     hbm("swiglu_quant_cfg5_%dx%d" % (total, I), 5 * total * I + 4 * sh.numel(),
@@ -362,6 +373,8 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
                                                      qh.data_ptr(), I, sh.data_ptr(), stream)))
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
     mfma("grouped_cfg5_mlp_quant_gateup_swiglu_down", flops5,
+         qgu.numel() + qd.numel() + routed * (H * 2 + I + H * 2), moe_fused, iters=50)
+    mfma("grouped_cfg5_mlp_swiglu_as_separate_launch", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=50)
     # weighted combine of the expert rows back into token order (bf16 rounding at every step)
     e_sorted, order = torch.sort(topi, stable=True)

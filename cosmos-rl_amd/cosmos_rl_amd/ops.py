@@ -405,6 +405,44 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs: Tuple[torch.Tensor, torch.Ten
     return out
 
 
+def interleave_gate_up(gate: Tuple[torch.Tensor, torch.Tensor], up: Tuple[torch.Tensor, torch.Tensor]
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Gate and up expert weights (fp8 [E, I, K], block scales [E, I/128, K/128] each) as one [E, 2I, K] weight
+    whose 128-row blocks alternate gate, up, gate, up ... - the layout ``grouped_gemm_swiglu_quant`` takes.
+    Done once, when the weights are arranged."""
+    (qg, sg), (qu, su) = gate, up
+    E, I, K = qg.shape
+    if I % BLOCK or qu.shape != qg.shape or sg.shape != su.shape:
+        raise ValueError("gate and up must have the same shape with I a multiple of 128")
+    q = torch.stack([qg.view(torch.uint8).view(E, I // BLOCK, BLOCK, K), qu.view(torch.uint8).view(E, I // BLOCK, BLOCK, K)], dim=2)
+    s = torch.stack([sg, su], dim=2)
+    return q.reshape(E, 2 * I, K).view(FP8_DTYPE), s.reshape(E, 2 * I // BLOCK, K // BLOCK).contiguous()
+
+
+def grouped_gemm_swiglu_quant(lhs: Tuple[torch.Tensor, torch.Tensor], rhs_interleaved: Tuple[torch.Tensor, torch.Tensor],
+                              m_indices: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Grouped gate_up GEMM, SiLU(gate) * up and the 1x128 quantisation of the product in one launch
+    (group_gemms.py:194-218): returns (fp8 [M, I], fp32 [M, I/128]) - the input of the down GEMM.  Rows whose
+    m_indices is negative are left as allocated."""
+    a, sa = lhs
+    b, sb = rhs_interleaved
+    _need_gpu(a, sa, b, sb, m_indices)
+    M, K = a.shape
+    E, N2, Kb = b.shape
+    I = N2 // 2
+    if Kb != K or m_indices.numel() != M or tuple(sa.shape) != (M, K // BLOCK) or tuple(sb.shape) != (E, N2 // BLOCK, K // BLOCK):
+        raise ValueError("shape mismatch in grouped GEMM")
+    if m_indices.dtype != torch.int32:
+        m_indices = m_indices.to(torch.int32)
+    a, b, sa, sb = a.contiguous(), b.contiguous(), sa.contiguous(), sb.contiguous()
+    q = torch.empty((M, I), dtype=FP8_DTYPE, device=a.device)
+    s = torch.empty((M, I // BLOCK), dtype=torch.float32, device=a.device)
+    _lib.check(_lib.load().cfp8_gemm_grouped_swiglu_quant(a.data_ptr(), K, sa.data_ptr(), b.data_ptr(), sb.data_ptr(),
+                                                         m_indices.contiguous().data_ptr(), q.data_ptr(), I, s.data_ptr(),
+                                                         M, I, K, E, _stream()))
+    return q, s
+
+
 def create_indices_from_offsets_nosync(m_offsets: torch.Tensor, total: Optional[int] = None) -> torch.Tensor:
     """``dsgemm_utils.create_indices_from_offsets_nosync`` (group_gemms.py:157): expert id per
     row from the inclusive cumulative group ends.  Pass ``total`` (the number of rows, which the

@@ -65,17 +65,22 @@ class TorchBF16GroupGEMM(GroupGEMMStrategy):
 class DSGroupGEMM(GroupGEMMStrategy):
     """FP8 grouped GEMM: block-quantised expert weights, 1x128 activation groups."""
 
-    def __init__(self, custom_activation, use_triton_quant=True, fuse_swiglu=True, fuse_gate_up=False):
+    def __init__(self, custom_activation, use_triton_quant=True, fuse_swiglu=True, fuse_gate_up=False, fuse_epilogue=True):
         # ``use_triton_quant`` selected between two third-party quantisers in the reference
         # (group_gemms.py:188-191); both map to the one HIP group quantiser here.
         # fuse_swiglu: when the activation is SiLU, ``act(gate) * up`` and the 1x128 quantisation of the
         # product (group_gemms.py:209-218) run as one kernel and the bf16 product is never written.
         # fuse_gate_up: the gate and up projections (two GEMMs on the same input, :194-207) run as one
         # GEMM over the concatenated weights; costs a second copy of those weights.
+        # With both, the intermediate size a multiple of 128 and token rows padded to 128, the SwiGLU and
+        # the quantisation become the epilogue of that one GEMM (weights interleaved in 128-row blocks of
+        # gate and up): the [rows, 2 I] product never reaches memory.  Same bits as the unfused chain.
+        # ``fuse_epilogue=False`` keeps the GEMM and the SwiGLU quantiser as two launches.
         self.activation_function = custom_activation
         self.use_triton_quant = use_triton_quant
         self.fuse_swiglu = fuse_swiglu and self._is_silu(custom_activation)
         self.fuse_gate_up = fuse_gate_up
+        self.fuse_epilogue = fuse_epilogue
 
     @staticmethod
     def _is_silu(fn) -> bool:
@@ -108,7 +113,14 @@ class DSGroupGEMM(GroupGEMMStrategy):
         gate_up_input = self._quant(valid_tokens)
         # padding rows (m_indices < 0) are not written by the GEMMs: start from zeros so that what the
         # activation reads there is defined
-        if self.fuse_gate_up and intermediate_size % 128 == 0:
+        hidden_quantized = None
+        if self.fuse_gate_up and self.fuse_swiglu and self.fuse_epilogue and intermediate_size % 128 == 0 and total % 128 == 0:
+            inter = getattr(module, "_gate_up_fp8_interleaved", None)
+            if inter is None or inter[2] != (gate_fp8.data_ptr(), up_fp8.data_ptr()):
+                inter = (*ops.interleave_gate_up((gate_fp8, gate_s), (up_fp8, up_s)), (gate_fp8.data_ptr(), up_fp8.data_ptr()))
+                module._gate_up_fp8_interleaved = inter
+            hidden_quantized = ops.grouped_gemm_swiglu_quant(gate_up_input, (inter[0], inter[1]), m_indices)
+        elif self.fuse_gate_up and intermediate_size % 128 == 0:
             fused = getattr(module, "_gate_up_fp8_fused", None)
             if fused is None or fused[2] != (gate_fp8.data_ptr(), up_fp8.data_ptr()):
                 fused = (torch.cat([gate_fp8, up_fp8], dim=1), torch.cat([gate_s, up_s], dim=1),
@@ -122,7 +134,9 @@ class DSGroupGEMM(GroupGEMMStrategy):
             up_out = torch.zeros_like(gate_out)
             ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (gate_fp8, gate_s), gate_out, m_indices)
             ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (up_fp8, up_s), up_out, m_indices)
-        if self.fuse_swiglu:
+        if hidden_quantized is not None:
+            pass
+        elif self.fuse_swiglu:
             hidden_quantized = ops.swiglu_quant(gate_out, up_out)
         else:
             hidden_quantized = self._quant(self.activation_function(gate_out) * up_out)

@@ -219,4 +219,11 @@ __device__ __forceinline__ float silu32_det(float x) {
     return x / (1.0f + exp32_det(-x));
 }
 
+// two packed bf16 gate values and two up values -> two packed bf16 of bf16(bf16(silu(g)) * u)
+__device__ __forceinline__ u32 swiglu_pair(u32 g, u32 u) {
+    const float s0 = silu32_det(bf16_lo(g)), s1 = silu32_det(bf16_hi(g));
+    const u32 s = pack_bf16x2(s0, s1);
+    return pack_bf16x2(bf16_lo(s) * bf16_lo(u), bf16_hi(s) * bf16_hi(u));
+}
+
 }  // namespace cfp8

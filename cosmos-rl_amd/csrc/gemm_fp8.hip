@@ -45,6 +45,9 @@ struct GemmArgs {
     float* partial;
     size_t partial_bytes;
     int k_slices, slice_steps;
+    // grouped GEMM with the SwiGLU + 1x128 quantisation epilogue: scales of the quantised product [M, N / 256]
+    float* h_scales;
+    int64_t ld_hs;
 };
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int c) {
@@ -622,9 +625,10 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 // ---------------------------------------------------------------------------
 constexpr int kMaxTileWeightScales = 2048;
 
-template <int BM, int BN, int MODE, bool OUT_F32, bool SCALE_VEC>
+template <int BM, int BN, int MODE, bool OUT_F32, bool SCALE_VEC, bool SWIGLU = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8_kernel(const GemmArgs p) {
     static_assert((BM == 256 && BN == 128) || (BM == 128 && BN == 256), "eight 64 x 64 wave tiles");
+    static_assert(!SWIGLU || (MODE == kGrouped && BN == 256 && !OUT_F32), "the SwiGLU epilogue belongs to the grouped 128 x 256 tile");
     static_assert(MODE == kBlock || MODE == kGrouped, "block-scaled modes only");
     constexpr int WM = BM / 64;
     constexpr int STAGE = (BM + BN) * 128;  // 48 KiB
@@ -832,6 +836,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
 #undef CFP8_PRODUCT
 
     // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+    if constexpr (SWIGLU) {
+        // The tile's 256 weight rows are 128 gate rows followed by the 128 up rows of the same hidden columns
+        // (the caller interleaves the two projections in blocks of 128), so the tile holds everything one 1x128
+        // group of h = silu(gate) * up needs.  Both halves go to LDS rounded to bf16, as the GEMM would have
+        // written them; then four threads per token row form h, its group maximum and scale, and the fp8 bytes:
+        // the arithmetic of the separate SwiGLU quantiser, bit for bit, without the bf16 round trip through memory.
+        constexpr int GST = 272;                       // LDS row stride in bytes (128 bf16 + 16)
+        __syncthreads();                               // all waves are done reading the operand stages
+        uint8_t* const side = smem + (wn >> 1) * (128 * GST);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 v = acc[i][j];
+                *reinterpret_cast<uint2*>(side + (wm * 64 + j * 16 + lrow) * GST + ((wn & 1) * 64 + i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        __syncthreads();
+        const int r = t >> 2, c4 = t & 3;              // token row of the tile, 32-column part of the group
+        const uint8_t* const gp = smem + r * GST + c4 * 64;
+        const uint8_t* const up = gp + 128 * GST;
+        uint4 h[4];
+        u32 mx = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint4 g = *reinterpret_cast<const uint4*>(gp + e * 16), u = *reinterpret_cast<const uint4*>(up + e * 16);
+            h[e] = make_uint4(swiglu_pair(g.x, u.x), swiglu_pair(g.y, u.y), swiglu_pair(g.z, u.z), swiglu_pair(g.w, u.w));
+            mx = absmax8(mx, h[e]);
+        }
+        mx = pk_fold(mx);
+        mx = umax(mx, dpp<0xB1>(mx));                  // the four threads of a row are one DPP quad
+        mx = umax(mx, dpp<0x4E>(mx));
+        const float scale = scale_from_amax(amax_from_bits(mx));
+        const Divider d(scale);
+        const int m = m0 + r;
+        if (p.m_indices[m] == expert) {
+            uint8_t* const q = static_cast<uint8_t*>(p.out) + (int64_t)m * p.ld_out + tn * 128 + c4 * 32;
+            const uint2 b0 = cast8(h[0], d), b1 = cast8(h[1], d), b2 = cast8(h[2], d), b3 = cast8(h[3], d);
+            *reinterpret_cast<uint4*>(q) = make_uint4(b0.x, b0.y, b1.x, b1.y);
+            *reinterpret_cast<uint4*>(q + 16) = make_uint4(b2.x, b2.y, b3.x, b3.y);
+            if (c4 == 0) p.h_scales[(int64_t)m * p.ld_hs + tn] = scale;
+        }
+        return;
+    }
     if (OUT_F32) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -1388,6 +1436,27 @@ static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// grouped GEMM over interleaved gate / up weights with the SwiGLU + 1x128 quantisation epilogue
+static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
+    constexpr int BM = 128, BN = 256;
+    p.tiles_m = p.M / BM;
+    p.tiles_n = p.N / BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    const size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
+    const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    using Kern = void (*)(const GemmArgs);
+    const Kern kern = vec ? static_cast<Kern>(gemm_block_w8_kernel<BM, BN, kGrouped, false, true, true>)
+                          : static_cast<Kern>(gemm_block_w8_kernel<BM, BN, kGrouped, false, false, true>);
+    constexpr size_t lds_max = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
+    static std::atomic<bool> done[65][2];  // zero-initialised
+    const int slot = device_slot();
+    if (slot == 64) done[64][vec].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec])) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
+    return check_launch("gemm");
+}
+
 template <int MODE>
 static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) {
@@ -1597,4 +1666,35 @@ extern "C" int cfp8_gemm_grouped_block128(const void* a, int64_t ld_a, const flo
     p.sb_stride_n = kb; p.sb_stride_k = 1; p.sb_stride_e = nb * kb;
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
     return launch_gemm<kGrouped>(p, out_dtype, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cfp8_gemm_grouped_swiglu_quant(const void* a, int64_t ld_a, const float* sa, const void* b, const float* sb,
+                                              const int32_t* m_indices, void* q, int64_t ld_q, float* scales,
+                                              int64_t M, int64_t I, int64_t K, int64_t E, void* stream) {
+    using namespace cfp8;
+    if (M < 0 || I < 0 || K < 0) return set_error(CFP8_EINVAL, "gemm_grouped_swiglu_quant: negative shape");
+    if (M == 0 || I == 0) return CFP8_OK;
+    if (int rc = check_common("gemm_grouped_swiglu_quant", a, b, sa, sb, q, ld_a, K, 2 * I, CFP8_OUT_BF16, M, 2 * I, K)) return rc;
+    if (!m_indices || !scales) return set_error(CFP8_EINVAL, "gemm_grouped_swiglu_quant: null m_indices or scales");
+    if (E <= 0) return set_error(CFP8_EINVAL, "gemm_grouped_swiglu_quant: E must be positive");
+    if (M % 128 || I % 128 || K == 0 || (K >> 7) * 2 > kMaxTileWeightScales)
+        return set_error(CFP8_EINVAL, "gemm_grouped_swiglu_quant: needs M %% 128 == 0, I %% 128 == 0 and 0 < K <= %d (M=%lld I=%lld K=%lld)",
+                         kMaxTileWeightScales * 64, (long long)M, (long long)I, (long long)K);
+    if (ld_q < I || ld_q % 16 || (reinterpret_cast<uintptr_t>(q) & 15u))
+        return set_error(CFP8_EINVAL, "gemm_grouped_swiglu_quant: q must be 16-byte aligned with a pitch that is a multiple of 16 and >= I");
+    if (int rc = check_device()) return rc;
+    GemmArgs p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.sa = sa;
+    p.sb = sb;
+    p.m_indices = m_indices;
+    p.out = q;
+    p.h_scales = scales;
+    p.ld_hs = I / 128;
+    p.ld_a = ld_a; p.ld_b = K; p.ld_out = ld_q;
+    const int64_t nb = 2 * I / 128, kb = K / 128;
+    p.sb_stride_n = kb; p.sb_stride_k = 1; p.sb_stride_e = nb * kb;
+    p.M = (int)M; p.N = (int)(2 * I); p.K = (int)K;
+    return launch_grouped_swiglu(p, static_cast<hipStream_t>(stream));
 }

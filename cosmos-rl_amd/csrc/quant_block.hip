@@ -177,12 +177,7 @@ __global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __
 
 // SwiGLU fused with the 1x128 quantiser: h = bf16(bf16(silu(g)) * u) is formed in registers from the
 // two bf16 GEMM outputs and quantised like group128_kernel<DIV> does; h never exists in memory.
-// The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors.
-__device__ __forceinline__ u32 swiglu_pair(u32 g, u32 u) {
-    const float s0 = silu32_det(bf16_lo(g)), s1 = silu32_det(bf16_hi(g));
-    const u32 s = pack_bf16x2(s0, s1);
-    return pack_bf16x2(bf16_lo(s) * bf16_lo(u), bf16_hi(s) * bf16_hi(u));
-}
+// The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors (swiglu_pair).
 
 __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __restrict__ gate, int64_t ldg,
                                                               const uint4* __restrict__ up, int64_t ldu, int nvec,

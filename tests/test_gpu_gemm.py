@@ -246,6 +246,41 @@ def test_gemm_block128_cfg4_properties(dev):
 
 
 # ---------------------------------------------------------------------------- grouped
+@pytest.mark.parametrize("T,E,K,I,topk", [(300, 7, 512, 256, 2), (3300, 7, 1152, 1024, 2), (700, 5, 128, 128, 3), (2000, 9, 1024, 384, 2)])
+def test_grouped_swiglu_epilogue_bit_exact(dev, T, E, K, I, topk):
+    """Grouped gate_up GEMM with SwiGLU + 1x128 requantisation as its epilogue (interleaved weights) against the
+    grouped GEMM on the concatenated weights followed by the SwiGLU quantiser: same bytes, same scales; padding rows
+    untouched."""
+    g = torch.Generator().manual_seed(T + I)
+    logits = torch.rand(T, E, generator=g)
+    logits[:, 2] = -1.0  # an expert without tokens
+    token_of_row, m_indices, m_sizes, m_offsets = O.route_topk_contiguous(logits, topk, 128)
+    x = O.make_activation(T, K, seed=5)
+    xs = torch.zeros(token_of_row.numel(), K, dtype=torch.bfloat16)
+    valid = token_of_row >= 0
+    xs[valid] = x[token_of_row[valid]]
+    qx, sx = ops.groupwise_activation_quant(xs.to(dev))
+    qg, sg = ops.per_block_cast_to_fp8(O.make_weight((E, I, K), seed=6, std=0.05).to(dev))
+    qu, su = ops.per_block_cast_to_fp8(O.make_weight((E, I, K), seed=7, std=0.05).to(dev))
+    mi = m_indices.to(dev)
+    gu = torch.zeros(xs.shape[0], 2 * I, dtype=torch.bfloat16, device=dev)
+    ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (torch.cat([qg, qu], 1), torch.cat([sg, su], 1)), gu, mi)
+    q0, s0 = ops.swiglu_quant(gu[:, :I], gu[:, I:])
+    qi, si = ops.interleave_gate_up((qg, sg), (qu, su))
+    assert torch.equal(qi.view(torch.uint8)[:, 128:256], qu.view(torch.uint8)[:, :128]) and torch.equal(si[:, 1], su[:, 0])
+    q1 = torch.full((xs.shape[0], I), 0x55, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    s1 = torch.full((xs.shape[0], I // 128), -1.0, dtype=torch.float32, device=dev)
+    from cosmos_rl_amd import _lib
+    _lib.check(_lib.load().cfp8_gemm_grouped_swiglu_quant(qx.data_ptr(), K, sx.data_ptr(), qi.data_ptr(), si.data_ptr(), mi.data_ptr(),
+                                                         q1.data_ptr(), I, s1.data_ptr(), xs.shape[0], I, K, E,
+                                                         torch.cuda.current_stream().cuda_stream))
+    v = valid.to(dev)
+    assert torch.equal(q1.view(torch.uint8)[v], q0.view(torch.uint8)[v]) and torch.equal(s1[v].view(torch.int32), s0[v].view(torch.int32))
+    assert bool((q1.view(torch.uint8)[~v] == 0x55).all()) and bool((s1[~v] == -1.0).all())
+    q2, s2 = ops.grouped_gemm_swiglu_quant((qx, sx), (qi, si), mi)
+    assert torch.equal(q2.view(torch.uint8)[v], q0.view(torch.uint8)[v]) and torch.equal(s2[v], s0[v])
+
+
 def test_grouped_cfg5_full_size_properties(dev):
     """Config 5 at full size: 8192 tokens routed top-8 over 128 experts (65536 rows, groups padded to 128), expert MLP
     shapes [1536, 2048] and [2048, 768], through the host path of the reference (route -> gather -> DSGroupGEMM-style

@@ -197,7 +197,10 @@ def test_ds_group_gemm_strategy(dev):
     assert strat.fuse_swiglu and not strat.fuse_gate_up
     out_gu = group_gemms.DSGroupGEMM(act, fuse_gate_up=True).execute(
         xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
-    assert torch.equal(out_gu, out)
+    assert torch.equal(out_gu, out)                      # SwiGLU + requantisation as the epilogue of the one GEMM
+    out_gu2 = group_gemms.DSGroupGEMM(act, fuse_gate_up=True, fuse_epilogue=False).execute(
+        xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+    assert torch.equal(out_gu2, out)                     # one fused GEMM, then the SwiGLU quantiser
     out_plain = group_gemms.DSGroupGEMM(act, fuse_swiglu=False).execute(
         xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
     assert O.rel_frobenius(out_plain.float(), out.float()) <= 5e-3
