@@ -84,6 +84,7 @@ def test_graph_moe_chain(dev):
     wgu, wd = _bf16(dev, 1, E, 2 * I, H, std=0.05), _bf16(dev, 2, E, H, I, std=0.05)
     qgu, sgu = ops.per_block_cast_to_fp8(wgu)
     qd, sd = ops.per_block_cast_to_fp8(wd)
+    qgi, sgi = ops.interleave_gate_up((qgu[:, :I], sgu[:, :I // 128]), (qgu[:, I:], sgu[:, I // 128:]))
     rows_cap = T * K + E * 128
 
     def inputs(seed):
@@ -101,9 +102,13 @@ def test_graph_moe_chain(dev):
         gu = torch.zeros(rows_cap, 2 * I, dtype=torch.bfloat16, device=dev)
         ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qgu, sgu), gu, m_idx)
         qh, sh = ops.swiglu_quant(gu[:, :I], gu[:, I:])
+        qh_e, sh_e = ops.grouped_gemm_swiglu_quant((qx, sx), (qgi, sgi), m_idx)   # the same as the GEMM's epilogue
+        keep = (m_idx >= 0)[:, None]
+        qh_e = torch.where(keep, qh_e.view(torch.uint8), torch.zeros_like(qh_e.view(torch.uint8)))
+        sh_e = torch.where(keep, sh_e, torch.zeros_like(sh_e))
         dn = torch.zeros(rows_cap, H, dtype=torch.bfloat16, device=dev)
         ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qh, sh), (qd, sd), dn, m_idx)
         y = combine_expert_outputs(dn, r, wts)
-        return (r.row_tokens, r.row_map, m_idx, qx, gu, qh, dn, y)
+        return (r.row_tokens, r.row_map, m_idx, qx, gu, qh, dn, y, qh_e, sh_e)
 
     _replay_matches_eager(dev, inputs, fn)
