@@ -376,6 +376,24 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
          qgu.numel() + qd.numel() + routed * (H * 2 + I + H * 2), moe_fused, iters=50)
     mfma("grouped_cfg5_mlp_swiglu_as_separate_launch", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + 2 * I * 2 + I * 2 + H * 2), moe, iters=50)
+    # token gather + 1x128 quantisation in one pass (input side of the first grouped GEMM): reads the 8192 tokens
+    # (8 times, from the caches), writes fp8 rows and scales; against the two-launch form that writes and re-reads
+    # the gathered bf16 matrix
+    tok = torch.randn(T, H, generator=gen, device=dev).to(torch.bfloat16)
+    src = torch.full((total,), -1, dtype=torch.int32, device=dev)
+    e_sorted0, order0 = torch.sort(topi, stable=True)
+    first0 = torch.cumsum(counts, 0) - counts
+    dest = start[e_sorted0] + torch.arange(T * TOPK, device=dev) - first0[e_sorted0]
+    src.fill_(-1)
+    src[dest] = (order0 // TOPK).to(torch.int32)
+    gath = torch.empty(total, H, dtype=torch.bfloat16, device=dev)
+
+    def gather_then_quant():
+        check(lib.cfp8_gather_rows(tok.data_ptr(), H * 2, src.data_ptr(), total, H * 2, gath.data_ptr(), H * 2, stream))
+        check(lib.cfp8_quant_group128(gath.data_ptr(), total, H, H, qxs.data_ptr(), H, sxs.data_ptr(), 0, stream))
+    hbm("gather_quant_cfg5_%dx%d" % (total, H), T * H * 2 + total * H + 4 * sxs.numel() + 4 * total,
+        lambda: check(lib.cfp8_gather_quant_group128(tok.data_ptr(), H, src.data_ptr(), total, H, qxs.data_ptr(), H, sxs.data_ptr(), stream)))
+    hbm("gather_then_quant_cfg5_two_launches", T * H * 2 + total * H + 4 * sxs.numel() + 4 * total, gather_then_quant)
     # weighted combine of the expert rows back into token order (bf16 rounding at every step)
     e_sorted, order = torch.sort(topi, stable=True)
     first = torch.cumsum(counts, 0) - counts

@@ -100,6 +100,20 @@ class DSGroupGEMM(GroupGEMMStrategy):
         total = int(m_offsets[-1])
         valid_tokens = contig_tokens[:total]
         m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
+        contig_tokens[:total] = self._run(self._quant(valid_tokens), m_indices, total, module, contig_tokens.dtype)
+        return contig_tokens
+
+    def execute_from_tokens(self, tokens, row_tokens, m_sizes, m_offsets, module):
+        """``execute`` on ``tokens[row_tokens]`` (zero rows for -1) without building that matrix: the gather and the
+        1x128 quantisation of the first GEMM's input are one pass over the token matrix.  Returns the expert outputs
+        [rows, hidden] for the rows of the expert-grouped layout (``row_tokens``: token behind each row)."""
+        from cosmos_rl_amd.policy.kernel.moe.indices import permute_quantize_tokens
+        total = int(m_offsets[-1])
+        m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
+        return self._run(permute_quantize_tokens(tokens, row_tokens[:total]), m_indices, total, module, tokens.dtype)
+
+    def _run(self, gate_up_input, m_indices, total, module, dt):
+        """gate/up GEMMs, activation, requantisation, down GEMM on the quantised expert-grouped rows"""
 
         gate_fp8, gate_s = module.get_parameter("gate_proj_fp8"), module.get_parameter("gate_proj_scales")
         up_fp8, up_s = module.get_parameter("up_proj_fp8"), module.get_parameter("up_proj_scales")
@@ -107,10 +121,9 @@ class DSGroupGEMM(GroupGEMMStrategy):
 
         intermediate_size = module.get_parameter("gate_proj_weight").shape[1]
         hidden_size = module.get_parameter("down_proj_weight").shape[1]
-        dev, dt = contig_tokens.device, contig_tokens.dtype
+        dev = gate_up_input[0].device
 
         down_out = torch.empty((total, hidden_size), device=dev, dtype=dt)
-        gate_up_input = self._quant(valid_tokens)
         # padding rows (m_indices < 0) are not written by the GEMMs: start from zeros so that what the
         # activation reads there is defined
         hidden_quantized = None
@@ -141,8 +154,7 @@ class DSGroupGEMM(GroupGEMMStrategy):
         else:
             hidden_quantized = self._quant(self.activation_function(gate_out) * up_out)
         ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(hidden_quantized, (down_fp8, down_s), down_out, m_indices)
-        contig_tokens[:total] = down_out
-        return contig_tokens
+        return down_out
 
     @staticmethod
     def is_available() -> bool:

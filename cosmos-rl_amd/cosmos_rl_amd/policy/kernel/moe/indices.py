@@ -12,7 +12,7 @@ import torch
 
 from cosmos_rl_amd import _lib
 
-__all__ = ["generate_permute_indices", "permute_tokens"]
+__all__ = ["generate_permute_indices", "permute_tokens", "permute_quantize_tokens"]
 
 
 def _stream() -> int:
@@ -64,3 +64,18 @@ def permute_tokens(tokens: torch.Tensor, permuted_indices: torch.Tensor) -> torc
     _lib.check(_lib.load().cfp8_gather_rows(tokens.data_ptr(), tokens.stride(0) * tokens.element_size(), idx.data_ptr(),
                                             idx.numel(), row_bytes, out.data_ptr(), row_bytes, _stream()))
     return out
+
+
+def permute_quantize_tokens(tokens: torch.Tensor, permuted_indices: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``groupwise_activation_quant(tokens[permuted_indices])`` (zero rows for -1) in one pass: the 1x128-quantised
+    input of the first grouped GEMM (group_gemms.py:188-191) straight from the token matrix, without the gathered
+    bf16 copy.  Returns (fp8 [rows, H], fp32 [rows, ceil(H/128)])."""
+    if not tokens.is_cuda or tokens.dim() != 2 or tokens.stride(1) != 1 or tokens.dtype != torch.bfloat16:
+        raise ValueError("expected a 2-D bf16 GPU tensor with unit column stride")
+    H = tokens.shape[1]
+    idx = permuted_indices.to(torch.int32).contiguous()
+    q = torch.empty((idx.numel(), H), dtype=torch.float8_e4m3fn, device=tokens.device)
+    s = torch.empty((idx.numel(), (H + 127) // 128), dtype=torch.float32, device=tokens.device)
+    _lib.check(_lib.load().cfp8_gather_quant_group128(tokens.data_ptr(), tokens.stride(0), idx.data_ptr(), idx.numel(), H,
+                                                     q.data_ptr(), H, s.data_ptr(), _stream()))
+    return q, s

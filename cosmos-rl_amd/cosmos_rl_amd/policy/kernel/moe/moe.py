@@ -97,6 +97,10 @@ def grouped_experts_forward(x: torch.Tensor, token_mask: Optional[torch.Tensor],
     """``GroupedExperts.forward(x, token_mask, weights, indices)`` (moe.py:179-285) on one rank, with the
     experts of ``module`` run by ``strategy`` (a ``GroupGEMMStrategy``) instead of the per-expert loop."""
     routing = route_tokens(indices, token_mask, n_experts, alignment)
-    contig = permute_tokens(x, routing.row_tokens)
-    out = strategy.execute(contig, routing.m_sizes, routing.m_offsets, module)
+    if hasattr(strategy, "execute_from_tokens") and x.dtype == torch.bfloat16:
+        # the FP8 strategy quantises while it gathers: the expert-grouped bf16 copy of the tokens is never built
+        out = strategy.execute_from_tokens(x, routing.row_tokens, routing.m_sizes, routing.m_offsets, module)
+    else:
+        contig = permute_tokens(x, routing.row_tokens)
+        out = strategy.execute(contig, routing.m_sizes, routing.m_offsets, module)
     return combine_expert_outputs(out, routing, weights)

@@ -88,10 +88,13 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
 // over the 16-lane DPP row.  Every thread handles 4 groups of 4 consecutive
 // group-rows so that four loads are in flight per lane.
 // ---------------------------------------------------------------------------
-template <int MODE>
+// With GATHER, output row r quantises input row src_rows[r] (a zero row where that is negative): the token
+// gather in front of the grouped GEMM and the quantiser in one pass, without the gathered bf16 matrix.
+template <int MODE, bool GATHER = false>
 __global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__ x, int nvec,
                                                        int ngroups, int64_t ldx, uint2* __restrict__ q, int64_t ldq,
-                                                       float* __restrict__ scales, int64_t total_groups) {
+                                                       float* __restrict__ scales, int64_t total_groups,
+                                                       const int32_t* __restrict__ src_rows = nullptr) {
     const int sub = threadIdx.x & 15;
     const int64_t g0 = ((int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)) * 4;
     uint4 v[4];
@@ -105,7 +108,13 @@ __global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__
         gcol[i] = (int)(g - row[i] * ngroups);
         const int vec = gcol[i] * 16 + sub;
         ok[i] = g < total_groups && vec < nvec;
-        v[i] = ok[i] ? ld16<true>(x + row[i] * ldx + vec) : make_uint4(0, 0, 0, 0);
+        if (GATHER) {
+            const int32_t src = g < total_groups ? src_rows[row[i]] : -1;
+            // tokens are read several times (once per expert they go to): leave them in the caches
+            v[i] = ok[i] && src >= 0 ? ld16<false>(x + (int64_t)src * ldx + vec) : make_uint4(0, 0, 0, 0);
+        } else {
+            v[i] = ok[i] ? ld16<true>(x + row[i] * ldx + vec) : make_uint4(0, 0, 0, 0);
+        }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -268,6 +277,25 @@ extern "C" int cfp8_quant_group128(const void* x, int64_t rows, int64_t cols, in
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "quant_group128: misaligned pointer");
     if (int rc = check_device()) return rc;
     return launch_quant_group128(x, rows, cols, ld_x, q, ld_q, scales, mode, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int cfp8_gather_quant_group128(const void* x, int64_t ld_x, const int32_t* src_rows, int64_t rows_out, int64_t cols,
+                                          void* q, int64_t ld_q, float* scales, void* stream) {
+    using namespace cfp8;
+    if (rows_out < 0 || cols < 0) return set_error(CFP8_EINVAL, "gather_quant_group128: negative shape");
+    if (rows_out == 0 || cols == 0) return CFP8_OK;
+    if (!x || !src_rows || !q || !scales) return set_error(CFP8_EINVAL, "gather_quant_group128: null pointer");
+    if (cols % 8 || ld_x % 8 || ld_q % 8 || ld_x < cols || ld_q < cols)
+        return set_error(CFP8_EINVAL, "gather_quant_group128: cols=%lld ld_x=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
+                         (long long)cols, (long long)ld_x, (long long)ld_q);
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "gather_quant_group128: misaligned pointer");
+    const int64_t ngroups = (cols + 127) / 128, total = rows_out * ngroups, blocks = (total + 63) / 64;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gather_quant_group128: too many groups for one launch");
+    if (int rc = check_device()) return rc;
+    hipLaunchKernelGGL((group128_kernel<CFP8_GROUP_MODE_DIV, true>), dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(x), (int)(cols / 8), (int)ngroups, ld_x / 8, static_cast<uint2*>(q), ld_q / 8,
+                       scales, total, src_rows);
+    return check_launch("gather_quant_group128");
 }
 
 extern "C" int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t rows,

@@ -211,6 +211,13 @@ int cfp8_combine_rows(const void* rows, int64_t ld_rows, int64_t num_rows, const
 int cfp8_quant_mxfp4(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
                      void* scales, int64_t ld_scales, void* stream);
 
+/* cfp8_gather_rows followed by cfp8_quant_group128 (CFP8_GROUP_MODE_DIV) as one pass: row r of the
+ * output quantises row src_rows[r] of x (bf16 [*, cols], ld_x in elements), a zero row where src_rows[r] < 0.
+ * The gathered bf16 matrix [rows_out, cols] that the reference builds with torch indexing before
+ * group_gemms.py:188-191 is never written.  q fp8 [rows_out, cols] (ld_q), scales fp32 [rows_out, ceil(cols/128)]. */
+int cfp8_gather_quant_group128(const void* x, int64_t ld_x, const int32_t* src_rows, int64_t rows_out, int64_t cols,
+                               void* q, int64_t ld_q, float* scales, void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */

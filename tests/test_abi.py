@@ -83,6 +83,9 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_gemm_grouped_swiglu_quant(ptr, 128, ptr, ptr, ptr, ptr, ptr, 100, ptr, 128, 100, 128, 2, None) == _lib.EINVAL   # I % 128
     assert lib.cfp8_gemm_grouped_swiglu_quant(ptr, 128, ptr, ptr, ptr, ptr, ptr, 128, ptr, 64, 128, 128, 2, None) == _lib.EINVAL    # M % 128
     assert lib.cfp8_gemm_grouped_swiglu_quant(None, 128, None, None, None, None, None, 128, None, 0, 128, 128, 2, None) == 0
+    assert lib.cfp8_gather_quant_group128(ptr, 60, ptr, 4, 60, ptr, 64, ptr, None) == _lib.EINVAL
+    assert lib.cfp8_gather_quant_group128(None, 64, None, 4, 64, None, 64, None, None) == _lib.EINVAL
+    assert lib.cfp8_gather_quant_group128(None, 64, None, 0, 64, None, 64, None, None) == 0
     # empty problems succeed without pointers
     assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0

@@ -201,6 +201,9 @@ def test_ds_group_gemm_strategy(dev):
     out_gu2 = group_gemms.DSGroupGEMM(act, fuse_gate_up=True, fuse_epilogue=False).execute(
         xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
     assert torch.equal(out_gu2, out)                     # one fused GEMM, then the SwiGLU quantiser
+    # straight from the token matrix: the gather and the first quantisation in one pass
+    out_ft = strat.execute_from_tokens(x.to(dev), tok.to(torch.int32).to(dev), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
+    assert torch.equal(out_ft, out[:out_ft.shape[0]])
     out_plain = group_gemms.DSGroupGEMM(act, fuse_swiglu=False).execute(
         xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod).cpu()
     assert O.rel_frobenius(out_plain.float(), out.float()) <= 5e-3

@@ -272,3 +272,25 @@ def test_combine_rows_slot_limits(dev):
     _lib.check(_lib.load().cfp8_combine_rows(None, H, 0, None, None, _lib.IN_BF16, T, 0, H, 0, out.data_ptr(), H,
                                              torch.cuda.current_stream().cuda_stream))
     assert not bool(out.any())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,H,R", [(300, 2048, 1000), (50, 264, 333), (8, 128, 1), (1000, 7168, 513)])
+def test_permute_quantize_tokens_is_gather_then_quant(dev, T, H, R):
+    from cosmos_rl_amd import ops
+    from cosmos_rl_amd.policy.kernel.moe.indices import permute_quantize_tokens, permute_tokens
+    g = torch.Generator().manual_seed(T + H)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    x[3 % T, 5] = 300.0
+    idx = torch.randint(-1, T, (R,), generator=g, dtype=torch.int32)
+    idx[0] = -1
+    xd = torch.zeros(T, H + 8, dtype=torch.bfloat16, device=dev)[:, :H]      # a row pitch larger than H
+    xd.copy_(x)
+    q1, s1 = permute_quantize_tokens(xd, idx.to(dev))
+    q0, s0 = ops.groupwise_activation_quant(permute_tokens(x.to(dev), idx.to(dev)))
+    assert torch.equal(q1.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(s1.view(torch.int32), s0.view(torch.int32))
+    from oracle import fp8_oracle as O
+    xs = torch.zeros(R, H, dtype=torch.bfloat16)
+    xs[idx >= 0] = x[idx[idx >= 0].long()]
+    qo, so = O.quant_group128(xs)
+    assert torch.equal(q1.view(torch.uint8).cpu(), qo) and torch.equal(s1.cpu().view(torch.int32), so.view(torch.int32))
