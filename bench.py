@@ -303,6 +303,22 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         mfma(f"linear_rowwise_cfg3_M{M}", 2.0 * M * N3 * K3, N3 * K3 + 4 * N3 + M * K3 * 2 + M * N3 * 2,
              lambda: check(lib.cfp8_linear_rowwise(x.data_ptr(), K3, qw3.data_ptr(), K3, sw3.data_ptr(), o.data_ptr(), N3, 0,
                                                    M, N3, K3, ws.data_ptr(), wsb, stream)), iters=50)
+        if M >= 64:
+            # the GEMM alone on the quantised operands, and the vendor library's rowwise scaled GEMM
+            # (torch._scaled_mm) on the same bytes beside it - a comparison figure, nothing here calls it otherwise
+            qx, sx = ops.quant_rowwise(x)
+            fl, by = 2.0 * M * N3 * K3, N3 * K3 + 4 * N3 + M * K3 + M * N3 * 2
+            mfma(f"scaled_mm_rowwise_cfg3_M{M}_gemm_only", fl, by,
+                 lambda: check(lib.cfp8_scaled_mm_rowwise(qx.data_ptr(), K3, sx.data_ptr(), qw3.data_ptr(), K3, sw3.data_ptr(),
+                                                          o.data_ptr(), N3, 0, M, N3, K3, stream)), iters=50)
+            try:
+                sb = sw3.reshape(1, N3)
+                torch._scaled_mm(qx, qw3.t(), scale_a=sx, scale_b=sb, out_dtype=torch.bfloat16)
+                mfma(f"vendor_torch_scaled_mm_rowwise_cfg3_M{M}", fl, by,
+                     lambda: torch._scaled_mm(qx, qw3.t(), scale_a=sx, scale_b=sb, out_dtype=torch.bfloat16), iters=50)
+            except Exception as e:  # the comparison is optional: a torch build without this path must not fail the bench
+                out[f"vendor_torch_scaled_mm_rowwise_cfg3_M{M}"] = {"error": f"{type(e).__name__}: {str(e)[:120]}"}
+            del qx, sx
         del x, o, ws
     del qw3, sw3
 
