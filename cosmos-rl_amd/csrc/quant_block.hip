@@ -90,32 +90,46 @@ __global__ __launch_bounds__(256) void block128_kernel(const uint16_t* __restric
 // ---------------------------------------------------------------------------
 // With GATHER, output row r quantises input row src_rows[r] (a zero row where that is negative): the token
 // gather in front of the grouped GEMM and the quantiser in one pass, without the gathered bf16 matrix.
+// Groups are numbered row-major (row * ngroups + column) in 32 bits; a thread divides once and steps
+// through its four consecutive groups.  Every load is unconditional on a clamped address (what must read
+// as zero is cleared afterwards), so all four are in flight before the first is used.
 template <int MODE, bool GATHER = false>
 __global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__ x, int nvec,
-                                                       int ngroups, int64_t ldx, uint2* __restrict__ q, int64_t ldq,
-                                                       float* __restrict__ scales, int64_t total_groups,
+                                                       u32 ngroups, int64_t ldx, uint2* __restrict__ q, int64_t ldq,
+                                                       float* __restrict__ scales, u32 rows, u32 total_groups,
                                                        const int32_t* __restrict__ src_rows = nullptr) {
     const int sub = threadIdx.x & 15;
-    const int64_t g0 = ((int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)) * 4;
+    const u32 g0 = (blockIdx.x * 16u + (threadIdx.x >> 4)) * 4u;
     uint4 v[4];
-    int64_t row[4];
-    int gcol[4];
+    u32 row[4], gcol[4];
     bool ok[4];
+    {
+        u32 r = g0 / ngroups, c = g0 - r * ngroups;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t g = g0 + i;
-        row[i] = g / ngroups;
-        gcol[i] = (int)(g - row[i] * ngroups);
-        const int vec = gcol[i] * 16 + sub;
-        ok[i] = g < total_groups && vec < nvec;
-        if (GATHER) {
-            const int32_t src = g < total_groups ? src_rows[row[i]] : -1;
-            // tokens are read several times (once per expert they go to): leave them in the caches
-            v[i] = ok[i] && src >= 0 ? ld16<false>(x + (int64_t)src * ldx + vec) : make_uint4(0, 0, 0, 0);
-        } else {
-            v[i] = ok[i] ? ld16<true>(x + row[i] * ldx + vec) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+            row[i] = r;
+            gcol[i] = c;
+            if (++c == ngroups) c = 0, ++r;
         }
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int vec = (int)gcol[i] * 16 + sub;
+        ok[i] = g0 + i < total_groups && vec < nvec;
+        const u32 rc = row[i] < rows ? row[i] : rows - 1;
+        const int vc = vec < nvec ? vec : nvec - 1;
+        if (GATHER) {
+            const int32_t src = src_rows[rc];
+            ok[i] = ok[i] && src >= 0;
+            // tokens are read several times (once per expert they go to): leave them in the caches
+            v[i] = ld16<false>(x + (int64_t)(src >= 0 ? src : 0) * ldx + vc);
+        } else {
+            v[i] = ld16<true>(x + (int64_t)rc * ldx + vc);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (!ok[i]) v[i] = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const u32 m = row16_max(pk_fold(absmax8(0u, v[i])));
@@ -147,40 +161,55 @@ __global__ __launch_bounds__(256) void group128_kernel(const uint4* __restrict__
                 out = make_uint2(o[0], o[1]);
             }
         }
-        if (ok[i]) q[row[i] * ldq + gcol[i] * 16 + sub] = out;
-        if (sub == 0 && g0 + i < total_groups) scales[row[i] * ngroups + gcol[i]] = scale;
+        const int vec = (int)gcol[i] * 16 + sub;
+        if (g0 + i < total_groups && vec < nvec) q[(int64_t)row[i] * ldq + vec] = out;
+        if (sub == 0 && g0 + i < total_groups) scales[g0 + i] = scale;
     }
 }
 
 // ---------------------------------------------------------------------------
 // block dequantiser: y[i, j] = fp8[i, j] * s[i / 128, j / 128]
+// A thread owns one 8-column vector of four consecutive rows (one scale, four loads in flight); the block is
+// BX vectors wide and 256 / BX row quads high, BX chosen by the host to fit the row length, so no index is divided.
 // ---------------------------------------------------------------------------
-template <typename OutVec, bool F32>
+template <bool F32>
 __global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __restrict__ q,
                                                                const float* __restrict__ s, int64_t rows,
-                                                               int64_t cols, int tiles_c, void* __restrict__ y) {
-    const int64_t nvec_row = cols / 8;
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= rows * nvec_row) return;
-    const int64_t r = idx / nvec_row, cv = idx - r * nvec_row;
-    const uint2 w = *reinterpret_cast<const uint2*>(q + r * cols + cv * 8);
-    const float sc = s[(r >> 7) * tiles_c + (cv >> 4)];
-    float f[8];
-    f32x2 p;
-    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, false); f[0] = p[0]; f[1] = p[1];
-    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.x, true);  f[2] = p[0]; f[3] = p[1];
-    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, false); f[4] = p[0]; f[5] = p[1];
-    p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w.y, true);  f[6] = p[0]; f[7] = p[1];
+                                                               int64_t cols, int nvec_row, int tiles_c, void* __restrict__ y) {
+    const int cv = blockIdx.x * blockDim.x + threadIdx.x;
+    if (cv >= nvec_row) return;
+    // (one pass of this loop unless the matrix has more row quads than the grid's y extent can hold)
+    for (int64_t r0 = ((int64_t)blockIdx.y * blockDim.y + threadIdx.y) * 4; r0 < rows;
+         r0 += (int64_t)gridDim.y * blockDim.y * 4) {
+        const float sc = s[(r0 >> 7) * tiles_c + (cv >> 4)];
+        uint2 w[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] *= sc;
-    if (F32) {
-        float4* o = reinterpret_cast<float4*>(static_cast<float*>(y) + r * cols + cv * 8);
-        o[0] = make_float4(f[0], f[1], f[2], f[3]);
-        o[1] = make_float4(f[4], f[5], f[6], f[7]);
-    } else {
-        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(y) + r * cols + cv * 8);
-        *o = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
-                        pack_bf16x2(f[6], f[7]));
+        for (int k = 0; k < 4; ++k) {
+            const int64_t r = r0 + k < rows ? r0 + k : rows - 1;
+            const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + r * cols + (int64_t)cv * 8));
+            w[k] = make_uint2(t[0], t[1]);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (r0 + k >= rows) break;
+            float f[8];
+            f32x2 p;
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].x, false); f[0] = p[0]; f[1] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].x, true);  f[2] = p[0]; f[3] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].y, false); f[4] = p[0]; f[5] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].y, true);  f[6] = p[0]; f[7] = p[1];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] *= sc;
+            const int64_t at = (r0 + k) * cols + (int64_t)cv * 8;
+            if (F32) {
+                uint4* o = reinterpret_cast<uint4*>(static_cast<float*>(y) + at);
+                st16<true>(o, make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])));
+                st16<true>(o + 1, make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]), __float_as_uint(f[7])));
+            } else {
+                st16<true>(reinterpret_cast<uint4*>(static_cast<uint16_t*>(y) + at),
+                           make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])));
+            }
+        }
     }
 }
 
@@ -190,24 +219,29 @@ __global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __
 
 __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __restrict__ gate, int64_t ldg,
                                                               const uint4* __restrict__ up, int64_t ldu, int nvec,
-                                                              int ngroups, uint2* __restrict__ q, int64_t ldq,
-                                                              float* __restrict__ scales, int64_t total_groups) {
+                                                              u32 ngroups, uint2* __restrict__ q, int64_t ldq,
+                                                              float* __restrict__ scales, u32 rows, u32 total_groups) {
     const int sub = threadIdx.x & 15;
-    const int64_t g0 = ((int64_t)blockIdx.x * 16 + (threadIdx.x >> 4)) * 2;
+    const u32 g0 = (blockIdx.x * 16u + (threadIdx.x >> 4)) * 2u;
     uint4 vg[2], vu[2];
-    int64_t row[2];
-    int gcol[2];
+    u32 row[2], gcol[2];
+    row[0] = g0 / ngroups;
+    gcol[0] = g0 - row[0] * ngroups;
+    gcol[1] = gcol[0] + 1 == ngroups ? 0 : gcol[0] + 1;
+    row[1] = gcol[1] == 0 ? row[0] + 1 : row[0];
     bool ok[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int64_t g = g0 + i;
-        row[i] = g / ngroups;
-        gcol[i] = (int)(g - row[i] * ngroups);
-        const int vec = gcol[i] * 16 + sub;
-        ok[i] = g < total_groups && vec < nvec;
-        vg[i] = ok[i] ? ld16<true>(gate + row[i] * ldg + vec) : make_uint4(0, 0, 0, 0);
-        vu[i] = ok[i] ? ld16<true>(up + row[i] * ldu + vec) : make_uint4(0, 0, 0, 0);
+        const int vec = (int)gcol[i] * 16 + sub;
+        ok[i] = g0 + i < total_groups && vec < nvec;
+        const int64_t rc = row[i] < rows ? row[i] : rows - 1;  // unconditional loads on clamped addresses
+        const int vc = vec < nvec ? vec : nvec - 1;
+        vg[i] = ld16<true>(gate + rc * ldg + vc);
+        vu[i] = ld16<true>(up + rc * ldu + vc);
     }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        if (!ok[i]) vg[i] = vu[i] = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const uint4 h = make_uint4(swiglu_pair(vg[i].x, vu[i].x), swiglu_pair(vg[i].y, vu[i].y),
@@ -216,25 +250,28 @@ __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __res
         const float scale = scale_from_amax(amax_from_bits(m));
         const Divider d(scale);
         const uint2 out = cast8(h, d);
-        if (ok[i]) st8<false>(q + row[i] * ldq + gcol[i] * 16 + sub, out);
-        if (sub == 0 && g0 + i < total_groups) scales[row[i] * ngroups + gcol[i]] = scale;
+        if (ok[i]) st8<false>(q + (int64_t)row[i] * ldq + gcol[i] * 16 + sub, out);
+        if (sub == 0 && g0 + i < total_groups) scales[g0 + i] = scale;
     }
 }
+
+// Groups are numbered in 32 bits, and a block's first group index must not wrap.
+constexpr int64_t kMaxGroups = 0xFFFFFF00ll;
 
 int launch_quant_group128(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
                           float* scales, int mode, hipStream_t st) {
     const int64_t ngroups = (cols + 127) / 128;
     const int64_t total = rows * ngroups;
-    const int64_t blocks = (total + 63) / 64;
-    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "quant_group128: too many groups for one launch");
+    if (total > kMaxGroups) return set_error(CFP8_EINVAL, "quant_group128: too many groups for one launch");
+    const unsigned blocks = (unsigned)((total + 63) / 64);
     const uint4* xv = static_cast<const uint4*>(x);
     uint2* qv = static_cast<uint2*>(q);
     if (mode == CFP8_GROUP_MODE_DIV)
-        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DIV>, dim3((unsigned)blocks), dim3(256), 0, st, xv,
-                           (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
+        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DIV>, dim3(blocks), dim3(256), 0, st, xv, (int)(cols / 8),
+                           (u32)ngroups, ld_x / 8, qv, ld_q / 8, scales, (u32)rows, (u32)total, nullptr);
     else
-        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DEEPEP>, dim3((unsigned)blocks), dim3(256), 0, st, xv,
-                           (int)(cols / 8), (int)ngroups, ld_x / 8, qv, ld_q / 8, scales, total);
+        hipLaunchKernelGGL(group128_kernel<CFP8_GROUP_MODE_DEEPEP>, dim3(blocks), dim3(256), 0, st, xv, (int)(cols / 8),
+                           (u32)ngroups, ld_x / 8, qv, ld_q / 8, scales, (u32)rows, (u32)total, nullptr);
     return check_launch("quant_group128");
 }
 
@@ -289,12 +326,12 @@ extern "C" int cfp8_gather_quant_group128(const void* x, int64_t ld_x, const int
         return set_error(CFP8_EINVAL, "gather_quant_group128: cols=%lld ld_x=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
                          (long long)cols, (long long)ld_x, (long long)ld_q);
     if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "gather_quant_group128: misaligned pointer");
-    const int64_t ngroups = (cols + 127) / 128, total = rows_out * ngroups, blocks = (total + 63) / 64;
-    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gather_quant_group128: too many groups for one launch");
+    const int64_t ngroups = (cols + 127) / 128, total = rows_out * ngroups;
+    if (total > kMaxGroups) return set_error(CFP8_EINVAL, "gather_quant_group128: too many groups for one launch");
     if (int rc = check_device()) return rc;
-    hipLaunchKernelGGL((group128_kernel<CFP8_GROUP_MODE_DIV, true>), dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint4*>(x), (int)(cols / 8), (int)ngroups, ld_x / 8, static_cast<uint2*>(q), ld_q / 8,
-                       scales, total, src_rows);
+    hipLaunchKernelGGL((group128_kernel<CFP8_GROUP_MODE_DIV, true>), dim3((unsigned)((total + 63) / 64)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint4*>(x), (int)(cols / 8), (u32)ngroups, ld_x / 8,
+                       static_cast<uint2*>(q), ld_q / 8, scales, (u32)rows_out, (u32)total, src_rows);
     return check_launch("gather_quant_group128");
 }
 
@@ -309,12 +346,12 @@ extern "C" int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, con
                          (long long)cols, (long long)ld_gate, (long long)ld_up, (long long)ld_q);
     if (!aligned16(gate) || !aligned16(up) || (reinterpret_cast<uintptr_t>(q) & 7u))
         return set_error(CFP8_EINVAL, "swiglu_quant_group128: misaligned pointer");
-    const int64_t ngroups = (cols + 127) / 128, total = rows * ngroups, blocks = (total + 31) / 32;
-    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "swiglu_quant_group128: too many groups for one launch");
+    const int64_t ngroups = (cols + 127) / 128, total = rows * ngroups;
+    if (total > kMaxGroups) return set_error(CFP8_EINVAL, "swiglu_quant_group128: too many groups for one launch");
     if (int rc = check_device()) return rc;
-    hipLaunchKernelGGL(swiglu_group128_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(swiglu_group128_kernel, dim3((unsigned)((total + 31) / 32)), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(gate), ld_gate / 8, static_cast<const uint4*>(up), ld_up / 8, (int)(cols / 8),
-                       (int)ngroups, static_cast<uint2*>(q), ld_q / 8, scales, total);
+                       (u32)ngroups, static_cast<uint2*>(q), ld_q / 8, scales, (u32)rows, (u32)total);
     return check_launch("swiglu_quant_group128");
 }
 
@@ -327,16 +364,20 @@ extern "C" int cfp8_dequant_block128(const void* q, const float* scales, int64_t
     if (cols % 8) return set_error(CFP8_EINVAL, "dequant_block128: cols=%lld must be a multiple of 8", (long long)cols);
     if ((reinterpret_cast<uintptr_t>(q) & 7u) || !aligned16(y)) return set_error(CFP8_EINVAL, "dequant_block128: misaligned pointer");
     if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "dequant_block128: unknown out_dtype %d", out_dtype);
-    const int64_t blocks = (rows * (cols / 8) + 255) / 256;
-    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "dequant_block128: too large for one launch");
+    const int64_t nvec_row = cols / 8;
+    const int bx = nvec_row > 128 ? 256 : nvec_row > 64 ? 128 : 64, by = 256 / bx;
+    int64_t gx = (nvec_row + bx - 1) / bx, gy = (rows + 4 * by - 1) / (4 * by);
+    if (gx > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "dequant_block128: shape exceeds the grid limits");
+    if (gy > 65535) gy = 65535;  // the kernel strides over the remaining row quads
     if (int rc = check_device()) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int tc = (int)((cols + 127) / 128);
+    const dim3 grid((unsigned)gx, (unsigned)gy), block(bx, by);
     if (out_dtype == CFP8_OUT_F32)
-        hipLaunchKernelGGL((dequant_block128_kernel<float4, true>), dim3((unsigned)blocks), dim3(256), 0, st,
-                           static_cast<const uint8_t*>(q), scales, rows, cols, tc, y);
+        hipLaunchKernelGGL(dequant_block128_kernel<true>, grid, block, 0, st, static_cast<const uint8_t*>(q), scales, rows, cols,
+                           (int)nvec_row, tc, y);
     else
-        hipLaunchKernelGGL((dequant_block128_kernel<uint4, false>), dim3((unsigned)blocks), dim3(256), 0, st,
-                           static_cast<const uint8_t*>(q), scales, rows, cols, tc, y);
+        hipLaunchKernelGGL(dequant_block128_kernel<false>, grid, block, 0, st, static_cast<const uint8_t*>(q), scales, rows, cols,
+                           (int)nvec_row, tc, y);
     return check_launch("dequant_block128");
 }
