@@ -300,6 +300,24 @@ def test_block128_cfg4_and_dequant_roundtrip(dev):
     assert torch.equal(yb.cpu(), yo.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("shape", [(1, 8), (5, 24), (130, 520), (131, 1032), (257, 2056), (1048700, 8)])
+def test_weight_dequant_shapes(dev, shape):
+    """Ragged rows and columns at each block width of the dequantiser (64, 128, 256 vectors), and a matrix with
+    more row quads than the grid's y extent holds (the kernel then strides): bit-equal to the oracle, both dtypes."""
+    M, N = shape
+    g = torch.Generator().manual_seed(M * 31 + N)
+    q = torch.randint(0, 256, (M, N), generator=g, dtype=torch.uint8)
+    q[q == 0x7F] = 0x7E
+    q[q == 0xFF] = 0xFE
+    s = torch.rand((M + 127) // 128, (N + 127) // 128, generator=g) * 3e-3 + 1e-5
+    yo = O.weight_dequant(q, s)
+    qd = q.to(dev).view(torch.float8_e4m3fn)
+    y = ops.weight_dequant(qd, s.to(dev), out_dtype=torch.float32)
+    assert torch.equal(y.cpu(), yo)
+    yb = ops.weight_dequant(qd, s.to(dev), out_dtype=torch.bfloat16)
+    assert torch.equal(yb.cpu(), yo.to(torch.bfloat16))
+
+
 # ---------------------------------------------------------------------------- 1x128 groups
 @pytest.mark.parametrize("shape", [(4, 128), (33, 896), (7, 200), (1, 8), (129, 2048), (64, 7168)])
 def test_group128(dev, shape):
