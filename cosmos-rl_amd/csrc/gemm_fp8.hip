@@ -372,26 +372,37 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 // ---------------------------------------------------------------------------
 // Rowwise GEMM, large full tiles: 256 x 256 x 128 per workgroup, four wavefronts
 // (one per SIMD, 2 x 2), each owning a 128 x 128 block = 64 accumulators of
-// 16 x 16 (all 256 AGPRs).  With one wave per SIMD nothing hides a stall, so the
-// K step is written as a software pipeline of 32 groups of two MFMAs, each
-// group preceded by at most one global load or LDS store and one fragment read:
+// 16 x 16 (all 256 AGPRs).  Operand tiles go from global memory straight into
+// LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions).
+// Such a load puts lane l's 16 bytes at byte l * 16 of its 1 KiB destination, so
+// the LDS layout is dictated by which bytes each lane asks for: a stage is
+// row-major, row r at r * 128, and lane l of a load of 8 rows fetches chunk
+// (l & 7) ^ ((r >> 1) & 7) of row r = l >> 3.  Eight consecutive lanes then read
+// one whole 128-byte line of global memory, and the 16 rows of an MFMA fragment
+// read (ds_read_b128, one chunk per lane) fall into 16 different 16-byte bank
+// groups: coalesced on one side, conflict-free on the other.
+// With one wave per SIMD nothing hides a stall, so the K step is written as a
+// software pipeline of 32 groups of two MFMAs, each group preceded by at most
+// one direct-to-LDS load and one fragment read.  LDS holds two activation
+// stages and three weight stages of 32 KiB (all 160 KiB); step kt computes from
+// activation stage kt % 2 and weight stage kt % 3:
 //
-//   S0 (w0,x0): LDS reads x1          + stores of the staged tile kt+1 (first half)
-//   S1 (w0,x1): LDS reads w1          + stores (second half)
-//   -- wait for own LDS traffic, barrier: stage nxt complete, stage cur free --
-//   S2 (w1,x0): LDS reads next w0     + global loads of tile kt+2 (first half) -> registers
-//   S3 (w1,x1): LDS reads next x0     + global loads (second half)
+//   S0 (w0,x0): LDS reads x1
+//   S1 (w0,x1): LDS reads w1
+//   -- wait for all but the eight newest loads and for own LDS reads, barrier: tile kt+1 complete, both stages of tile kt free --
+//   S2 (w1,x0): LDS reads next w0     + loads of activation tile kt+2
+//   S3 (w1,x1): LDS reads next x0     + loads of weight tile kt+3 (the eight newest at the next barrier)
 //
-// so a global load has a full K step (~2048 MFMA cycles) to land before its LDS
-// store, and every fragment is read at least 16 MFMAs before its first use.
+// so an activation load has one K step (~2048 MFMA cycles) to land and a weight
+// load two (weights come from HBM, activations mostly from the caches), and
+// every fragment is read at least 16 MFMAs before its first use.  The tile's
+// row scales are fetched the same way into the activation stage that no tile
+// needs any more, one and a half steps before the epilogue.
 // The epilogue turns each wave's block through LDS so that every global store
 // is 16 bytes per lane and 256 contiguous bytes per output row, non-temporal
 // (the output must not evict operand tiles from L2).
 // Requires M % 256 == 0 and N % 256 == 0 (every address is then a per-lane part
 // plus a wave-uniform part).
-// Measured on config 3, M = 8192: 2.05 PFLOP/s against 1.55 for the 8-wave
-// kernel above; a variant with direct-to-LDS loads (global_load_lds_dwordx4) was
-// correct but slower: each such load holds the wave's issue for > 100 cycles.
 // ---------------------------------------------------------------------------
 #define CFP8_PHASE_END() __builtin_amdgcn_sched_barrier(0)
 #define CFP8_MMA2(wb, wh, xb, xh, g)                                                                   \
@@ -406,7 +417,8 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 template <bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p) {
     constexpr int BM = 256, BN = 256;
-    constexpr int STAGE = (BM + BN) * 128;  // 64 KiB
+    constexpr int XS = BM * 128, WS = BN * 128;  // one activation / weight stage: 32 KiB each
+    constexpr int WBASE = 2 * XS;                // LDS: two activation stages, then three weight stages = 160 KiB
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     int tm, tn;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -416,33 +428,30 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     const int wm = wave & 1, wn = wave >> 1;
     const int lrow = lane & 15, quarter = lane >> 4;
     const int KT = p.K >> 7;
+    const int last = KT - 1;
 
-    // global -> registers -> LDS.  Per K step 64 wave-wide loads of 1 KiB (8 rows x 128 B): wave w
-    // takes u = w, w + 4, ...; u < 32: activation rows u * 8 .., u >= 32: weight rows (u - 32) * 8 ..
-    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
-    // Wave-uniform bases and strides of this wave's row blocks (u >> 1 = (wave >> 1) + 2 i).  They pass
-    // through an empty asm so that the compiler keeps them in SGPRs for the whole K loop: left alone it
-    // re-reads the kernel arguments inside the loop, and every scalar load has to be waited for with
-    // lgkmcnt(0), which drains the LDS queue of the fragment reads in flight.
-    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_a;
-    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_b;
+    // Direct-to-LDS load i (0..7) of one operand's K step covers rows (wave + 4 i) * 8 .. + 7 of the tile.
+    // The wave-uniform bases and strides pass through an empty asm so that the compiler keeps them in SGPRs for
+    // the whole K loop: left alone it re-reads the kernel arguments inside the loop, and every scalar load has to be
+    // waited for with lgkmcnt(0), which drains the LDS queue of the fragment reads in flight.
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
     uint32_t a_step = 32u * (uint32_t)p.ld_a, b_step = 32u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
     asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));
-    const int uodd = wave & 1;  // u & 1 is the same for all of a wave's loads
-    const uint32_t va_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_a + (uint32_t)(st_c * 16);
-    const uint32_t vb_lane = (uint32_t)(uodd * 8 + st_row8) * (uint32_t)p.ld_b + (uint32_t)(st_c * 16);
-    const int l_lane = lds_chunk_offset(uodd * 8 + st_row8, st_c);
-    i32x4 R[16];  // ext-vector type on purpose: an array of uint4 structs stays in scratch memory
-    auto gload = [&](int kt, int i) {  // i < 8: activation rows, i >= 8: weight rows (wave < 4)
-        const uint64_t base = (i < 8 ? a_wave + (uint64_t)i * a_step : b_wave + (uint64_t)(i - 8) * b_step) + ((uint64_t)kt << 7);
-        // an address built from an integer must be told that it is global memory (else: flat loads)
-        typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
-        typedef const __attribute__((address_space(1))) i32x4* gvec_t;
-        R[i] = *(gvec_t)((gptr_t)base + (i < 8 ? va_lane : vb_lane));
+    // (r >> 1) & 7 of row r = (wave + 4 i) * 8 + (lane >> 3) is (wave & 1) * 4 + (lane >> 4)
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;  // an address built from an integer must be told that it is global memory
+    auto dma_x = [&](int kt, int stage, int i) {
+        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, 0, 0);
     };
-    auto lstore = [&](int stage, int i) {
-        const int u = wave + 4 * i, isB = u >> 5, rb = (u & 31) >> 1;
-        *reinterpret_cast<i32x4*>(smem + stage * STAGE + isB * (BM * 128) + rb * 2048 + l_lane) = R[i];
+    auto dma_w = [&](int kt, int stage, int i) {
+        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, 0, 0);
     };
 
     f32x4 acc[8][8];  // [n tile][m tile]
@@ -451,12 +460,14 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int x_off = lds_chunk_offset(wm * 128 + lrow, 2 * quarter);
-    const int x_off2 = lds_chunk_offset(wm * 128 + lrow, 2 * quarter + 1);
-    const int w_off = BM * 128 + lds_chunk_offset(wn * 128 + lrow, 2 * quarter);
-    const int w_off2 = BM * 128 + lds_chunk_offset(wn * 128 + lrow, 2 * quarter + 1);
-    auto frag = [&](int stage, int off, int off2, int tile16) {
-        const uint8_t* base = smem + stage * STAGE + tile16 * 2048;
+    // fragment of 16 rows: lane (lrow, quarter) reads chunks 2 quarter and 2 quarter + 1 of its row
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
         const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
         const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
         i32x8 r;
@@ -466,40 +477,18 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     };
     i32x8 W[2][4], X[2][4];  // weight / activation fragments of the two halves of the wave's block
 
-    // prologue: tile 0 -> stage 0 (through registers); tile 1: activation half -> stage 1, weight half stays
-    // in registers 8..15; activation half of tile 2 -> registers 0..7
-    const int last = KT - 1;
-    // The tile's 256 activation scales and 256 weight scales go to LDS behind the two stages now, so that the
-    // epilogue does not start with a global round trip.
-    float* const scale_lds = reinterpret_cast<float*>(smem + 2 * STAGE);  // [0, 256): sa, [256, 512): sb
-    {
-        const float s_a = p.sa[m0 + t], s_b = p.sb[n0 + t];
-        scale_lds[t] = s_a;
-        scale_lds[256 + t] = s_b;
-    }
-    // (tiles 0 and 1 are requested together: the fragment registers are still free to hold tile 0)
-    {
-        i32x4 T0[16];
+    // prologue: activation tiles 0, 1 and weight tiles 0, 1, 2 into their stages
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            gload(0, i);
-            T0[i] = R[i];
-        }
+    for (int i = 0; i < 8; ++i) dma_x(0, 0, i);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) gload(1 < last ? 1 : last, i);
-        CFP8_PHASE_END();
+    for (int i = 0; i < 8; ++i) dma_w(0, 0, i);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const i32x4 keep = R[i];
-            R[i] = T0[i];
-            lstore(0, i);
-            R[i] = keep;
-        }
-    }
+    for (int i = 0; i < 8; ++i) dma_x(1 < last ? 1 : last, 1, i);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) lstore(1, i);
+    for (int i = 0; i < 8; ++i) dma_w(1 < last ? 1 : last, 1, i);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) gload(2 < last ? 2 : last, i);
+    for (int i = 0; i < 8; ++i) dma_w(2 < last ? 2 : last, 2, i);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -508,47 +497,57 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     }
     CFP8_PHASE_END();
 
+    // Step kt computes from activation stage kt % 2 and weight stage kt % 3.  After its barrier nobody reads either
+    // any more: activation tile kt + 2 and then weight tile kt + 3 are requested into them.  The next barrier needs
+    // activation tile kt + 2 and weight tile kt + 2 (requested a step earlier), i.e. everything but the eight newest
+    // loads: an activation load has one K step to land, a weight load two.
+    int ws_cur = 0;  // kt % 3
+    const int scale_step = last > 0 ? last - 1 : 0;
     for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1, nxt = cur ^ 1;
-        // past the end: re-read the last tile, never consumed
-        const int kb = kt + 2 < last ? kt + 2 : last;  // weight half, loaded in S0/S1
-        const int ka = kt + 3 < last ? kt + 3 : last;  // activation half, loaded in S2/S3
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ws_cur == 2 ? 0 : ws_cur + 1;
+        const int kw = kt + 3 < last ? kt + 3 : last;  // past the end: the last tile again, never consumed
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g < 4) X[1][g] = frag(cur, x_off, x_off2, 4 + g);
-            if (g & 1) gload(kb, 8 + (g >> 1));
-            else lstore(nxt, 8 + (g >> 1));
+            if (g < 4) X[1][g] = frag(xs_cur, x_off, x_off2, 4 + g);
             CFP8_MMA2(0, 0, 0, 0, g);
             CFP8_PHASE_END();
         }
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g < 4) W[1][g] = frag(cur, w_off, w_off2, 4 + g);
-            if (g & 1) gload(kb, 12 + (g >> 1));
-            else lstore(nxt, 12 + (g >> 1));
+            if (g < 4) W[1][g] = frag(ws_cur * WS, w_off, w_off2, 4 + g);
             CFP8_MMA2(0, 0, 1, 1, g);
             CFP8_PHASE_END();
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         CFP8_PHASE_END();
+        if (kt == scale_step) {
+            // no activation tile goes into stage (last + 1) % 2 any more: it takes the tile's 256 activation scales and
+            // 256 weight scales for the epilogue (64 of each per wave, 4 bytes per lane), a step and a half ahead
+            uint8_t* dst = smem + ((last + 1) & 1) * XS + wave * 256;
+            __builtin_amdgcn_global_load_lds((gbl_void*)(p.sa + m0 + wave * 64 + lane), (lds_void*)dst, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_void*)(p.sb + n0 + wave * 64 + lane), (lds_void*)(dst + 1024), 4, 0, 0);
+        }
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g < 4) W[0][g] = frag(nxt, w_off, w_off2, g);  // after the last step: stale data, unused
-            if (g & 1) gload(ka, g >> 1);
-            else lstore(cur, g >> 1);
+            if (g < 4) W[0][g] = frag(ws_nxt * WS, w_off, w_off2, g);  // after the last step: stale data, unused
+            if (kt + 2 <= last) dma_x(kt + 2, kt & 1, g);
             CFP8_MMA2(1, 1, 0, 0, g);
             CFP8_PHASE_END();
         }
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g < 4) X[0][g] = frag(nxt, x_off, x_off2, g);
-            if (g & 1) gload(ka, 4 + (g >> 1));
-            else lstore(cur, 4 + (g >> 1));
+            if (g < 4) X[0][g] = frag(xs_nxt, x_off, x_off2, g);
+            dma_w(kw, ws_cur, g);
             CFP8_MMA2(1, 1, 1, 1, g);
             CFP8_PHASE_END();
         }
+        ws_cur = ws_nxt;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the scales have landed, and nothing may still land in the stages
+    __syncthreads();
+    const float* const scale_lds = reinterpret_cast<const float*>(smem + ((last + 1) & 1) * XS);  // [0, 256): sa, [256, 512): sb
 
     float sam[8];
 #pragma unroll
@@ -577,7 +576,7 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     for (int i = 0; i < 8; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(scale_lds + 256 + wn * 128 + i * 16 + quarter * 4);
     __syncthreads();  // all waves are done reading the operand stages
     constexpr int EST = 272;
-    uint8_t* const ebuf = smem + wave * (64 * EST);
+    uint8_t* const ebuf = smem + WBASE + wave * (64 * EST);  // in the weight stages: the scales sit in an activation stage
     const int rd_row = lane >> 4, rd_chunk = lane & 15;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -943,7 +942,7 @@ static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 256;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
-    constexpr size_t lds = (size_t)2 * 512 * 128 + 2 * 256 * sizeof(float);  // two operand stages + the tile's scales
+    constexpr size_t lds = (size_t)(2 + 3) * 256 * 128;  // two activation stages and three weight stages: all 160 KiB
     static std::atomic<bool> raised[65][2];  // zero-initialised
     const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
     const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256_kernel<true>)

@@ -41,8 +41,9 @@ def rowwise_operands(M, N, K, seed, dev):
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 64, 256), (17, 80, 384), (64, 128, 512), (100, 272, 896),
                                    (128, 128, 128), (200, 272, 384), (256, 512, 256), (300, 1024, 1024), (513, 528, 640),
                                    (1024, 768, 3584),
-                                   # full 256x256 tiles: the four-wave pipelined kernel, K of 1, 3 and 28 steps
-                                   (768, 256, 128), (1024, 512, 384), (2048, 1280, 896),
+                                   # full 256x256 tiles: the four-wave pipelined kernel (two activation and three weight
+                                   # stages in LDS), K of 1, 2, 3, 4, 5 and 7 steps
+                                   (768, 256, 128), (1024, 512, 384), (2048, 1280, 896), (768, 512, 512), (1024, 256, 640),
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
                                    (2048, 8448, 256),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
