@@ -630,7 +630,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     static_assert(!SWIGLU || (MODE == kGrouped && BN == 256 && !OUT_F32), "the SwiGLU epilogue belongs to the grouped 128 x 256 tile");
     static_assert(MODE == kBlock || MODE == kGrouped, "block-scaled modes only");
     constexpr int WM = BM / 64;
-    constexpr int STAGE = (BM + BN) * 128;  // 48 KiB
+    constexpr int XS = BM * 128, WS = BN * 128;  // one activation / weight stage
+    constexpr int WBASE = 2 * XS;                // LDS: two activation stages, three weight stages, then the scales
+    constexpr int SBASE = WBASE + 3 * WS;
     constexpr int A_IT = BM / 64, B_IT = BN / 64;  // wave-wide loads (8 rows x 128 B) per wave and K step: 4 + 2 or 2 + 4
     constexpr int NB = BN / 128;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -653,28 +655,29 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     const int KT = p.K >> 7;
     const int last = KT - 1;
 
-    // global -> registers -> LDS: wave w takes the 16-row blocks (w >> 1) + 4 i of each operand, the half (w & 1) of them
-    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
-    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_a;
-    uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)(wave >> 1) * 16) * (uint64_t)p.ld_b;
+    // global -> LDS directly (as in gemm_rowwise_256_kernel: row-major stages, 16-byte chunks XOR-ed by (row >> 1) & 7):
+    // load i of an operand's K step covers rows (wave + 8 i) * 8 .. + 7 of its tile
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
     uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
     asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));  // keep them in SGPRs for the whole loop
-    const uint32_t va_lane = (uint32_t)((wave & 1) * 8 + st_row8) * (uint32_t)p.ld_a + (uint32_t)(st_c * 16);
-    const uint32_t vb_lane = (uint32_t)((wave & 1) * 8 + st_row8) * (uint32_t)p.ld_b + (uint32_t)(st_c * 16);
-    const int l_lane = lds_chunk_offset((wave & 1) * 8 + st_row8, st_c) + (wave >> 1) * 2048;
-    i32x4 R[6];
-    auto gload = [&](int kt, int i) {
-        const uint64_t base = (i < A_IT ? a_wave + (uint64_t)i * a_step : b_wave + (uint64_t)(i - A_IT) * b_step) + ((uint64_t)kt << 7);
-        typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
-        typedef const __attribute__((address_space(1))) i32x4* gvec_t;
-        R[i] = *(gvec_t)((gptr_t)base + (i < A_IT ? va_lane : vb_lane));
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+    auto dma_x = [&](int kt, int stage, int i) {
+        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, 0, 0);
     };
-    auto lstore = [&](int stage, int i) {
-        *reinterpret_cast<i32x4*>(smem + stage * STAGE + (i < A_IT ? i * 8192 : BM * 128 + (i - A_IT) * 8192) + l_lane) = R[i];
+    auto dma_w = [&](int kt, int stage, int i) {
+        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, 0, 0);
     };
 
     // activation scales: 8 K steps of this tile's rows per fetch, 4 consecutive floats per thread
-    float* const sg_buf = reinterpret_cast<float*>(smem + 2 * STAGE);  // [2][8][BM]
+    float* const sg_buf = reinterpret_cast<float*>(smem + SBASE);  // [2][8][BM]
     float* const sn_lds = sg_buf + 2 * 8 * BM;                         // [KT][NB]
     const int sg_row = t >> 1, sg_half = t & 1;
     const float* const sg_ptr = p.sa + (int64_t)(m0 + (sg_row < BM ? sg_row : BM - 1)) * KT;
@@ -704,12 +707,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         P[1][i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const int x_off = lds_chunk_offset(wm * 64 + lrow, 2 * quarter);
-    const int x_off2 = lds_chunk_offset(wm * 64 + lrow, 2 * quarter + 1);
-    const int w_off = BM * 128 + lds_chunk_offset(wn * 64 + lrow, 2 * quarter);
-    const int w_off2 = BM * 128 + lds_chunk_offset(wn * 64 + lrow, 2 * quarter + 1);
-    auto frag = [&](int stage, int off, int off2, int tile16) {
-        const uint8_t* base = smem + stage * STAGE + tile16 * 2048;
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
         const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
         const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
         i32x8 r;
@@ -727,31 +731,24 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
     };
 
-    // prologue: scales, then tiles 0 and 1 requested together; tile 0 goes to stage 0, tile 1 stays in R
+    // prologue: activation tiles 0, 1 and weight tiles 0, 1, 2 into their stages, and the scales
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) dma_w(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) dma_w(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < B_IT; ++i) dma_w(2 < last ? 2 : last, 2, i);
     sg_load(0);
     for (int idx = t; idx < KT * NB; idx += 512) {
         const int k = idx / NB, nb = idx - k * NB;
         sn_lds[idx] = sbp[(int64_t)((n0 >> 7) + nb) * p.sb_stride_n + (int64_t)k * p.sb_stride_k];
     }
-    {
-        i32x4 T0[6];
-#pragma unroll
-        for (int i = 0; i < 6; ++i) {
-            gload(0, i);
-            T0[i] = R[i];
-        }
-#pragma unroll
-        for (int i = 0; i < 6; ++i) gload(1 < last ? 1 : last, i);
-        CFP8_PHASE_END();
-        sg_store(0);
-#pragma unroll
-        for (int i = 0; i < 6; ++i) {
-            const i32x4 keep = R[i];
-            R[i] = T0[i];
-            lstore(0, i);
-            R[i] = keep;
-        }
-    }
+    sg_store(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     // (the same order as in the loop's tail: the compiler merges both when it counts outstanding reads at the loop head)
     X[0] = frag(0, x_off, x_off2, 0);
@@ -770,14 +767,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(P[pj][i][e], sc, acc[i][j][e])
 #define CFP8_PRODUCT(i, j, pj) \
     P[pj][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[j], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0)
+    // Step kt computes from activation stage kt % 2 and weight stage kt % 3; behind its barrier activation tile kt + 2
+    // and then weight tile kt + 3 are requested into them.  The next barrier needs everything but those B_IT newest
+    // loads: an activation load has one K step to land, a weight load two.
+    int ws_cur = 0;  // kt % 3
     for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1, nxt = cur ^ 1;
-        const int kl = kt + 2 < last ? kt + 2 : last;  // past the end: re-read the last tile, never consumed
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ws_cur == 2 ? 0 : ws_cur + 1;
+        const int kx = kt + 2 < last ? kt + 2 : last;  // past the end: the last tile again, never consumed
+        const int kw = kt + 3 < last ? kt + 3 : last;
         // group 0
-        X[2] = frag(cur, x_off, x_off2, 2);
-        lstore(nxt, 0);
-        lstore(nxt, 1);
-        lstore(nxt, 2);
+        X[2] = frag(xs_cur, x_off, x_off2, 2);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             CFP8_RESCALE(i, 2, 0, sc2p);
@@ -785,13 +785,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
         CFP8_PHASE_END();
         // group 1
-        X[3] = frag(cur, x_off, x_off2, 3);
-        lstore(nxt, 3);
-        lstore(nxt, 4);
-        lstore(nxt, 5);
-        gload(kl, 0);
-        gload(kl, 1);
-        gload(kl, 2);
+        X[3] = frag(xs_cur, x_off, x_off2, 3);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             CFP8_RESCALE(i, 3, 1, sc3p);
@@ -799,17 +793,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
         if ((kt & 7) == 7) sg_store((kt >> 3) + 1);
         CFP8_PHASE_END();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (B_IT == 2) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         CFP8_PHASE_END();
         // tail
         const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
         sc2p = sm[2] * s_n;
         sc3p = sm[3] * s_n;
-        X[0] = frag(nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
-        gload(kl, 3);
-        gload(kl, 4);
-        gload(kl, 5);
+        X[0] = frag(xs_nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
+#pragma unroll
+        for (int i = 0; i < A_IT; ++i) dma_x(kx, kt & 1, i);
         if ((kt & 7) == 6) sg_load((kt >> 3) + 1);
         CFP8_PHASE_END();
 #pragma unroll
@@ -819,13 +813,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             CFP8_PRODUCT(i, 2, 0);
             CFP8_PRODUCT(i, 3, 1);
             CFP8_PHASE_END();
-            W[i] = frag(nxt, w_off, w_off2, i);
+            W[i] = frag(ws_nxt * WS, w_off, w_off2, i);
+            if (i < B_IT) dma_w(kw, ws_cur, i);
             CFP8_PHASE_END();
         }
-        X[1] = frag(nxt, x_off, x_off2, 1);
+        X[1] = frag(xs_nxt, x_off, x_off2, 1);
         read_scales(kt + 1);
         CFP8_PHASE_END();
+        ws_cur = ws_nxt;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in the stages: the epilogues reuse them
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         CFP8_RESCALE(i, 2, 0, sc2p);
@@ -1417,8 +1414,8 @@ static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_n = p.N / BN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
-    // two operand stages, the turned activation scales of two groups of 8 K steps, the tile's weight scales
-    const size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
+    // two activation and three weight stages, the turned activation scales of two groups of 8 K steps, the tile's weight scales
+    const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
     const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
     using Kern = void (*)(const GemmArgs);
     const Kern table[2][2] = {{gemm_block_w8_kernel<BM, BN, MODE, false, false>, gemm_block_w8_kernel<BM, BN, MODE, true, false>},
@@ -1426,7 +1423,7 @@ static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int f32 = out_dtype == CFP8_OUT_F32;
     const Kern kern = table[vec][f32];
     // the limit is raised to the largest size this kernel can ask for, once per device and instantiation
-    constexpr size_t lds_max = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
+    constexpr size_t lds_max = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
     static std::atomic<bool> done[65][2][2];  // zero-initialised
     const int slot = device_slot();
     if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
@@ -1442,12 +1439,12 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     p.tiles_n = p.N / BN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
-    const size_t lds = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
+    const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
     const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
     using Kern = void (*)(const GemmArgs);
     const Kern kern = vec ? static_cast<Kern>(gemm_block_w8_kernel<BM, BN, kGrouped, false, true, true>)
                           : static_cast<Kern>(gemm_block_w8_kernel<BM, BN, kGrouped, false, false, true>);
-    constexpr size_t lds_max = (size_t)2 * (BM + BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
+    constexpr size_t lds_max = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + kMaxTileWeightScales * sizeof(float);
     static std::atomic<bool> done[65][2];  // zero-initialised
     const int slot = device_slot();
     if (slot == 64) done[64][vec].store(false, std::memory_order_relaxed);
