@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     for (int i = 0; i < 8; ++i) dma_w(1 < last ? 1 : last, 1, i);
 #pragma unroll
     for (int i = 0; i < 8; ++i) dma_w(2 < last ? 2 : last, 2, i);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(24)" ::: "memory");  // tile 0 has landed; the other three loads stay in flight
     __syncthreads();
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -607,14 +607,16 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 // ---------------------------------------------------------------------------
 // Block-scaled and grouped GEMM, full tiles: 256 x 128 (block) or 128 x 256 (grouped, whose groups are
 // 128 rows) x 128 per workgroup, eight wavefronts (two per SIMD), each a 64 x 64 block = 4 x tiles
-// times 4 w tiles.  One wave keeps only one LDS instruction in progress at a time, so the K step is
-// laid out around its LDS queue:
+// times 4 w tiles.  Operand tiles go straight from global memory into LDS as in gemm_rowwise_256_kernel
+// (row-major stages with XOR-ed chunks; two activation stages and three weight stages).  One wave keeps
+// only one LDS instruction in progress at a time, so the K step is laid out around its LDS queue:
 //
-//   group 0: read x2 | 3 LDS stores of tile kt+1 | per w tile i: rescale of last step's (i, x2), MFMA (i, x0)
-//   group 1: read x3 | 3 LDS stores, 3 global loads of tile kt+2 | per i: rescale of last step's (i, x3), MFMA (i, x1)
-//   wait for own LDS traffic, barrier: stage nxt complete, stage cur free
-//   tail:    next step's x0 | 3 global loads | per i: rescale of (i, x0), (i, x1), MFMAs (i, x2), (i, x3),
-//            then next step's w tile i into the registers those MFMAs just consumed; next step's x1 and scales
+//   group 0: read x2 | per w tile i: rescale of last step's (i, x2), MFMA (i, x0)
+//   group 1: read x3 | per i: rescale of last step's (i, x3), MFMA (i, x1)
+//   wait for all but the newest weight loads and for own LDS reads, barrier: tile kt+1 complete, tile kt's stages free
+//   tail:    next step's x0 | loads of activation tile kt+2 | per i: rescale of (i, x0), (i, x1), MFMAs (i, x2), (i, x3),
+//            then next step's w tile i into the registers those MFMAs just consumed and a load of weight tile kt+3;
+//            next step's x1 and scales
 //
 // No MFMA after the barrier waits for LDS, every rescale (acc += products * s_m * s_n, VALU) reads MFMA
 // results issued at least five MFMAs earlier, and the first MFMAs of a step find their fragments read
@@ -731,7 +733,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
     };
 
-    // prologue: activation tiles 0, 1 and weight tiles 0, 1, 2 into their stages, and the scales
+    // prologue: activation tiles 0, 1 and weight tiles 0, 1, 2 into their stages, and the scales.  (The compiler waits
+    // for every direct-to-LDS load in flight before an LDS store, here those of the scales: it cannot tell that they
+    // go elsewhere.  So everything is requested at once and awaited together.)
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) dma_x(0, 0, i);
 #pragma unroll
@@ -791,20 +795,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             CFP8_RESCALE(i, 3, 1, sc3p);
             CFP8_PRODUCT(i, 1, 1);
         }
-        if ((kt & 7) == 7) sg_store((kt >> 3) + 1);
         CFP8_PHASE_END();
         if (B_IT == 2) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         CFP8_PHASE_END();
-        // tail
+        // tail.  The next group's activation scales are stored here, before this step's loads are requested: the
+        // compiler makes an LDS store wait for every direct-to-LDS load in flight (it cannot tell that they go
+        // elsewhere), and at this point only the weight loads of the previous step are, a whole step old.  The scales
+        // were fetched a step earlier and are first read two barriers later, at the end of step 8 g + 7.
+        if ((kt & 7) == 6) sg_store((kt >> 3) + 1);
         const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
         sc2p = sm[2] * s_n;
         sc3p = sm[3] * s_n;
         X[0] = frag(xs_nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) dma_x(kx, kt & 1, i);
-        if ((kt & 7) == 6) sg_load((kt >> 3) + 1);
+        if ((kt & 7) == 5) sg_load((kt >> 3) + 1);
         CFP8_PHASE_END();
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
