@@ -64,6 +64,28 @@ def test_scaled_mm_rowwise(dev, M, N, K):
     check_bf16(out16, ref, f"rowwise {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(768, 512, 384), (1024, 768, 1024)])
+def test_scaled_mm_rowwise_pitched_operands(dev, M, N, K):
+    """The 256x256 kernel fetches its tiles with per-lane addresses built from the leading dimensions: operands that are
+    column slices of wider buffers (row pitch K + 128 and K + 256, data pointers offset into the buffer) give the
+    same result as contiguous ones."""
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K + 7, dev=dev)
+    ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
+    abuf = torch.full((M, K + 128), 0x7E, dtype=torch.uint8, device=dev)   # neighbours hold 448.0: a wrong pitch shows
+    bbuf = torch.full((N, K + 256), 0x7E, dtype=torch.uint8, device=dev)
+    abuf[:, 64:64 + K] = qx.to(dev)
+    bbuf[:, 128:128 + K] = qw.to(dev)
+    a = abuf.view(torch.float8_e4m3fn)[:, 64:64 + K]
+    b = bbuf.view(torch.float8_e4m3fn)[:, 128:128 + K]
+    assert a.stride(0) == K + 128 and b.stride(0) == K + 256
+    out32 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    assert O.rel_frobenius(out32.cpu(), ref) <= TIGHT
+    same = ops.scaled_mm(f8(qx, dev), f8(qw, dev).t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    assert torch.equal(out32, same)
+    out16 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.bfloat16)
+    check_bf16(out16, ref, f"pitched rowwise {M}x{N}x{K}")
+
+
 def test_scaled_mm_one_hot_and_pow2(dev):
     """One-hot activation rows reproduce single weight entries exactly; power-of-two scales make
     the epilogue exact, so the fp32 output must equal the oracle bit for bit."""
