@@ -646,15 +646,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     int tm, tn;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const uint8_t* bptr = p.b;
-    const float* sbp = p.sb;
-    int expert = 0;
-    if (MODE == kGrouped) {
-        expert = p.m_indices[m0];  // groups start on multiples of 128 = BM rows
-        if (expert < 0) return;    // a tile of padding (uniform for the workgroup)
-        bptr += (int64_t)expert * p.N * p.ld_b;
-        sbp += (int64_t)expert * p.sb_stride_e;
-    }
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave % WM, wn = wave / WM;
@@ -665,9 +656,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     // global -> LDS directly (as in gemm_rowwise_256_kernel: row-major stages, 16-byte chunks XOR-ed by (row >> 1) & 7):
     // load i of an operand's K step covers rows (wave + 8 i) * 8 .. + 7 of its tile
     uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
-    uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
     uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
-    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));  // keep them in SGPRs for the whole loop
+    asm volatile("" : "+s"(a_wave), "+s"(a_step), "+s"(b_step));  // keep them in SGPRs for the whole loop
     const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
     const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
@@ -678,6 +668,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
         __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, 0, 0);
     };
+    // The activation tiles do not depend on the group: in the grouped form they are requested before the group's
+    // expert is known (one dependent scalar load less in front of the first tile).
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(1 < last ? 1 : last, 1, i);
+    const uint8_t* bptr = p.b;
+    const float* sbp = p.sb;
+    int expert = 0;
+    if (MODE == kGrouped) {
+        expert = p.m_indices[m0];  // groups start on multiples of 128 = BM rows
+        if (expert < 0) {          // a tile of padding (uniform for the workgroup)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS once the workgroup has gone
+            return;
+        }
+        bptr += (int64_t)expert * p.N * p.ld_b;
+        sbp += (int64_t)expert * p.sb_stride_e;
+    }
+    uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+    asm volatile("" : "+s"(b_wave));
     auto dma_w = [&](int kt, int stage, int i) {
         const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
         __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, 0, 0);
@@ -738,15 +748,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
     };
 
-    // prologue: activation tiles 0, 1 and weight tiles 0, 1, 2 into their stages, and the scales.  (The compiler waits
+    // prologue: (activation tiles 0 and 1 are under way) weight tiles 0, 1, 2 into their stages, and the scales.  (The compiler waits
     // for every direct-to-LDS load in flight before an LDS store, here those of the scales: it cannot tell that they
     // go elsewhere.  So everything is requested at once and awaited together.)
 #pragma unroll
-    for (int i = 0; i < A_IT; ++i) dma_x(0, 0, i);
-#pragma unroll
     for (int i = 0; i < B_IT; ++i) dma_w(0, 0, i);
-#pragma unroll
-    for (int i = 0; i < A_IT; ++i) dma_x(1 < last ? 1 : last, 1, i);
 #pragma unroll
     for (int i = 0; i < B_IT; ++i) dma_w(1 < last ? 1 : last, 1, i);
 #pragma unroll
