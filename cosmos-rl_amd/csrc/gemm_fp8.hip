@@ -294,7 +294,21 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
         __syncthreads();
     }
 
-    // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+    // epilogue: lane holds out[m][n .. n+3] for every (i, j).  Everything the epilogue reads from global memory (row
+    // and column scales, which rows belong to the group) is read before its first store: loads and stores share one
+    // counter, so a load behind a store waits for the store's acknowledgement.
+    float sam[TM];
+    f32x4 sbn[TN];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int m = m0 + wm * WTM + j * 16 + lrow;
+        sam[j] = (MODE == kRowwise && m < p.M) ? p.sa[m] : 1.f;
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        const int n = n0 + wn * WTN + i * 16 + quarter * 4;
+        sbn[i] = (MODE == kRowwise && n < p.N) ? *reinterpret_cast<const f32x4*>(p.sb + n) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
     if constexpr (!OUT_F32 && BM >= 128) {
         // bf16, large tiles: scale, convert and turn the wave's block through LDS so that global
         // stores are 16 bytes per lane, a full row segment of the wave's block at a time, and
@@ -304,24 +318,30 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
         constexpr int RPI = 64 / LPR;                 // rows per wave-wide store
         constexpr int HR = WTM / 2;                   // the block goes through LDS in two halves of HR rows
         static_assert(HR % 16 == 0 && WM * WN * HR * EST <= 2 * (BM + BN) * 128, "epilogue buffer must fit the operand stages");
-        __syncthreads();                              // every wave is done reading the operand stages
         uint8_t* const ebuf = smem + wave * (HR * EST);
         const int rd_row = lane / LPR, rd_chunk = lane % LPR;
+        bool keep[2][HR / RPI];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < HR / RPI; ++r) {
+                const int m = m0 + wm * WTM + h * HR + r * RPI + rd_row, n = n0 + wn * WTN + rd_chunk * 8;
+                bool ok = m < p.M && n < p.N;         // N % 16 == 0: an 8-wide chunk is inside or outside as a whole
+                if (MODE == kGrouped && ok) ok = p.m_indices[m] == expert;
+                keep[h][r] = ok;
+            }
+        __syncthreads();                              // every wave is done reading the operand stages
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
             for (int jj = 0; jj < TM / 2; ++jj) {
                 const int j = h * (TM / 2) + jj;
-                const int m = m0 + wm * WTM + j * 16 + lrow;
-                const float sam = (MODE == kRowwise && m < p.M) ? p.sa[m] : 1.f;
 #pragma unroll
                 for (int i = 0; i < TN; ++i) {
                     f32x4 v = acc[i][j];
                     if (MODE == kRowwise) {
-                        const int n = n0 + wn * WTN + i * 16 + quarter * 4;
-                        const f32x4 sbn = n < p.N ? *reinterpret_cast<const f32x4*>(p.sb + n) : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = v[e] * sam * sbn[e];
+                        for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
                     }
                     *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
                         make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -332,9 +352,7 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
             for (int r = 0; r < HR / RPI; ++r) {
                 const int row = r * RPI + rd_row;
                 const int m = m0 + wm * WTM + h * HR + row, n = n0 + wn * WTN + rd_chunk * 8;
-                bool ok = m < p.M && n < p.N;         // N % 16 == 0: an 8-wide chunk is inside or outside as a whole
-                if (MODE == kGrouped && ok) ok = p.m_indices[m] == expert;
-                if (ok) {
+                if (keep[h][r]) {
                     const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
                     __builtin_nontemporal_store(d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n));
                 }
@@ -342,22 +360,25 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
         }
         return;
     }
+    bool keep[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + wm * WTM + j * 16 + lrow;
-        if (m >= p.M) continue;
-        if (MODE == kGrouped && p.m_indices[m] != expert) continue;
-        float sam = 1.f;
-        if (MODE == kRowwise) sam = p.sa[m];
+        keep[j] = m < p.M;
+        if (MODE == kGrouped && keep[j]) keep[j] = p.m_indices[m] == expert;
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int m = m0 + wm * WTM + j * 16 + lrow;
+        if (!keep[j]) continue;
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
             const int n = n0 + wn * WTN + i * 16 + quarter * 4;
             if (n >= p.N) continue;  // N % 16 == 0: a group of four is inside or outside as a whole
             f32x4 v = acc[i][j];
             if (MODE == kRowwise) {
-                const f32x4 sbn = *reinterpret_cast<const f32x4*>(p.sb + n);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam * sbn[e];
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
             }
             if (OUT_F32) {
                 *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
@@ -895,10 +916,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         return;
     }
     if (OUT_F32) {
+        // (which rows belong to the group is read before the first store: a load behind a store would have to wait
+        // for the store's acknowledgement, loads and stores share one counter)
+        bool keep[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) keep[j] = MODE != kGrouped || p.m_indices[m0 + wm * 64 + j * 16 + lrow] == expert;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int m = m0 + wm * 64 + j * 16 + lrow;
-            if (MODE == kGrouped && p.m_indices[m] != expert) continue;
+            if (!keep[j]) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int n = n0 + wn * 64 + i * 16 + quarter * 4;
@@ -909,10 +935,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
     // bf16: turn the wave's 64 x 64 block through LDS in two halves of 32 rows (row stride 144 B), so that
     // global stores are 16 bytes per lane and 128 contiguous bytes per row, non-temporal
-    __syncthreads();  // all waves are done reading the operand stages
     constexpr int EST = 144;
     uint8_t* const ebuf = smem + wave * (32 * EST);
     const int rd_row = lane >> 3, rd_chunk = lane & 7;
+    // Which of this lane's eight output rows belong to the group is read now, before the first store: loads and
+    // stores share one counter, so a load behind a store waits for the store's acknowledgement - per row, that
+    // was most of a short-K tile's epilogue.
+    bool keep[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            keep[h][r] = MODE != kGrouped || p.m_indices[m0 + wm * 64 + h * 32 + r * 8 + rd_row] == expert;
+    __syncthreads();  // all waves are done reading the operand stages
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -930,7 +965,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         for (int r = 0; r < 4; ++r) {
             const int row = r * 8 + rd_row;  // 0..31 within the half
             const int m = m0 + wm * 64 + h * 32 + row;
-            if (MODE == kGrouped && p.m_indices[m] != expert) continue;
+            if (!keep[h][r]) continue;
             const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
             __builtin_nontemporal_store(
                 d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
