@@ -23,6 +23,7 @@
 //   block:    every K step is one 128-block; its MFMA result is folded into the
 //             running sum as acc += part * (sa[m, kb] * sb[n / 128, kb]).
 #include <atomic>
+#include <type_traits>
 
 #include "cfp8_common.h"
 
@@ -431,6 +432,10 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 // plus a wave-uniform part).
 // ---------------------------------------------------------------------------
 #define CFP8_PHASE_END() __builtin_amdgcn_sched_barrier(0)
+// Wait until at most `vm` of this wave's loads are outstanding and its LDS reads are done, then the workgroup barrier.
+// Written out as instructions: in front of a barrier it knows of, the compiler waits for every load it has issued,
+// including the direct-to-LDS loads that are meant to stay in flight across the barrier.
+#define CFP8_WAIT_BARRIER(vm) asm volatile("s_waitcnt vmcnt(" #vm ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define CFP8_MMA2(wb, wh, xb, xh, g)                                                                   \
     {                                                                                                  \
         _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                \
@@ -545,8 +550,7 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
             CFP8_MMA2(0, 0, 1, 1, g);
             CFP8_PHASE_END();
         }
-        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
+        CFP8_WAIT_BARRIER(8);
         CFP8_PHASE_END();
         if (kt == scale_step) {
             // no activation tile goes into stage (last + 1) % 2 any more: it takes the tile's 256 activation scales and
@@ -626,6 +630,197 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
             const int m = m0 + wm * 128 + h * 64 + row;
             __builtin_nontemporal_store(
                 d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 128 + rd_chunk * 8));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same pipeline on 256 x 128 tiles (256 activation rows, 128 weight rows), for problems whose 256 x 256
+// tiles would fill the 256 CUs badly (a few hundred to a thousand tokens): four waves as 2 x 2, each a
+// 128 x 64 block = 32 accumulator tiles.  A step is two groups of 16 MFMAs:
+//
+//   S0 (w, x0): LDS reads x1              + loads of weight tile kt+2 into weight stage (kt+2) % 3
+//   -- wait for all but those four loads and for own LDS reads, barrier: tile kt+1 complete --
+//   S1 (w, x1): LDS reads next w, next x0 + loads of activation tile kt+2 into activation stage kt % 2
+//
+// LDS: two activation stages of 32 KiB, three weight stages of 16 KiB and the tile's scales (fetched in the
+// prologue).
+// Requires M % 256 == 0 and N % 128 == 0.
+// ---------------------------------------------------------------------------
+// (Budgeted for two waves per SIMD, i.e. 256 registers: with all 512 on offer the compiler spreads the 128
+// accumulators over both register files and copies them to and fro around the MFMAs.)
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_rowwise_256x128_kernel(const GemmArgs p) {
+    constexpr int BM = 256, BN = 128;
+    constexpr int XS = BM * 128, WS = BN * 128;
+    constexpr int WBASE = 2 * XS, SBASE = WBASE + 3 * WS;  // 112 KiB of stages, then 384 scales
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+
+    // direct-to-LDS loads as in gemm_rowwise_256_kernel: load i covers rows (wave + 4 i) * 8 .. + 7 of its operand's tile
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, b_step = 32u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
+    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+    auto dma_x = [&](int kt, int stage, int i) {  // i < 8
+        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, 0, 0);
+    };
+    auto dma_w = [&](int kt, int stage, int i) {  // i < 4
+        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
+        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, 0, 0);
+    };
+
+    f32x4 acc[4][8];  // [n tile][m tile]
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+    i32x8 W[4], X[2][4];  // the wave's four weight fragments; X[h]: the halves of its 128 rows
+    float* const scale_lds = reinterpret_cast<float*>(smem + SBASE);  // [0, 256): sa, [256, 384): sb
+
+    // prologue: tiles 0 and 1 and the scales (weight tile 2 follows in the first step)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(1 < last ? 1 : last, 1, i);
+    __builtin_amdgcn_global_load_lds((gbl_void*)(p.sa + m0 + wave * 64 + lane), (lds_void*)(scale_lds + wave * 64), 4, 0, 0);
+    if (wave < 2) __builtin_amdgcn_global_load_lds((gbl_void*)(p.sb + n0 + wave * 64 + lane), (lds_void*)(scale_lds + 256 + wave * 64), 4, 0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < 4; ++g) X[0][g] = frag(0, x_off, x_off2, g);
+#pragma unroll
+    for (int g = 0; g < 3; ++g) W[g] = frag(0, w_off, w_off2, g);
+    CFP8_PHASE_END();
+
+    // Both groups walk the weight fragments in order (MFMA pair g uses W[g >> 1]), so a fragment's registers can take
+    // the next step's fragment as soon as its last pair has been issued; the last one is read at the start of S0.
+#define CFP8_MMA2N(xh, g)                                                                              \
+    {                                                                                                  \
+        _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                \
+            const int i = (g) >> 1, j = ((g)&1) * 2 + e;                                               \
+            acc[i][(xh)*4 + j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(                     \
+                W[i], X[xh][j], acc[i][(xh)*4 + j], 0, 0, 0, 0, 0, 0);                                 \
+        }                                                                                              \
+    }
+    int ws_cur = 0;  // kt % 3
+    for (int kt = 0; kt < KT; ++kt) {
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ws_cur == 2 ? 0 : ws_cur + 1;
+        const int ws_prv = ws_cur == 0 ? 2 : ws_cur - 1;  // (kt + 2) % 3
+        const int kx = kt + 2 < last ? kt + 2 : last;     // past the end: the last tile again, never consumed
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g == 0) W[3] = frag(ws_cur * WS, w_off, w_off2, 3);
+            else if (g <= 4) X[1][g - 1] = frag(xs_cur, x_off, x_off2, 4 + g - 1);
+            if (g < 4) dma_w(kx, ws_prv, g);
+            CFP8_MMA2N(0, g);
+            CFP8_PHASE_END();
+        }
+        CFP8_WAIT_BARRIER(4);
+        CFP8_PHASE_END();
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            // (after the last step: stale data, unused)
+            if (g == 0) X[0][0] = frag(xs_nxt, x_off, x_off2, 0);
+            if (g == 1) X[0][1] = frag(xs_nxt, x_off, x_off2, 1);
+            if (g == 2) W[0] = frag(ws_nxt * WS, w_off, w_off2, 0);
+            if (g == 3) X[0][2] = frag(xs_nxt, x_off, x_off2, 2);
+            if (g == 4) W[1] = frag(ws_nxt * WS, w_off, w_off2, 1);
+            if (g == 5) X[0][3] = frag(xs_nxt, x_off, x_off2, 3);
+            if (g == 6) W[2] = frag(ws_nxt * WS, w_off, w_off2, 2);
+            dma_x(kx, kt & 1, g);
+            CFP8_MMA2N(1, g);
+            CFP8_PHASE_END();
+        }
+        ws_cur = ws_nxt;
+    }
+#undef CFP8_MMA2N
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the epilogue reuses the stages: nothing may still land there
+
+    float sam[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sam[j] = scale_lds[wm * 128 + j * 16 + lrow];
+    f32x4 sbn[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(scale_lds + 256 + wn * 64 + i * 16 + quarter * 4);
+    if (OUT_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + wn * 64 + i * 16 + quarter * 4;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int m = m0 + wm * 128 + j * 16 + lrow;
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
+                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: the wave's 128 x 64 block goes through LDS in two halves of 64 rows (row stride 144 B), so that global
+    // stores are 16 bytes per lane and 128 contiguous bytes per row, non-temporal
+    __syncthreads();  // all waves are done reading the operand stages
+    constexpr int EST = 144;
+    uint8_t* const ebuf = smem + wave * (64 * EST);
+    const int rd_row = lane >> 3, rd_chunk = lane & 7;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = h * 4 + jj;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
+                *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const int row = r * 8 + rd_row;  // 0..63 within the half
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            const int m = m0 + wm * 128 + h * 64 + row;
+            __builtin_nontemporal_store(
+                d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
         }
     }
 }
@@ -828,9 +1023,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             CFP8_PRODUCT(i, 1, 1);
         }
         CFP8_PHASE_END();
-        if (B_IT == 2) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
+        if (B_IT == 2) CFP8_WAIT_BARRIER(2);
+        else CFP8_WAIT_BARRIER(4);
         CFP8_PHASE_END();
         // tail.  The next group's activation scales are stored here, before this step's loads are requested: the
         // compiler makes an LDS store wait for every direct-to-LDS load in flight (it cannot tell that they go
@@ -986,6 +1180,23 @@ static int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 64;
     return dev >= 0 && dev < 64 ? dev : 64;
+}
+
+static int launch_rowwise_256x128(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 128;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    constexpr size_t lds = (size_t)(2 * 256 + 3 * 128) * 128 + 384 * sizeof(float);
+    static std::atomic<bool> raised[65][2];  // zero-initialised
+    const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
+    const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256x128_kernel<true>)
+                       : reinterpret_cast<const void*>(gemm_rowwise_256x128_kernel<false>);
+    const int slot = device_slot();
+    if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (v) hipLaunchKernelGGL(gemm_rowwise_256x128_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL(gemm_rowwise_256x128_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    return check_launch("gemm");
 }
 
 static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
@@ -1532,6 +1743,14 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kBlock && p.M > 512 && (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128) >= 384)
         return launch_cfg<256, 128, 4, 2, kBlock>(p, out_dtype, st);
     // measured on config 3 (N = 18944, K = 3584): 129..256 rows run 10 % faster as one 256 x 128 tile-row,
+    if (MODE == kRowwise && p.M % 256 == 0 && p.N % 128 == 0 && (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0) {
+        // 256 x 128 tiles of the direct-to-LDS pipeline (2.1 PFLOP/s in steady state against 2.4 for 256 x 256 tiles)
+        // wherever 256 x 256 tiles would leave at least half of the CUs idle (2048 x 3584 x 3584: 38 against 52 us,
+        // 1024 x 4608 x 3584: 37 against 50 us, 1024 x 3584 x 18944: 155 against 205 us), and for N that is not a
+        // multiple of 256
+        const int64_t t256 = (int64_t)(p.M / 256) * ((p.N + 255) / 256);
+        if (p.N % 256 != 0 || t256 <= 128) return launch_rowwise_256x128(p, out_dtype, st);
+    }
     // 257..512 rows 7 % faster on 256 x 256 tiles than on 128 x 128
     if (MODE == kRowwise && p.M > 128 && p.M <= 256) return launch_cfg<256, 128, 4, 2, kRowwise>(p, out_dtype, st);
     if (MODE == kRowwise && p.M > 256 && p.M <= 512) return launch_cfg<256, 256, 2, 4, kRowwise>(p, out_dtype, st);

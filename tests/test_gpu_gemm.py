@@ -44,6 +44,9 @@ def rowwise_operands(M, N, K, seed, dev):
                                    # full 256x256 tiles: the four-wave pipelined kernel (two activation and three weight
                                    # stages in LDS), K of 1, 2, 3, 4, 5 and 7 steps
                                    (768, 256, 128), (1024, 512, 384), (2048, 1280, 896), (768, 512, 512), (1024, 256, 640),
+                                   # 256 x 128 tiles of the same pipeline: 256 and 512 tokens, few tiles, N not a multiple of 256;
+                                   # K of 1, 2, 3, 4, 5 and 7 steps
+                                   (256, 128, 128), (512, 256, 256), (256, 2176, 384), (768, 384, 512), (1024, 1152, 640), (1024, 3584, 896),
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
                                    (2048, 8448, 256),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
