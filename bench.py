@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 hot path on one MI355X.
 
-Headline workload (BASELINE config 2): tensorwise FP8 quantisation of every linear weight of a
+Headline workload (benchmark config 2): tensorwise FP8 quantisation of every linear weight of a
 Qwen2.5-7B-shaped decoder (197 bf16 tensors, 7 070 285 824 elements, random init N(0, 0.02),
 already resident in HBM).  One step = one `cfp8_quant_tensorwise_multi` call over all tensors
 (grid amax -> scale -> e4m3 cast), i.e. one full weight-sync quantisation pass.

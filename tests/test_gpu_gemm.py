@@ -113,7 +113,7 @@ def test_scaled_mm_one_hot_and_pow2(dev):
 
 @pytest.mark.parametrize("M", [1, 64, 1024])
 def test_fp8_linear_cfg3_shapes(dev, M):
-    """BASELINE config 3 at reduced N (the full N runs in the property test below): per-token
+    """benchmark config 3 at reduced N (the full N runs in the property test below): per-token
     activation quantisation inside the call, bytes of the intermediate checked through the result."""
     N, K = 2048, 3584
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=1236 + M, dev=dev)

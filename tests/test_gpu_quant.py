@@ -39,7 +39,7 @@ def all_bf16_patterns():
 
 # ---------------------------------------------------------------------------- rowwise
 def test_rowwise_cfg1(dev):
-    """BASELINE config 1: [4864, 896], N(0, 0.02) with 0.1% x20 outliers, seed 1235."""
+    """benchmark config 1: [4864, 896], N(0, 0.02) with 0.1% x20 outliers, seed 1235."""
     w = O.make_weight((4864, 896), seed=1235, outlier_frac=1e-3, outlier_mul=20.0)
     q, s = ops.scaled_fp8_quant(w.to(dev), scale=None, use_per_token_if_dynamic=True)
     assert q.dtype == torch.float8_e4m3fn and tuple(s.shape) == (4864, 1)
@@ -280,7 +280,7 @@ def test_block128_transposed(dev, shape):
 
 
 def test_block128_cfg4_and_dequant_roundtrip(dev):
-    """BASELINE config 4 weight [7168, 18432] -> scales [56, 144]; a 512x512 corner against the
+    """benchmark config 4 weight [7168, 18432] -> scales [56, 144]; a 512x512 corner against the
     oracle, the whole tensor through weight_dequant (the in-tree inverse pins the layout)."""
     w = O.make_weight((7168, 18432), seed=1238)
     wd = w.to(dev)
