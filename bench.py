@@ -331,6 +331,26 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         del x, o, ws
     del qw3, sw3
 
+    # the four linear layers of one Qwen2.5-7B decoder block (vLLM's packed layout) at 2048 tokens, activation
+    # quantisation inside the call
+    ML = 2048
+    for nm, (n, k) in [("qkv_4608x3584", (4608, 3584)), ("o_3584x3584", (3584, 3584)),
+                       ("gate_up_37888x3584", (37888, 3584)), ("down_3584x18944", (3584, 18944))]:
+        name = f"linear_rowwise_{nm}_M{ML}"
+        if only and only not in name:
+            continue
+        w = torch.empty(n, k, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+        qw, sw = ops.quant_rowwise(w)
+        del w
+        x = torch.randn(ML, k, generator=gen, device=dev).to(torch.bfloat16)
+        o = torch.empty(ML, n, dtype=torch.bfloat16, device=dev)
+        wsb = lib.cfp8_linear_workspace_bytes_split(ML, n, k)
+        ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+        mfma(name, 2.0 * ML * n * k, n * k + 4 * n + ML * k * 2 + ML * n * 2,
+             lambda: check(lib.cfp8_linear_rowwise(x.data_ptr(), k, qw.data_ptr(), k, sw.data_ptr(), o.data_ptr(), n, 0,
+                                                   ML, n, k, ws.data_ptr(), wsb, stream)), iters=50)
+        del qw, sw, x, o, ws
+
     # MXFP4 quantisation of the gate_up expert weights of GPT-OSS-20B: [32 experts x 5760, 2880]
     RX, KX = 32 * 5760, 2880
     wx = torch.empty(RX, KX, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
