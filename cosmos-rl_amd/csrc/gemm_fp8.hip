@@ -395,7 +395,9 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 // Rowwise GEMM, large full tiles: 256 x 256 x 128 per workgroup, four wavefronts
 // (one per SIMD, 2 x 2), each owning a 128 x 128 block = 64 accumulators of
 // 16 x 16 (all 256 AGPRs).  Operand tiles go from global memory straight into
-// LDS (global_load_lds_dwordx4: no staging registers, no LDS store instructions).
+// LDS (buffer_load_dwordx4 ... lds: no staging registers, no LDS store instructions;
+// in the buffer form the wave-uniform part of an address is a scalar offset, so a
+// load costs two scalar additions and no vector arithmetic).
 // Such a load puts lane l's 16 bytes at byte l * 16 of its 1 KiB destination, so
 // the LDS layout is dictated by which bytes each lane asks for: a stage is
 // row-major, row r at r * 128, and lane l of a load of 8 rows fetches chunk
@@ -475,14 +477,17 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
     typedef __attribute__((address_space(1))) const void gbl_void;
     typedef __attribute__((address_space(3))) void lds_void;
-    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;  // an address built from an integer must be told that it is global memory
+    // buffer form of the load: descriptor in SGPRs (base = this wave's first row, no bounds), per-lane offset in one
+    // VGPR, the wave-uniform part of the address as the scalar offset - no vector arithmetic per load
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, 0xFFFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(b_wave), 0, 0xFFFFFFFF, 0x00020000);
     auto dma_x = [&](int kt, int stage, int i) {
-        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
     };
     auto dma_w = [&](int kt, int stage, int i) {
-        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
     };
 
     f32x4 acc[8][8];  // [n tile][m tile]
@@ -675,14 +680,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
     typedef __attribute__((address_space(1))) const void gbl_void;
     typedef __attribute__((address_space(3))) void lds_void;
-    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, 0xFFFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(b_wave), 0, 0xFFFFFFFF, 0x00020000);
     auto dma_x = [&](int kt, int stage, int i) {  // i < 8
-        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
     };
     auto dma_w = [&](int kt, int stage, int i) {  // i < 4
-        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
     };
 
     f32x4 acc[4][8];  // [n tile][m tile]
@@ -879,10 +885,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
     typedef __attribute__((address_space(1))) const void gbl_void;
     typedef __attribute__((address_space(3))) void lds_void;
-    typedef const __attribute__((address_space(1))) uint8_t* gptr_t;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, 0xFFFFFFFF, 0x00020000);
     auto dma_x = [&](int kt, int stage, int i) {
-        const uint64_t base = a_wave + (uint64_t)i * a_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + va_lane), (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
     };
     // The activation tiles do not depend on the group: in the grouped form they are requested before the group's
     // expert is known (one dependent scalar load less in front of the first tile).
@@ -904,9 +910,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
     uint64_t b_wave = reinterpret_cast<uint64_t>(bptr) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
     asm volatile("" : "+s"(b_wave));
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(b_wave), 0, 0xFFFFFFFF, 0x00020000);
     auto dma_w = [&](int kt, int stage, int i) {
-        const uint64_t base = b_wave + (uint64_t)i * b_step + ((uint64_t)kt << 7);
-        __builtin_amdgcn_global_load_lds((gbl_void*)((gptr_t)base + vb_lane), (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
     };
 
     // activation scales: 8 K steps of this tile's rows per fetch, 4 consecutive floats per thread
