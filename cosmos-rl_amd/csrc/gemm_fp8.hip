@@ -640,6 +640,231 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 }
 
 // ---------------------------------------------------------------------------
+// Persistent form of the 256 x 256 kernel: one workgroup per CU walks tiles b, b + gridDim.x, ...  The K steps of
+// consecutive tiles form one stream: the loads of a tile's last two steps already fetch the first steps of the next
+// tile, so a tile does not start with a round trip to memory, and the epilogue of a tile runs while those loads
+// are in flight.  The weight stage that the last step would have filled is left free instead and serves the
+// epilogue (the tile's scales and the buffer that turns the wave's block into row-contiguous stores, 16 rows at a
+// time); it is filled right after.  Requires K >= 384.
+// ---------------------------------------------------------------------------
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_rowwise_256p_kernel(const GemmArgs p) {
+    constexpr int BM = 256, BN = 256;
+    constexpr int XS = BM * 128, WS = BN * 128;
+    constexpr int WBASE = 2 * XS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int ntiles = p.tiles_m * p.tiles_n;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+    __builtin_assume(KT >= 3);
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, b_step = 32u * (uint32_t)p.ld_b;
+    asm volatile("" : "+s"(a_step), "+s"(b_step));
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    auto tile_rsrc = [&](int pid, int& m0, int& n0, __amdgpu_buffer_rsrc_t& ra, __amdgpu_buffer_rsrc_t& rb) {
+        int tm, tn;
+        tile_of_block(pid, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * BM;
+        n0 = tn * BN;
+        const uint64_t aw = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+        const uint64_t bw = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+        ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(aw), 0, 0xFFFFFFFF, 0x00020000);
+        rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(bw), 0, 0xFFFFFFFF, 0x00020000);
+    };
+    auto dma_x = [&](__amdgpu_buffer_rsrc_t r, int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    auto dma_w = [&](__amdgpu_buffer_rsrc_t r, int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+
+    int pid = blockIdx.x;
+    int m0, n0;
+    __amdgpu_buffer_rsrc_t ra, rb;
+    tile_rsrc(pid, m0, n0, ra, rb);
+    // stages of the stream's next step: activation stage xs (0 or XS), weight stage ws (0..2)
+    int xs = 0, ws = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(ra, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(rb, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(ra, 1, 1, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(rb, 1, 1, i);
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (;;) {
+        // the third weight step of this tile
+        {
+            const int w2 = ws == 0 ? 2 : ws - 1;  // (ws + 2) % 3
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dma_w(rb, 2, w2, i);
+        }
+        CFP8_WAIT_BARRIER(40);  // the activations of the second step have landed: they are older than the stores of the epilogue
+        const int pid_n = pid + (int)gridDim.x;
+        const bool has_next = pid_n < ntiles;
+        int m0n = m0, n0n = n0;
+        __amdgpu_buffer_rsrc_t ran = ra, rbn = rb;
+        if (has_next) tile_rsrc(pid_n, m0n, n0n, ran, rbn);
+
+        f32x4 acc[8][8];  // [n tile][m tile]
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        i32x8 W[2][4], X[2][4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            W[0][g] = frag(ws * WS, w_off, w_off2, g);
+            X[0][g] = frag(xs, x_off, x_off2, g);
+        }
+        CFP8_PHASE_END();
+
+        int ws_free = 0;
+        auto step = [&](int kt, auto wait_count) {
+            const int xs_nxt = xs ^ XS;
+            const int ws_nxt = ws == 2 ? 0 : ws + 1;
+            // loads of stream steps + 2 (activations) and + 3 (weights): past this tile's end they fetch the next tile
+            const bool xn = kt + 2 >= KT, wnx = kt + 3 >= KT;
+            const __amdgpu_buffer_rsrc_t rx = xn ? ran : ra, rw = wnx ? rbn : rb;
+            const int kx = xn ? kt + 2 - KT : kt + 2, kw = wnx ? kt + 3 - KT : kt + 3;
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g < 4) X[1][g] = frag(xs, x_off, x_off2, 4 + g);
+                CFP8_MMA2(0, 0, 0, 0, g);
+                CFP8_PHASE_END();
+            }
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g < 4) W[1][g] = frag(ws * WS, w_off, w_off2, 4 + g);
+                CFP8_MMA2(0, 0, 1, 1, g);
+                CFP8_PHASE_END();
+            }
+            if constexpr (decltype(wait_count)::value == 40) CFP8_WAIT_BARRIER(40);
+            else CFP8_WAIT_BARRIER(8);
+            CFP8_PHASE_END();
+            if (kt == last) {
+                // the weight stage of this step stays free for the epilogue; it takes the tile's scales now
+                uint8_t* dst = smem + WBASE + ws * WS + 24576 + wave * 256;
+                const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<float*>(p.sa) + m0 + wave * 64, 0, 0xFFFFFFFF, 0x00020000);
+                const __amdgpu_buffer_rsrc_t rsb = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<float*>(p.sb) + n0 + wave * 64, 0, 0xFFFFFFFF, 0x00020000);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsa, (lds_void*)dst, 4, (uint32_t)lane * 4u, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsb, (lds_void*)(dst + 1024), 4, (uint32_t)lane * 4u, 0, 0, 0);
+                ws_free = ws;
+            }
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g < 4) W[0][g] = frag(ws_nxt * WS, w_off, w_off2, g);
+                dma_x(rx, kx, xs == 0 ? 0 : 1, g);
+                CFP8_MMA2(1, 1, 0, 0, g);
+                CFP8_PHASE_END();
+            }
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g < 4) X[0][g] = frag(xs_nxt, x_off, x_off2, g);
+                if (kt != last) dma_w(rw, kw, ws, g);
+                CFP8_MMA2(1, 1, 1, 1, g);
+                CFP8_PHASE_END();
+            }
+            xs = xs_nxt;
+            ws = ws_nxt;
+        };
+        // the first step of a tile only needs loads that are older than the stores of the previous tile's epilogue
+        // (at most 32 of them, and the eight loads of the third weight step are younger still)
+        step(0, std::integral_constant<int, 40>{});
+        for (int kt = 1; kt < KT; ++kt) step(kt, std::integral_constant<int, 8>{});
+        // the scales have landed (the eight loads behind them belong to the next tile); every wave is done with the
+        // stage that serves the epilogue
+        CFP8_WAIT_BARRIER(8);
+
+        const float* const scale_lds = reinterpret_cast<const float*>(smem + WBASE + ws_free * WS + 24576);
+        float sam[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sam[j] = scale_lds[wm * 128 + j * 16 + lrow];
+        f32x4 sbn[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sbn[i] = *reinterpret_cast<const f32x4*>(scale_lds + 256 + wn * 128 + i * 16 + quarter * 4);
+        if (OUT_F32) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int n = n0 + wn * 128 + i * 16 + quarter * 4;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int m = m0 + wm * 128 + j * 16 + lrow;
+                    f32x4 v = acc[i][j];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
+                    __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+                }
+            }
+        } else {
+            constexpr int EST = 272;
+            uint8_t* const ebuf = smem + WBASE + ws_free * WS + wave * (16 * EST);
+            const int rd_row = lane >> 4, rd_chunk = lane & 15;
+            const uint32_t ebuf_wr =
+                (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(ebuf + lrow * EST + quarter * 8));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    f32x4 v = acc[i][j];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j] * sbn[i][e];
+                    // written as an instruction: in front of an LDS store it knows of, the compiler waits for the loads
+                    // of the next tile that are still on their way into other parts of LDS
+                    const uint64_t two = (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32);
+                    asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(ebuf_wr), "v"(two), "n"(i * 32) : "memory");
+                }
+                // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = r * 4 + rd_row;
+                    const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+                    const int m = m0 + wm * 128 + j * 16 + row;
+                    __builtin_nontemporal_store(
+                        d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 128 + rd_chunk * 8));
+                }
+            }
+        }
+        if (!has_next) break;
+        pid = pid_n;
+        m0 = m0n;
+        n0 = n0n;
+        ra = ran;
+        rb = rbn;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with its part of the epilogue buffer
+    }
+    // the loads past the last tile (they fetched its first steps once more) land before the workgroup gives up its LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// ---------------------------------------------------------------------------
 // The same pipeline on 256 x 128 tiles (256 activation rows, 128 weight rows), for problems whose 256 x 256
 // tiles would fill the 256 CUs badly (a few hundred to a thousand tokens): four waves as 2 x 2, each a
 // 128 x 64 block = 32 accumulator tiles.  A step is two groups of 16 MFMAs:
@@ -1189,6 +1414,40 @@ static int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached
     return dev >= 0 && dev < 64 ? dev : 64;
 }
 
+static int cu_count() {  // compute units of the current device
+    static std::atomic<int> cached[64];  // zero-initialised
+    const int slot = device_slot();
+    if (slot < 64) {
+        const int c = cached[slot].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0)
+        return 256;
+    if (slot < 64) cached[slot].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
+static int launch_rowwise_256p(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 256;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    const int cus = cu_count();
+    const int64_t blocks = tiles < cus ? tiles : cus;
+    constexpr size_t lds = (size_t)(2 + 3) * 256 * 128;
+    static std::atomic<bool> raised[65][2];  // zero-initialised
+    const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
+    const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_256p_kernel<true>)
+                       : reinterpret_cast<const void*>(gemm_rowwise_256p_kernel<false>);
+    const int slot = device_slot();
+    if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (v) hipLaunchKernelGGL(gemm_rowwise_256p_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL(gemm_rowwise_256p_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
+    return check_launch("gemm");
+}
+
 static int launch_rowwise_256x128(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 128;
@@ -1207,6 +1466,9 @@ static int launch_rowwise_256x128(GemmArgs& p, int out_dtype, hipStream_t st) {
 }
 
 static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
+    // more tiles than CUs: one workgroup per CU that walks its tiles and loads the next one under the current one
+    // (8192 x 18944 x 3584: 427-439 against 470 us)
+    if (p.K >= 384 && (int64_t)(p.M / 256) * (p.N / 256) > cu_count()) return launch_rowwise_256p(p, out_dtype, st);
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 256;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;

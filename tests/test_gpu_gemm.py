@@ -47,6 +47,10 @@ def rowwise_operands(M, N, K, seed, dev):
                                    # 256 x 128 tiles of the same pipeline: 256 and 512 tokens, few tiles, N not a multiple of 256;
                                    # K of 1, 2, 3, 4, 5 and 7 steps
                                    (256, 128, 128), (512, 256, 256), (256, 2176, 384), (768, 384, 512), (1024, 1152, 640), (1024, 3584, 896),
+                                   # more 256 x 256 tiles than CUs: every workgroup walks several tiles and loads the next
+                                   # one under the current one; 408 tiles and K of 3 steps, 405 tiles and 4 steps (a second
+                                   # round that not every workgroup takes part in), 512 tiles (+ 16 as a second launch) and 5 steps
+                                   (4352, 6144, 384), (2304, 11520, 512), (2048, 16896, 640),
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
                                    (2048, 8448, 256),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
