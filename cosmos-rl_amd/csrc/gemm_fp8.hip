@@ -1226,8 +1226,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     CFP8_PHASE_END();
     float sc2p = 0.f, sc3p = 0.f;  // scales of the products still waiting in P from the previous step
 
-#define CFP8_RESCALE(i, j, pj, sc)                                                                   \
-    _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(P[pj][i][e], sc, acc[i][j][e])
+// (the empty statement pins the four FMAs to this place: their results are not needed before the next step, and the
+// compiler would otherwise sink them past the branches of the tail, half of them to just behind the barrier)
+#define CFP8_RESCALE(i, j, pj, sc)                                                                            \
+    {                                                                                                         \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(P[pj][i][e], sc, acc[i][j][e]); \
+        asm volatile("" : "+v"(acc[i][j]));                                                                   \
+    }
 #define CFP8_PRODUCT(i, j, pj) \
     P[pj][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[j], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0)
     // Step kt computes from activation stage kt % 2 and weight stage kt % 3; behind its barrier activation tile kt + 2
@@ -1941,6 +1946,335 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// ---------------------------------------------------------------------------
+// Persistent form of the 256 x 128 block-scaled kernel (as gemm_rowwise_256p_kernel is of the rowwise one): one
+// workgroup per CU walks tiles b, b + gridDim.x, ...; the K steps of consecutive tiles form one stream of loads,
+// so a tile starts on operands, fragments and scales that arrived under the previous tile, and its epilogue runs
+// with the next tile's loads in flight.  Beyond the stages LDS holds the epilogue buffers of the eight waves
+// (16 rows each) and the weight scales of two tiles, which limits K to 1792 steps.  Requires K >= 384.
+// ---------------------------------------------------------------------------
+constexpr int kMaxPersistentBlockSteps = 1792;  // what fits into LDS
+constexpr int kPersistentBlockSteps = 32;       // what the dispatch sends here
+
+template <bool OUT_F32, bool SCALE_VEC>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8p_kernel(const GemmArgs p) {
+    constexpr int BM = 256, BN = 128;
+    constexpr int XS = BM * 128, WS = BN * 128;
+    constexpr int WBASE = 2 * XS;
+    constexpr int SBASE = WBASE + 3 * WS;            // turned activation scales: [2][8][BM]
+    constexpr int EST = 144;                         // row stride of an epilogue buffer (64 bf16 + 16 B)
+    constexpr int EBASE = SBASE + 2 * 8 * BM * 4;    // epilogue buffers: 16 rows per wave
+    constexpr int NBASE = EBASE + 8 * 16 * EST;      // weight scales of the current and the next tile
+    constexpr int A_IT = 4, B_IT = 2;
+    constexpr int NSTORES = OUT_F32 ? 16 : 8;        // global stores of one wave's epilogue
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int ntiles = p.tiles_m * p.tiles_n;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 3, wn = wave >> 2;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+    __builtin_assume(KT >= 3);
+    const int KTP = (KT + 63) & ~63;                 // floats of one weight-scale buffer
+    const int G = (KT + 7) >> 3;                     // groups of eight K steps per tile
+    uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;
+    asm volatile("" : "+s"(a_step), "+s"(b_step));
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(3))) void lds_void;
+    auto tile_rsrc = [&](int pid, int& m0, int& n0, __amdgpu_buffer_rsrc_t& ra, __amdgpu_buffer_rsrc_t& rb) {
+        int tm, tn;
+        tile_of_block(pid, p.tiles_m, p.tiles_n, tm, tn);
+        m0 = tm * BM;
+        n0 = tn * BN;
+        const uint64_t aw = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+        const uint64_t bw = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+        ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(aw), 0, 0xFFFFFFFF, 0x00020000);
+        rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(bw), 0, 0xFFFFFFFF, 0x00020000);
+    };
+    auto dma_x = [&](__amdgpu_buffer_rsrc_t r, int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    auto dma_w = [&](__amdgpu_buffer_rsrc_t r, int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    // the KT weight scales of the tile at column n0 into buffer par, 64 per wave-wide load (4 bytes per lane)
+    auto dma_sn = [&](int n0_, int par) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(p.sb) + (int64_t)(n0_ >> 7) * p.sb_stride_n, 0, 0xFFFFFFFF, 0x00020000);
+        for (int base = wave * 64; base < KT; base += 512) {
+            const int k = base + lane < KT ? base + lane : last;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + NBASE + (par * KTP + base) * 4), 4,
+                                                     (uint32_t)k * (uint32_t)p.sb_stride_k * 4u, 0, 0, 0);
+        }
+    };
+    float* const sg_buf = reinterpret_cast<float*>(smem + SBASE);
+    const float* const sn_lds = reinterpret_cast<const float*>(smem + NBASE);
+    f32x4 sg = {0.f, 0.f, 0.f, 0.f};
+    // (scalar base and one per-lane offset: no per-lane pointers to keep in registers across the loop)
+    auto sg_load = [&](int m0_, int g) {  // four of the K / 128 scales of this thread's activation row of the tile at m0_
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(p.sa) + (int64_t)m0_ * KT, 0, 0xFFFFFFFF, 0x00020000);
+        int te = t;  // (addresses rebuilt at every use: kept across the K loop they would cost registers it does not have)
+        asm volatile("" : "+v"(te));
+        const int k0 = 8 * g + 4 * (te & 1);
+        const int row = (te >> 1) * KT;
+        if (SCALE_VEC) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, (row + (k0 + 4 <= KT ? k0 : KT - 4)) * 4, 0, 0);
+            sg = f32x4{__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3])};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                sg[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, (row + ((k0 + e) < KT ? (k0 + e) : last)) * 4, 0, 0));
+        }
+    };
+    auto sg_store = [&](int par) {
+        int te = t;
+        asm volatile("" : "+v"(te));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sg_buf[((par & 1) * 8 + 4 * (te & 1) + e) * BM + (te >> 1)] = sg[e];
+    };
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+    i32x8 W[4], X[4];
+    float sm[4], s_n;
+    auto read_scales = [&](int gpar_, int snpar_, int k) {  // s_m of the wave's four x tiles and s_n of its weight block for step k
+        const float* const sgk = sg_buf + (((gpar_ + (k >> 3)) & 1) * 8 + (k & 7)) * BM + wm * 64 + lrow;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sm[j] = sgk[j * 16];
+        s_n = sn_lds[snpar_ * KTP + k];
+    };
+
+    int pid = blockIdx.x;
+    int m0, n0;
+    __amdgpu_buffer_rsrc_t ra, rb;
+    tile_rsrc(pid, m0, n0, ra, rb);
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(ra, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < A_IT; ++i) dma_x(ra, 1, 1, i);
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+#pragma unroll
+        for (int i = 0; i < B_IT; ++i) dma_w(rb, k, k, i);
+    dma_sn(n0, 0);
+    sg_load(m0, 0);
+    sg_store(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    X[0] = frag(0, x_off, x_off2, 0);
+    CFP8_PHASE_END();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        W[i] = frag(0, w_off, w_off2, i);
+        CFP8_PHASE_END();
+    }
+    X[1] = frag(0, x_off, x_off2, 1);
+    read_scales(0, 0, 0);
+    CFP8_PHASE_END();
+
+    f32x4 acc[4][4], P[2][4];  // [w tile][x tile]; raw products of two x tiles
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        P[0][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        P[1][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float sc2p = 0.f, sc3p = 0.f;  // scales of the products still waiting in P from the previous step
+    int xs = 0, ws = 0;            // stages of the stream's current step: activation stage (0 or XS bytes), weight stage 0..2
+    int gpar = 0, snpar = 0;       // scale buffers of the current tile: first group of activation scales, weight scales
+
+// (the empty statement pins the four FMAs to this place: their results are not needed before the next step, and the
+// compiler would otherwise sink them past the branches below to the end of the step, out of the MFMAs' shadow)
+#define CFP8_RESCALE(i, j, pj, sc)                                                                            \
+    {                                                                                                         \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = __builtin_fmaf(P[pj][i][e], sc, acc[i][j][e]); \
+        asm volatile("" : "+v"(acc[i][j]));                                                                   \
+    }
+#define CFP8_PRODUCT(i, j, pj) \
+    P[pj][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[j], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0)
+    for (;;) {
+        const int pid_n = pid + (int)gridDim.x;
+        const bool has_next = pid_n < ntiles;
+        int m0n = m0, n0n = n0;
+        __amdgpu_buffer_rsrc_t ran = ra, rbn = rb;
+        if (has_next) tile_rsrc(pid_n, m0n, n0n, ran, rbn);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+        auto step = [&](int kt, auto wait_count) {
+            const int xs_nxt = xs ^ XS;
+            const int ws_nxt = ws == 2 ? 0 : ws + 1;
+            // loads of stream steps + 2 (activations) and + 3 (weights): past this tile's end they fetch the next tile
+            const bool xn = kt + 2 >= KT, wnx = kt + 3 >= KT;
+            const __amdgpu_buffer_rsrc_t rx = xn ? ran : ra, rw = wnx ? rbn : rb;
+            const int kx = xn ? kt + 2 - KT : kt + 2, kw = wnx ? kt + 3 - KT : kt + 3;
+            // group 0
+            X[2] = frag(xs, x_off, x_off2, 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                CFP8_RESCALE(i, 2, 0, sc2p);
+                CFP8_PRODUCT(i, 0, 0);
+            }
+            CFP8_PHASE_END();
+            // group 1
+            X[3] = frag(xs, x_off, x_off2, 3);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                CFP8_RESCALE(i, 3, 1, sc3p);
+                CFP8_PRODUCT(i, 1, 1);
+            }
+            CFP8_PHASE_END();
+            // all but the two newest weight loads; in a tile's first step the stores of the previous tile's
+            // epilogue are younger than everything this barrier needs
+            if constexpr (decltype(wait_count)::value == 0) CFP8_WAIT_BARRIER(2);
+            else if constexpr (OUT_F32) CFP8_WAIT_BARRIER(18);
+            else CFP8_WAIT_BARRIER(10);
+            CFP8_PHASE_END();
+            // tail.  Scales fetched a step earlier go to LDS first (an LDS store the compiler knows of waits for every
+            // load in flight; here those are a whole step old): the next group of this tile, or the first group of
+            // the next tile, which is read from the end of the tile's last step on, one barrier later.
+            if ((kt & 7) == 6 && kt + 2 <= last) sg_store(gpar + (kt >> 3) + 1);
+            if (kt == last - 1) sg_store(gpar + G);
+            const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
+            sc2p = sm[2] * s_n;
+            sc3p = sm[3] * s_n;
+            X[0] = frag(xs_nxt, x_off, x_off2, 0);
+            if (kt == last - 1) dma_sn(n0n, snpar ^ 1);  // older than this step's two weight loads: landed at the next barrier
+#pragma unroll
+            for (int i = 0; i < A_IT; ++i) dma_x(rx, kx, xs == 0 ? 0 : 1, i);
+            if ((kt & 7) == 5 && kt + 3 <= last) sg_load(m0, (kt >> 3) + 1);
+            if (kt == last - 2) sg_load(m0n, 0);
+            CFP8_PHASE_END();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                CFP8_RESCALE(i, 0, 0, sc0);
+                CFP8_RESCALE(i, 1, 1, sc1);
+                CFP8_PRODUCT(i, 2, 0);
+                CFP8_PRODUCT(i, 3, 1);
+                CFP8_PHASE_END();
+                W[i] = frag(ws_nxt * WS, w_off, w_off2, i);
+                if (i < B_IT) dma_w(rw, kw, ws, i);
+                CFP8_PHASE_END();
+            }
+            X[1] = frag(xs_nxt, x_off, x_off2, 1);
+            if (kt == last) read_scales(gpar + G, snpar ^ 1, 0);
+            else read_scales(gpar, snpar, kt + 1);
+            CFP8_PHASE_END();
+            xs = xs_nxt;
+            ws = ws_nxt;
+        };
+        step(0, std::integral_constant<int, 1>{});
+        for (int kt = 1; kt < KT; ++kt) step(kt, std::integral_constant<int, 0>{});
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            CFP8_RESCALE(i, 2, 0, sc2p);
+            CFP8_RESCALE(i, 3, 1, sc3p);
+        }
+        sc2p = 0.f;  // the products left in P belong to this tile
+        sc3p = 0.f;
+
+        // epilogue: lane holds out[m][n .. n+3] for every (i, j).  Its per-lane addresses are derived here, from a
+        // lane number the compiler cannot see through: hoisted out of the tile loop they would occupy registers
+        // across the K loop, which has none to spare.
+        int le = lane;
+        asm volatile("" : "+v"(le));
+        const int lrow_e = le & 15, quarter_e = le >> 4;
+        if (OUT_F32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int m = m0 + wm * 64 + j * 16 + lrow_e;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + wn * 64 + i * 16 + quarter_e * 4;
+                    __builtin_nontemporal_store(acc[i][j], reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+                }
+            }
+        } else {
+            // bf16: 16 rows of the wave's 64 x 64 block at a time through the wave's own buffer, so that global stores
+            // are 16 bytes per lane and 128 contiguous bytes per row
+            uint8_t* const ebuf = smem + EBASE + wave * (16 * EST);
+            const int rd_row = le >> 3, rd_chunk = le & 7;
+            const uint32_t ebuf_wr = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(ebuf + lrow_e * EST + quarter_e * 8));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f32x4 v = acc[i][j];
+                    // written as an instruction: in front of an LDS store it knows of, the compiler waits for the
+                    // loads of the next tile that are on their way into other parts of LDS
+                    const uint64_t two = (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32);
+                    asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(ebuf_wr), "v"(two), "n"(i * 32) : "memory");
+                }
+                // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const int row = r * 8 + rd_row;
+                    const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+                    const int m = m0 + wm * 64 + j * 16 + row;
+                    __builtin_nontemporal_store(
+                        d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
+                }
+            }
+        }
+        if (!has_next) break;
+        pid = pid_n;
+        m0 = m0n;
+        n0 = n0n;
+        ra = ran;
+        rb = rbn;
+        gpar = (gpar + G) & 1;
+        snpar ^= 1;
+    }
+#undef CFP8_RESCALE
+#undef CFP8_PRODUCT
+    // the loads past the last tile (they fetched its first steps once more) land before the workgroup gives up its LDS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+static int launch_block_w8p(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 128;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    const int cus = cu_count();
+    const int64_t blocks = tiles < cus ? tiles : cus;
+    const int KT = p.K >> 7;
+    // stages, turned activation scales, epilogue buffers, weight scales of two tiles
+    const size_t lds = (size_t)(2 * 256 + 3 * 128) * 128 + 2 * 8 * 256 * sizeof(float) + 8 * 16 * 144 + (size_t)2 * ((KT + 63) & ~63) * sizeof(float);
+    const bool vec = KT % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    using Kern = void (*)(const GemmArgs);
+    const Kern table[2][2] = {{gemm_block_w8p_kernel<false, false>, gemm_block_w8p_kernel<true, false>},
+                              {gemm_block_w8p_kernel<false, true>, gemm_block_w8p_kernel<true, true>}};
+    const int f32 = out_dtype == CFP8_OUT_F32;
+    const Kern kern = table[vec][f32];
+    constexpr size_t lds_max = 160 * 1024;
+    static std::atomic<bool> done[65][2][2];  // zero-initialised
+    const int slot = device_slot();
+    if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec][f32])) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
+    return check_launch("gemm");
+}
+
 template <int BM, int BN, int MODE>
 static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / BM;
@@ -2008,7 +2342,14 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
     if (MODE == kBlock && p.M > 512 && p.M % 256 == 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
         (p.K >> 7) <= kMaxTileWeightScales)
+    {
+        // more tiles than CUs and a short K: one workgroup per CU that walks its tiles, so that a tile does not begin
+        // and end on an idle CU (8192 x 4096 x 512: 35 against 42 us, 4096 x 7168 x 2048: 79 against 83 us; from
+        // K = 7168 on both forms run level, the K loop is all there is)
+        if ((p.K >> 7) >= 3 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 256) * (p.N / 128) > cu_count())
+            return launch_block_w8p(p, out_dtype, st);
         return launch_block_w8<256, 128, kBlock>(p, out_dtype, st);
+    }
     if (MODE == kBlock && p.M > 512 && (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128) >= 384)
         return launch_cfg<256, 128, 4, 2, kBlock>(p, out_dtype, st);
     // measured on config 3 (N = 18944, K = 3584): 129..256 rows run 10 % faster as one 256 x 128 tile-row,
