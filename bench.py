@@ -287,6 +287,17 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
                                      o4.data_ptr(), N4, 0, M4, N4, K4, stream))
     mfma("gemm_block128_cfg4_4096x18432x7168_incl_act_quant", 2.0 * M4 * N4 * K4, N4 * K4 + M4 * K4 * 2 + M4 * N4 * 2, gemm4, iters=50)
     del x4, qx4, sx4, o4, q4, s4
+    # a short-K block-scaled GEMM (the shape of DeepSeek-V3's q_b projection at 4096 tokens): many tiles of few K steps each
+    Mq, Nq, Kq = 4096, 24576, 1536
+    qxq = torch.randint(0, 120, (Mq, Kq), generator=gen, device=dev, dtype=torch.uint8)
+    qwq = torch.randint(0, 120, (Nq, Kq), generator=gen, device=dev, dtype=torch.uint8)
+    sxq = torch.rand(Mq, Kq // 128, generator=gen, device=dev) + 0.5
+    swq = torch.rand(Nq // 128, Kq // 128, generator=gen, device=dev) + 0.5
+    oq = torch.empty(Mq, Nq, dtype=torch.bfloat16, device=dev)
+    mfma("gemm_block128_short_k_4096x24576x1536_gemm_only", 2.0 * Mq * Nq * Kq, Nq * Kq + Mq * Kq + Mq * Nq * 2,
+         lambda: check(lib.cfp8_gemm_block128(qxq.data_ptr(), Kq, sxq.data_ptr(), qwq.data_ptr(), Kq, swq.data_ptr(), Kq // 128, 1,
+                                              oq.data_ptr(), Nq, 0, Mq, Nq, Kq, stream)), iters=50)
+    del qxq, qwq, sxq, swq, oq
 
     # config 3: FP8 linear [M, 3584] x [18944, 3584]^T, per-token activation quant inside the call
     N3, K3 = 18944, 3584
