@@ -1947,36 +1947,47 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
 }
 
 // ---------------------------------------------------------------------------
-// Persistent form of the 256 x 128 block-scaled kernel (as gemm_rowwise_256p_kernel is of the rowwise one): one
-// workgroup per CU walks tiles b, b + gridDim.x, ...; the K steps of consecutive tiles form one stream of loads,
-// so a tile starts on operands, fragments and scales that arrived under the previous tile, and its epilogue runs
-// with the next tile's loads in flight.  Beyond the stages LDS holds the epilogue buffers of the eight waves
-// (16 rows each) and the weight scales of two tiles, which limits K to 1792 steps.  Requires K >= 384.
+// Persistent form of the eight-wave block-scaled (256 x 128) and grouped (128 x 256) kernel, as
+// gemm_rowwise_256p_kernel is of the rowwise one: one workgroup per CU walks tiles b, b + gridDim.x, ... (grouped:
+// those that are not padding); the K steps of consecutive tiles form one stream of loads, so a tile starts on
+// operands, fragments and scales that arrived under the previous tile, and its epilogue runs with the next tile's
+// loads in flight.  Beyond the stages LDS holds the epilogue buffers of the eight waves (16 rows each), the weight
+// scales of two tiles and, grouped, the expert of every row of two tiles.  Requires K >= 384; plain epilogues only.
 // ---------------------------------------------------------------------------
-constexpr int kMaxPersistentBlockSteps = 1792;  // what fits into LDS
-constexpr int kPersistentBlockSteps = 32;       // what the dispatch sends here
+constexpr int kPersistentBlockSteps = 32;  // K steps up to which the dispatch sends a problem here (LDS would hold 384)
 
-template <bool OUT_F32, bool SCALE_VEC>
+// One int of a table that no kernel writes, by a scalar load.  Behind the first store of a kernel the compiler turns
+// such a read into a vector load, and then waits for every load in flight, the direct-to-LDS ones included.
+__device__ __forceinline__ int scalar_table_load(const int32_t* table, int index) {
+    const int32_t* const ptr = table + index;  // uniform
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ptr) : "memory");
+    return v;
+}
+
+template <int BM, int BN, int MODE, bool OUT_F32>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8p_kernel(const GemmArgs p) {
-    constexpr int BM = 256, BN = 128;
+    static_assert((BM == 256 && BN == 128 && MODE == kBlock) || (BM == 128 && BN == 256 && MODE == kGrouped), "eight 64 x 64 wave tiles");
+    constexpr int WM = BM / 64;
     constexpr int XS = BM * 128, WS = BN * 128;
     constexpr int WBASE = 2 * XS;
     constexpr int SBASE = WBASE + 3 * WS;            // turned activation scales: [2][8][BM]
     constexpr int EST = 144;                         // row stride of an epilogue buffer (64 bf16 + 16 B)
     constexpr int EBASE = SBASE + 2 * 8 * BM * 4;    // epilogue buffers: 16 rows per wave
-    constexpr int NBASE = EBASE + 8 * 16 * EST;      // weight scales of the current and the next tile
-    constexpr int A_IT = 4, B_IT = 2;
-    constexpr int NSTORES = OUT_F32 ? 16 : 8;        // global stores of one wave's epilogue
+    constexpr int IBASE = EBASE + 8 * 16 * EST;      // grouped: the expert of each row of the current and the next tile, [2][128]
+    constexpr int NBASE = IBASE + 2 * 128 * 4;       // weight scales of the current and the next tile
+    constexpr int A_IT = BM / 64, B_IT = BN / 64;
+    constexpr int NB = BN / 128;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int ntiles = p.tiles_m * p.tiles_n;
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = wave & 3, wn = wave >> 2;
+    const int wm = wave % WM, wn = wave / WM;
     const int lrow = lane & 15, quarter = lane >> 4;
     const int KT = p.K >> 7;
     const int last = KT - 1;
     __builtin_assume(KT >= 3);
-    const int KTP = (KT + 63) & ~63;                 // floats of one weight-scale buffer
+    const int KTP = (KT * NB + 63) & ~63;            // floats of one weight-scale buffer
     const int G = (KT + 7) >> 3;                     // groups of eight K steps per tile
     uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;
     asm volatile("" : "+s"(a_step), "+s"(b_step));
@@ -1984,13 +1995,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
     typedef __attribute__((address_space(3))) void lds_void;
-    auto tile_rsrc = [&](int pid, int& m0, int& n0, __amdgpu_buffer_rsrc_t& ra, __amdgpu_buffer_rsrc_t& rb) {
+    auto tile_expert = [&](int pid) {  // grouped: the expert of the tile's rows, negative for a tile of padding
+        int tm, tn;
+        tile_of_block(pid, p.tiles_m, p.tiles_n, tm, tn);
+        return scalar_table_load(p.m_indices, tm * BM);  // groups start on multiples of 128 = BM rows
+    };
+    auto next_tile = [&](int pid) {  // the next tile of this workgroup that is not padding
+        int q = pid + (int)gridDim.x;
+        if (MODE == kGrouped)
+            while (q < ntiles && tile_expert(q) < 0) q += (int)gridDim.x;
+        return q;
+    };
+    auto tile_rsrc = [&](int pid, int& m0, int& n0, int& expert, __amdgpu_buffer_rsrc_t& ra, __amdgpu_buffer_rsrc_t& rb) {
         int tm, tn;
         tile_of_block(pid, p.tiles_m, p.tiles_n, tm, tn);
         m0 = tm * BM;
         n0 = tn * BN;
+        expert = MODE == kGrouped ? scalar_table_load(p.m_indices, m0) : 0;
         const uint64_t aw = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
-        const uint64_t bw = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+        const uint64_t bw = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)expert * (uint64_t)p.N + (uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
         ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(aw), 0, 0xFFFFFFFF, 0x00020000);
         rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(bw), 0, 0xFFFFFFFF, 0x00020000);
     };
@@ -2002,14 +2025,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, vb_lane,
                                                  (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
     };
-    // the KT weight scales of the tile at column n0 into buffer par, 64 per wave-wide load (4 bytes per lane)
-    auto dma_sn = [&](int n0_, int par) {
+    // the KT x NB weight scales of the tile at column n0 into buffer par, 64 per wave-wide load (4 bytes per lane);
+    // grouped: also the expert of each of the tile's rows (the epilogue writes only the rows of the tile's expert)
+    auto dma_sn = [&](int m0_, int n0_, int expert_, int par) {
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(p.sb) + (int64_t)(n0_ >> 7) * p.sb_stride_n, 0, 0xFFFFFFFF, 0x00020000);
-        for (int base = wave * 64; base < KT; base += 512) {
-            const int k = base + lane < KT ? base + lane : last;
+            const_cast<float*>(p.sb) + (int64_t)expert_ * p.sb_stride_e + (int64_t)(n0_ >> 7) * p.sb_stride_n, 0, 0xFFFFFFFF, 0x00020000);
+        for (int base = wave * 64; base < KT * NB; base += 512) {
+            const int idx = base + lane < KT * NB ? base + lane : KT * NB - 1;
+            const int kk = NB == 2 ? idx >> 1 : idx, nb = NB == 2 ? idx & 1 : 0;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + NBASE + (par * KTP + base) * 4), 4,
-                                                     (uint32_t)k * (uint32_t)p.sb_stride_k * 4u, 0, 0, 0);
+                                                     ((uint32_t)nb * (uint32_t)p.sb_stride_n + (uint32_t)kk * (uint32_t)p.sb_stride_k) * 4u, 0, 0, 0);
+        }
+        if (MODE == kGrouped && wave < 2) {
+            const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<int32_t*>(p.m_indices) + m0_ + wave * 64, 0, 0xFFFFFFFF, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ri, (lds_void*)(smem + IBASE + (par * 128 + wave * 64) * 4), 4, (uint32_t)lane * 4u, 0, 0, 0);
         }
     };
     float* const sg_buf = reinterpret_cast<float*>(smem + SBASE);
@@ -2017,24 +2047,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     f32x4 sg = {0.f, 0.f, 0.f, 0.f};
     // (scalar base and one per-lane offset: no per-lane pointers to keep in registers across the loop)
     auto sg_load = [&](int m0_, int g) {  // four of the K / 128 scales of this thread's activation row of the tile at m0_
+        // one 16-byte buffer load whatever K is: buffer loads need dword alignment only, what lies past a row's end is
+        // the next row's (never used), and past the end of the array the descriptor's size makes the load return zeros
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float*>(p.sa) + (int64_t)m0_ * KT, 0, 0xFFFFFFFF, 0x00020000);
+            const_cast<float*>(p.sa) + (int64_t)m0_ * KT, 0, (int)(((int64_t)(p.M - m0_) * KT < (1 << 29) ? (int64_t)(p.M - m0_) * KT : (1 << 29) - 1) * 4), 0x00020000);
         int te = t;  // (addresses rebuilt at every use: kept across the K loop they would cost registers it does not have)
         asm volatile("" : "+v"(te));
-        const int k0 = 8 * g + 4 * (te & 1);
-        const int row = (te >> 1) * KT;
-        if (SCALE_VEC) {
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, (row + (k0 + 4 <= KT ? k0 : KT - 4)) * 4, 0, 0);
-            sg = f32x4{__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3])};
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                sg[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, (row + ((k0 + e) < KT ? (k0 + e) : last)) * 4, 0, 0));
-        }
+        if (BM < 256 && te >= 2 * BM) return;
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, ((te >> 1) * KT + 8 * g + 4 * (te & 1)) * 4, 0, 0);
+        sg = f32x4{__uint_as_float(v[0]), __uint_as_float(v[1]), __uint_as_float(v[2]), __uint_as_float(v[3])};
     };
     auto sg_store = [&](int par) {
         int te = t;
         asm volatile("" : "+v"(te));
+        if (BM < 256 && te >= 2 * BM) return;
 #pragma unroll
         for (int e = 0; e < 4; ++e) sg_buf[((par & 1) * 8 + 4 * (te & 1) + e) * BM + (te >> 1)] = sg[e];
     };
@@ -2059,13 +2085,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         const float* const sgk = sg_buf + (((gpar_ + (k >> 3)) & 1) * 8 + (k & 7)) * BM + wm * 64 + lrow;
 #pragma unroll
         for (int j = 0; j < 4; ++j) sm[j] = sgk[j * 16];
-        s_n = sn_lds[snpar_ * KTP + k];
+        s_n = sn_lds[snpar_ * KTP + k * NB + (NB == 2 ? wn >> 1 : 0)];
     };
 
     int pid = blockIdx.x;
-    int m0, n0;
+    if (MODE == kGrouped) {
+        while (pid < ntiles && tile_expert(pid) < 0) pid += (int)gridDim.x;
+        if (pid >= ntiles) return;  // nothing but padding for this workgroup (uniform)
+    }
+    int m0, n0, expert;
     __amdgpu_buffer_rsrc_t ra, rb;
-    tile_rsrc(pid, m0, n0, ra, rb);
+    tile_rsrc(pid, m0, n0, expert, ra, rb);
 #pragma unroll
     for (int i = 0; i < A_IT; ++i) dma_x(ra, 0, 0, i);
 #pragma unroll
@@ -2074,7 +2104,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     for (int k = 0; k < 3; ++k)
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) dma_w(rb, k, k, i);
-    dma_sn(n0, 0);
+    dma_sn(m0, n0, expert, 0);
     sg_load(m0, 0);
     sg_store(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -2110,11 +2140,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
 #define CFP8_PRODUCT(i, j, pj) \
     P[pj][i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[j], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0)
     for (;;) {
-        const int pid_n = pid + (int)gridDim.x;
+        const int pid_n = next_tile(pid);
         const bool has_next = pid_n < ntiles;
-        int m0n = m0, n0n = n0;
+        int m0n = m0, n0n = n0, expert_n = expert;
         __amdgpu_buffer_rsrc_t ran = ra, rbn = rb;
-        if (has_next) tile_rsrc(pid_n, m0n, n0n, ran, rbn);
+        if (has_next) tile_rsrc(pid_n, m0n, n0n, expert_n, ran, rbn);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -2143,11 +2173,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
                 CFP8_PRODUCT(i, 1, 1);
             }
             CFP8_PHASE_END();
-            // all but the two newest weight loads; in a tile's first step the stores of the previous tile's
+            // all but the B_IT newest weight loads; in a tile's first step the 8 or 16 stores of the previous tile's
             // epilogue are younger than everything this barrier needs
-            if constexpr (decltype(wait_count)::value == 0) CFP8_WAIT_BARRIER(2);
-            else if constexpr (OUT_F32) CFP8_WAIT_BARRIER(18);
-            else CFP8_WAIT_BARRIER(10);
+            if constexpr (decltype(wait_count)::value == 0) {
+                if constexpr (B_IT == 2) CFP8_WAIT_BARRIER(2);
+                else CFP8_WAIT_BARRIER(4);
+            } else if constexpr (B_IT == 2) {
+                if constexpr (OUT_F32) CFP8_WAIT_BARRIER(18);
+                else CFP8_WAIT_BARRIER(10);
+            } else {
+                if constexpr (OUT_F32) CFP8_WAIT_BARRIER(20);
+                else CFP8_WAIT_BARRIER(12);
+            }
             CFP8_PHASE_END();
             // tail.  Scales fetched a step earlier go to LDS first (an LDS store the compiler knows of waits for every
             // load in flight; here those are a whole step old): the next group of this tile, or the first group of
@@ -2158,7 +2195,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             sc2p = sm[2] * s_n;
             sc3p = sm[3] * s_n;
             X[0] = frag(xs_nxt, x_off, x_off2, 0);
-            if (kt == last - 1) dma_sn(n0n, snpar ^ 1);  // older than this step's two weight loads: landed at the next barrier
+            if (kt == last - 1) dma_sn(m0n, n0n, expert_n, snpar ^ 1);  // older than this step's weight loads: landed at the next barrier
 #pragma unroll
             for (int i = 0; i < A_IT; ++i) dma_x(rx, kx, xs == 0 ? 0 : 1, i);
             if ((kt & 7) == 5 && kt + 3 <= last) sg_load(m0, (kt >> 3) + 1);
@@ -2198,14 +2235,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         int le = lane;
         asm volatile("" : "+v"(le));
         const int lrow_e = le & 15, quarter_e = le >> 4;
+        // grouped: rows that do not belong to the tile's expert stay unwritten.  Their stores are issued all the same,
+        // with an offset past the end of the buffer descriptor (the hardware drops them): the barrier of the next tile's
+        // first step counts on a fixed number of stores in front of the loads it lets pass.
+        const int32_t* const row_expert = reinterpret_cast<const int32_t*>(smem + IBASE) + snpar * 128 + wm * 64;
+        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+            static_cast<uint8_t*>(p.out) + (int64_t)m0 * p.ld_out * (OUT_F32 ? 4 : 2), 0, 0x80000000u, 0x00020000);
         if (OUT_F32) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int m = m0 + wm * 64 + j * 16 + lrow_e;
+                const int r = wm * 64 + j * 16 + lrow_e;
+                const bool keep = MODE != kGrouped || row_expert[j * 16 + lrow_e] == expert;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int n = n0 + wn * 64 + i * 16 + quarter_e * 4;
-                    __builtin_nontemporal_store(acc[i][j], reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+                    if (MODE == kGrouped) {
+                        const f32x4 v = acc[i][j];
+                        __builtin_amdgcn_raw_buffer_store_b128(u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}, ro,
+                                                               keep ? (uint32_t)((r * (int)p.ld_out + n) * 4) : 0xFFFFFFF0u, 0, 0);
+                    } else {
+                        __builtin_nontemporal_store(acc[i][j], reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)(m0 + r) * p.ld_out + n));
+                    }
                 }
             }
         } else {
@@ -2229,9 +2279,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
                 for (int r = 0; r < 2; ++r) {
                     const int row = r * 8 + rd_row;
                     const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
-                    const int m = m0 + wm * 64 + j * 16 + row;
-                    __builtin_nontemporal_store(
-                        d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
+                    const int rr = wm * 64 + j * 16 + row;
+                    if (MODE == kGrouped) {
+                        const bool keep = row_expert[j * 16 + row] == expert;
+                        __builtin_amdgcn_raw_buffer_store_b128(u32x4{(u32)d[0], (u32)d[1], (u32)d[2], (u32)d[3]}, ro,
+                                                               keep ? (uint32_t)((rr * (int)p.ld_out + n0 + wn * 64 + rd_chunk * 8) * 2) : 0xFFFFFFF0u, 0, 0);
+                    } else {
+                        __builtin_nontemporal_store(
+                            d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)(m0 + rr) * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
+                    }
                 }
             }
         }
@@ -2241,6 +2297,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         n0 = n0n;
         ra = ran;
         rb = rbn;
+        expert = expert_n;
         gpar = (gpar + G) & 1;
         snpar ^= 1;
     }
@@ -2250,27 +2307,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+template <int BM, int BN, int MODE>
 static int launch_block_w8p(GemmArgs& p, int out_dtype, hipStream_t st) {
-    p.tiles_m = p.M / 256;
-    p.tiles_n = p.N / 128;
+    p.tiles_m = p.M / BM;
+    p.tiles_n = p.N / BN;
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
     const int cus = cu_count();
     const int64_t blocks = tiles < cus ? tiles : cus;
     const int KT = p.K >> 7;
     // stages, turned activation scales, epilogue buffers, weight scales of two tiles
-    const size_t lds = (size_t)(2 * 256 + 3 * 128) * 128 + 2 * 8 * 256 * sizeof(float) + 8 * 16 * 144 + (size_t)2 * ((KT + 63) & ~63) * sizeof(float);
-    const bool vec = KT % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + 8 * 16 * 144 + 2 * 128 * sizeof(int32_t) +
+                       (size_t)2 * ((KT * (BN / 128) + 63) & ~63) * sizeof(float);
     using Kern = void (*)(const GemmArgs);
-    const Kern table[2][2] = {{gemm_block_w8p_kernel<false, false>, gemm_block_w8p_kernel<true, false>},
-                              {gemm_block_w8p_kernel<false, true>, gemm_block_w8p_kernel<true, true>}};
     const int f32 = out_dtype == CFP8_OUT_F32;
-    const Kern kern = table[vec][f32];
+    const Kern kern = f32 ? static_cast<Kern>(gemm_block_w8p_kernel<BM, BN, MODE, true>) : static_cast<Kern>(gemm_block_w8p_kernel<BM, BN, MODE, false>);
     constexpr size_t lds_max = 160 * 1024;
-    static std::atomic<bool> done[65][2][2];  // zero-initialised
+    static std::atomic<bool> done[65][2];  // zero-initialised
     const int slot = device_slot();
-    if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
-    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec][f32])) return rc;
+    if (slot == 64) done[64][f32].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][f32])) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
     return check_launch("gemm");
 }
@@ -2325,8 +2381,15 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) {
         // groups are 128-row aligned, so a tile is 128 rows; 256 columns per workgroup (8 waves) read a
         // quarter fewer operand bytes per flop than 128
-        if (p.M % 128 == 0 && p.N % 256 == 0 && (int64_t)(p.M / 128) * (p.N / 256) >= 384 && (p.K >> 7) * 2 <= kMaxTileWeightScales)
+        if (p.M % 128 == 0 && p.N % 256 == 0 && (int64_t)(p.M / 128) * (p.N / 256) >= 384 && (p.K >> 7) * 2 <= kMaxTileWeightScales) {
+            // 12 to 32 K steps: one workgroup per CU that walks its tiles (73600 rows, K = 2048: N = 1536 279 against 293 us,
+            // N = 7168 1258 against 1360 us; K = 768: 177 against 172 us, that stays on the kernel below).  The epilogue
+            // addresses a tile's rows with 32-bit offsets.
+            if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 128) * (p.N / 256) > cu_count() &&
+                p.ld_out < (1 << 21))
+                return launch_block_w8p<128, 256, kGrouped>(p, out_dtype, st);
             return launch_block_w8<128, 256, kGrouped>(p, out_dtype, st);
+        }
         if (p.N % 256 == 0 && (int64_t)((p.M + 127) / 128) * (p.N / 256) >= 384)
             return launch_cfg<128, 256, 2, 4, kGrouped>(p, out_dtype, st);
         return launch_cfg<128, 128, 2, 2, kGrouped>(p, out_dtype, st);
@@ -2347,7 +2410,7 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
         // and end on an idle CU (8192 x 4096 x 512: 35 against 42 us, 4096 x 7168 x 2048: 79 against 83 us; from
         // K = 7168 on both forms run level, the K loop is all there is)
         if ((p.K >> 7) >= 3 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 256) * (p.N / 128) > cu_count())
-            return launch_block_w8p(p, out_dtype, st);
+            return launch_block_w8p<256, 128, kBlock>(p, out_dtype, st);
         return launch_block_w8<256, 128, kBlock>(p, out_dtype, st);
     }
     if (MODE == kBlock && p.M > 512 && (int64_t)((p.M + 255) / 256) * ((p.N + 127) / 128) >= 384)

@@ -379,12 +379,14 @@ def test_grouped_cfg5_full_size_properties(dev):
 
 
 @pytest.mark.parametrize("T,E,K,N,topk", [(300, 7, 512, 384, 2), (2600, 7, 384, 2048, 2), (3300, 7, 1152, 2048, 2), (3300, 7, 1024, 1792, 2),
-                                          (3300, 7, 128, 2048, 2)])
+                                          (3300, 7, 128, 2048, 2), (3300, 7, 1536, 2048, 2), (3300, 7, 2176, 2048, 2)])
 def test_grouped_gemm(dev, T, E, K, N, topk):
     """Ragged groups: top-2 routing over 6 experts plus an empty expert, groups padded to 128 rows;
     padding rows (index -1) must be left untouched.  The shapes with 3300 tokens have >= 384 tiles of
     128 x 256 (the eight-wave kernel): K of 9 steps (more than one group of 8 activation-scale steps, scalar
-    scale loads), 8 steps (16-byte scale loads) with N = 7 * 256, and a single step."""
+    scale loads), 8 steps (16-byte scale loads) with N = 7 * 256, and a single step; K of 12 and 17 steps take the
+    form of that kernel in which a workgroup walks several tiles (it has to step over the empty expert's padding tile
+    and leave padding rows unwritten through masked stores)."""
     g = torch.Generator().manual_seed(77)
     logits = torch.rand(T, E, generator=g)
     logits[:, 3] = -1.0  # expert 3 gets no token
