@@ -1965,9 +1965,10 @@ __device__ __forceinline__ int scalar_table_load(const int32_t* table, int index
     return v;
 }
 
-template <int BM, int BN, int MODE, bool OUT_F32>
+template <int BM, int BN, int MODE, bool OUT_F32, bool SWIGLU = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8p_kernel(const GemmArgs p) {
     static_assert((BM == 256 && BN == 128 && MODE == kBlock) || (BM == 128 && BN == 256 && MODE == kGrouped), "eight 64 x 64 wave tiles");
+    static_assert(!SWIGLU || (MODE == kGrouped && !OUT_F32), "the SwiGLU epilogue belongs to the grouped 128 x 256 tile");
     constexpr int WM = BM / 64;
     constexpr int XS = BM * 128, WS = BN * 128;
     constexpr int WBASE = 2 * XS;
@@ -2238,6 +2239,60 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         // grouped: rows that do not belong to the tile's expert stay unwritten.  Their stores are issued all the same,
         // with an offset past the end of the buffer descriptor (the hardware drops them): the barrier of the next tile's
         // first step counts on a fixed number of stores in front of the loads it lets pass.
+        if constexpr (SWIGLU) {
+            // The tile's 256 weight rows are 128 gate rows followed by the 128 up rows of the same hidden columns, so the
+            // tile holds everything one 1x128 group of h = silu(gate) * up needs.  32 token rows at a time (the epilogue
+            // buffers hold no more): the four waves that own them put both halves into LDS rounded to bf16, as the GEMM
+            // would have written them; then sixteen threads per row form h, its group maximum and scale, and the fp8
+            // bytes - the arithmetic of the separate SwiGLU quantiser, bit for bit.  Two stores per wave and pass.
+            constexpr int GST = 272;  // LDS row stride in bytes (128 bf16 + 16)
+            uint8_t* const sw = smem + EBASE;  // [gate, up][32 rows][GST]
+            const int32_t* const tile_expert_of_row = reinterpret_cast<const int32_t*>(smem + IBASE) + snpar * 128;
+            const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+                static_cast<uint8_t*>(p.out) + (int64_t)m0 * p.ld_out, 0, 0x80000000u, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(
+                p.h_scales + (int64_t)m0 * p.ld_hs, 0, 0x80000000u, 0x00020000);
+            const int tn = n0 >> 8;
+            int te = t;
+            asm volatile("" : "+v"(te));
+            const int r32 = te >> 4, c16 = te & 15;
+            const uint32_t sw_wr = (uint32_t) reinterpret_cast<uintptr_t>(
+                (lds_void*)(sw + (wn >> 1) * (32 * GST) + lrow_e * GST + ((wn & 1) * 64 + quarter_e * 4) * 2));
+            const uint32_t sw_rd = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(sw + r32 * GST + c16 * 16));
+#pragma unroll
+            for (int qp = 0; qp < 4; ++qp) {
+                if (qp) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // the previous pass has been read
+                if (wm == (qp >> 1)) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const f32x4 v = acc[i][(qp & 1) * 2 + jj];
+                            const uint64_t two = (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32);
+                            asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(sw_wr), "v"(two), "n"(jj * 16 * GST + i * 32) : "memory");
+                        }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                // (read by instructions of its own: in front of an LDS read it knows of, the compiler waits for the
+                // next tile's loads that are on their way into other parts of LDS)
+                u32x4 gv, uv;
+                asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&v"(gv), "=&v"(uv)
+                             : "v"(sw_rd), "n"(32 * GST)
+                             : "memory");
+                const uint4 g = make_uint4(gv[0], gv[1], gv[2], gv[3]), u = make_uint4(uv[0], uv[1], uv[2], uv[3]);
+                const uint4 h = make_uint4(swiglu_pair(g.x, u.x), swiglu_pair(g.y, u.y), swiglu_pair(g.z, u.z), swiglu_pair(g.w, u.w));
+                const u32 mx = row16_max(pk_fold(absmax8(0u, h)));  // the sixteen threads of a row are one DPP row
+                const float scale = scale_from_amax(amax_from_bits(mx));
+                const Divider d(scale);
+                const int r = qp * 32 + r32;  // row of the tile
+                const bool keep = tile_expert_of_row[r] == expert;
+                const uint2 b = cast8(h, d);
+                __builtin_amdgcn_raw_buffer_store_b64(u32x2{b.x, b.y}, rq, keep ? (uint32_t)(r * (int)p.ld_out + tn * 128 + c16 * 8) : 0xFFFFFFF0u, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(scale), rh, keep && c16 == 0 ? (uint32_t)((r * (int)p.ld_hs + tn) * 4) : 0xFFFFFFF0u, 0, 0);
+            }
+            // (the first barrier of the next tile's K loop separates its first pass from this tile's last reads)
+        } else {
         const int32_t* const row_expert = reinterpret_cast<const int32_t*>(smem + IBASE) + snpar * 128 + wm * 64;
         const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
             static_cast<uint8_t*>(p.out) + (int64_t)m0 * p.ld_out * (OUT_F32 ? 4 : 2), 0, 0x80000000u, 0x00020000);
@@ -2290,6 +2345,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
                     }
                 }
             }
+        }
         }
         if (!has_next) break;
         pid = pid_n;
@@ -2362,6 +2418,21 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     p.tiles_n = p.N / BN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && blocks > cu_count() && p.ld_out < (1 << 21) && p.ld_hs < (1 << 20)) {
+        // 12 to 32 K steps: one workgroup per CU that walks its tiles
+        const int cus = cu_count();
+        const int KT = p.K >> 7;
+        const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + 8 * 16 * 144 + 2 * 128 * sizeof(int32_t) +
+                           (size_t)2 * ((KT * 2 + 63) & ~63) * sizeof(float);
+        using Kern = void (*)(const GemmArgs);
+        const Kern kern = gemm_block_w8p_kernel<BM, BN, kGrouped, false, true>;
+        static std::atomic<bool> done[65];  // zero-initialised
+        const int slot = device_slot();
+        if (slot == 64) done[64].store(false, std::memory_order_relaxed);
+        if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), 160 * 1024, done[slot])) return rc;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(blocks < cus ? blocks : cus)), dim3(512), lds, st, p);
+        return check_launch("gemm");
+    }
     const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + (size_t)(p.K >> 7) * (BN / 128) * sizeof(float);
     const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
     using Kern = void (*)(const GemmArgs);

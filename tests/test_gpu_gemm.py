@@ -279,7 +279,9 @@ def test_gemm_block128_cfg4_properties(dev):
 
 
 # ---------------------------------------------------------------------------- grouped
-@pytest.mark.parametrize("T,E,K,I,topk", [(300, 7, 512, 256, 2), (3300, 7, 1152, 1024, 2), (700, 5, 128, 128, 3), (2000, 9, 1024, 384, 2)])
+@pytest.mark.parametrize("T,E,K,I,topk", [(300, 7, 512, 256, 2), (3300, 7, 1152, 1024, 2), (700, 5, 128, 128, 3), (2000, 9, 1024, 384, 2),
+                                          # K of 12 and 17 steps, more tiles than CUs: the form in which a workgroup walks several tiles
+                                          (3300, 7, 1536, 1024, 2), (3300, 7, 2176, 1024, 2)])
 def test_grouped_swiglu_epilogue_bit_exact(dev, T, E, K, I, topk):
     """Grouped gate_up GEMM with SwiGLU + 1x128 requantisation as its epilogue (interleaved weights) against the
     grouped GEMM on the concatenated weights followed by the SwiGLU quantiser: same bytes, same scales; padding rows
