@@ -2363,6 +2363,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// the walking kernels address a tile's weight scales with 32-bit byte offsets from the tile's first scale
+static bool scale_offsets_fit_32_bits(const GemmArgs& p) {
+    return p.sb_stride_n >= 0 && p.sb_stride_k >= 0 && (int64_t)(p.K >> 7) * p.sb_stride_k + 2 * p.sb_stride_n < (1ll << 29);
+}
+
 template <int BM, int BN, int MODE>
 static int launch_block_w8p(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / BM;
@@ -2418,7 +2423,8 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     p.tiles_n = p.N / BN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
-    if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && blocks > cu_count() && p.ld_out < (1 << 21) && p.ld_hs < (1 << 20)) {
+    if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && blocks > cu_count() && p.ld_out < (1 << 21) && p.ld_hs < (1 << 20) &&
+        scale_offsets_fit_32_bits(p)) {
         // 12 to 32 K steps: one workgroup per CU that walks its tiles
         const int cus = cu_count();
         const int KT = p.K >> 7;
@@ -2457,7 +2463,7 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
             // N = 7168 1258 against 1360 us; K = 768: 177 against 172 us, that stays on the kernel below).  The epilogue
             // addresses a tile's rows with 32-bit offsets.
             if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 128) * (p.N / 256) > cu_count() &&
-                p.ld_out < (1 << 21))
+                p.ld_out < (1 << 21) && scale_offsets_fit_32_bits(p))
                 return launch_block_w8p<128, 256, kGrouped>(p, out_dtype, st);
             return launch_block_w8<128, 256, kGrouped>(p, out_dtype, st);
         }
@@ -2480,7 +2486,8 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
         // more tiles than CUs and a short K: one workgroup per CU that walks its tiles, so that a tile does not begin
         // and end on an idle CU (8192 x 4096 x 512: 35 against 42 us, 4096 x 7168 x 2048: 79 against 83 us; from
         // K = 7168 on both forms run level, the K loop is all there is)
-        if ((p.K >> 7) >= 3 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 256) * (p.N / 128) > cu_count())
+        if ((p.K >> 7) >= 3 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 256) * (p.N / 128) > cu_count() &&
+            scale_offsets_fit_32_bits(p))
             return launch_block_w8p<256, 128, kBlock>(p, out_dtype, st);
         return launch_block_w8<256, 128, kBlock>(p, out_dtype, st);
     }
