@@ -2423,9 +2423,9 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     p.tiles_n = p.N / BN;
     const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
     if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
-    if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && blocks > cu_count() && p.ld_out < (1 << 21) && p.ld_hs < (1 << 20) &&
+    if ((p.K >> 7) >= 7 && (p.K >> 7) <= kPersistentBlockSteps && blocks > cu_count() && p.ld_out < (1 << 21) && p.ld_hs < (1 << 20) &&
         scale_offsets_fit_32_bits(p)) {
-        // 12 to 32 K steps: one workgroup per CU that walks its tiles
+        // 7 to 32 K steps: one workgroup per CU that walks its tiles
         const int cus = cu_count();
         const int KT = p.K >> 7;
         const size_t lds = (size_t)(2 * BM + 3 * BN) * 128 + 2 * 8 * BM * sizeof(float) + 8 * 16 * 144 + 2 * 128 * sizeof(int32_t) +
@@ -2459,10 +2459,11 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
         // groups are 128-row aligned, so a tile is 128 rows; 256 columns per workgroup (8 waves) read a
         // quarter fewer operand bytes per flop than 128
         if (p.M % 128 == 0 && p.N % 256 == 0 && (int64_t)(p.M / 128) * (p.N / 256) >= 384 && (p.K >> 7) * 2 <= kMaxTileWeightScales) {
-            // 12 to 32 K steps: one workgroup per CU that walks its tiles (73600 rows, K = 2048: N = 1536 279 against 293 us,
-            // N = 7168 1258 against 1360 us; K = 768: 177 against 172 us, that stays on the kernel below).  The epilogue
-            // addresses a tile's rows with 32-bit offsets.
-            if ((p.K >> 7) >= 12 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 128) * (p.N / 256) > cu_count() &&
+            // 7 to 32 K steps: one workgroup per CU that walks its tiles (73600 rows, N = 2048: K = 896 196 against 215 us,
+            // K = 1024 206 against 233 us, K = 1408 271 against 300 us; K = 2048, N = 7168: 1258 against 1360 us; K = 768:
+            // 177 against 172 us, and level from K = 4608 on, those stay on the kernel below).  The epilogue addresses a
+            // tile's rows with 32-bit offsets.
+            if ((p.K >> 7) >= 7 && (p.K >> 7) <= kPersistentBlockSteps && (int64_t)(p.M / 128) * (p.N / 256) > cu_count() &&
                 p.ld_out < (1 << 21) && scale_offsets_fit_32_bits(p))
                 return launch_block_w8p<128, 256, kGrouped>(p, out_dtype, st);
             return launch_block_w8<128, 256, kGrouped>(p, out_dtype, st);
