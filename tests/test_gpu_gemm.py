@@ -423,6 +423,35 @@ def test_grouped_gemm(dev, T, E, K, N, topk):
     assert torch.equal(out2.cpu()[rows0], out[perm])
 
 
+def test_walking_kernels_repeatable(dev):
+    """The kernels in which one workgroup walks several tiles keep loads of the next tile in flight across the
+    epilogue of the current one; a missing wait or barrier there would show as run-to-run differences.  The same
+    call five times gives the same bits, rowwise and block-scaled, fp32 and bf16 output."""
+    g = torch.Generator(device=dev).manual_seed(5)
+    for mode, (M, N, K) in (("row", (2304, 11520, 512)), ("row", (8192, 4864, 896)), ("blk", (1024, 12288, 1536)), ("blk", (2048, 6400, 640))):
+        qx = torch.randint(0, 256, (M, K), generator=g, device=dev, dtype=torch.uint8)
+        qw = torch.randint(0, 256, (N, K), generator=g, device=dev, dtype=torch.uint8)
+        qx[(qx & 0x7F) == 0x7F] = 0x30
+        qw[(qw & 0x7F) == 0x7F] = 0x30
+        a, b = qx.view(torch.float8_e4m3fn), qw.view(torch.float8_e4m3fn)
+        for dt in (torch.float32, torch.bfloat16):
+            runs = []
+            for _ in range(5):
+                if mode == "row":
+                    if not runs:
+                        sx = torch.rand(M, 1, generator=g, device=dev) + 0.5
+                        sw = torch.rand(N, 1, generator=g, device=dev) + 0.5
+                    runs.append(ops.scaled_mm(a, b.t(), sx, sw.t(), out_dtype=dt))
+                else:
+                    if not runs:
+                        sx = torch.rand(M, K // 128, generator=g, device=dev) + 0.5
+                        sw = torch.rand(N // 128, K // 128, generator=g, device=dev) + 0.5
+                    o = torch.empty(M, N, dtype=dt, device=dev)
+                    ops.gemm_fp8_fp8_bf16_nt((a, sx), (b, sw), o)
+                    runs.append(o)
+            assert all(torch.equal(runs[0], r) for r in runs[1:]), f"{mode} {M}x{N}x{K} {dt}: runs differ"
+
+
 def test_random_shapes_all_dispatch_paths(dev):
     """Seeded sweep over row counts on both sides of every dispatch threshold (16, 32, 64, 128, 256, 512, multiples of
     256 and not), N a multiple of 16 or 256, K 1..9 steps: rowwise mm, fused linear and block-scaled mm."""
