@@ -16,6 +16,7 @@ OUT_F32 = 1
 GROUP_MODE_DIV = 0
 GROUP_MODE_DEEPEP = 1
 TENSORWISE_AMAX_SLOTS = 64
+TENSORWISE_STATIC_MAX_TENSORS = 512
 IN_BF16, IN_F16, IN_F32 = 0, 1, 2
 COMBINE_BF16_STEPS, COMBINE_F32 = 0, 1
 
@@ -33,6 +34,7 @@ SIGNATURES = {
     "cfp8_quant_rowwise": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_quant_rowwise_from": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
+    "cfp8_quant_tensorwise_multi_static": (c_int, [POINTER(TensorDesc), c_int64, c_void_p]),
     "cfp8_tensorwise_amax_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_tensorwise_cast_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),

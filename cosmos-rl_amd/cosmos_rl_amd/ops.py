@@ -151,6 +151,33 @@ def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.
     return outs, scales
 
 
+def quant_tensorwise_multi_static(tensors: Sequence[torch.Tensor], outs: Sequence[torch.Tensor],
+                                  scales: torch.Tensor) -> None:
+    """``quant_tensorwise_multi`` into caller-owned ``outs`` (fp8, shaped like the inputs, contiguous)
+    and ``scales`` (fp32 [n]) through the entry point that allocates nothing: the amax slots are the
+    library's own fixed device array, so at most ``_lib.TENSORWISE_STATIC_MAX_TENSORS`` tensors per
+    call, and calls that overlap on one GPU race on that array.  Nothing is allocated here either;
+    non-contiguous inputs are refused instead of copied."""
+    n = len(tensors)
+    if len(outs) != n or scales.numel() != n or scales.dtype != torch.float32 or not scales.is_contiguous():
+        raise ValueError("outs and scales must match the tensors: one fp8 tensor and one fp32 scale each")
+    if n == 0:
+        return
+    _need_gpu(scales, *tensors, *outs)
+    descs = (_lib.TensorDesc * n)()
+    sbase = scales.data_ptr()
+    for i, (t, q) in enumerate(zip(tensors, outs)):
+        if t.dtype != torch.bfloat16 or q.dtype != FP8_DTYPE:
+            raise ValueError(f"tensor {i}: expected bfloat16 in and float8_e4m3fn out, got {t.dtype} and {q.dtype}")
+        if not t.is_contiguous() or not q.is_contiguous() or q.numel() != t.numel():
+            raise ValueError(f"tensor {i}: input and output must be contiguous and of equal size")
+        descs[i].x = t.data_ptr()
+        descs[i].q = q.data_ptr()
+        descs[i].scale = sbase + 4 * i
+        descs[i].numel = t.numel()
+    _lib.check(_lib.load().cfp8_quant_tensorwise_multi_static(descs, n, _stream()))
+
+
 def quant_tensorwise(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """One global amax, one fp32 scale (shape [1]), saturated cast: the tensorwise recipe
     selected at cosmos_rl/utils/fp8/fp8_util.py:121-137."""

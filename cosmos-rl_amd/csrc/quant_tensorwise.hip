@@ -13,6 +13,8 @@
 // The table of tensors travels in the kernel arguments (scalar loads), so the
 // library needs no device-side descriptor buffer.
 
+#include <mutex>
+
 #include "cfp8_common.h"
 
 namespace cfp8 {
@@ -164,7 +166,58 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
     return check_launch("quant_tensorwise");
 }
 
+// ---- amax slots owned by the library, for callers that cannot allocate -------------------------
+// One copy of this array lives on every GPU the library's code object is loaded on, at that GPU's
+// own address.  In host code the name below is only a handle for hipGetSymbolAddress; kernels and
+// every other use of the memory take the per-device pointer looked up in static_slots().
+constexpr int kStaticMaxTensors = CFP8_TENSORWISE_STATIC_MAX_TENSORS;
+static __device__ __align__(256) u32 scratch[kStaticMaxTensors * kAmaxSlots];
+
+constexpr int kMaxDevices = 64;
+static u32* g_static_slots[kMaxDevices];  // guarded by g_static_mutex; null until looked up
+static std::mutex g_static_mutex;
+
+// Device address of `scratch` on the current device, looked up once per device with that device
+// current.
+static int static_slots(u32** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return set_error(CFP8_EARCH, "quant_tensorwise_static: no current HIP device with an ordinal below %d", kMaxDevices);
+    }
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_slots[dev]) {
+        u32* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            return set_error(CFP8_ELAUNCH, "quant_tensorwise_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                             hipGetErrorString(e));
+        }
+        g_static_slots[dev] = ptr;
+    }
+    *out = g_static_slots[dev];
+    return CFP8_OK;
+}
+
 }  // namespace cfp8
+
+extern "C" int cfp8_quant_tensorwise_multi_static(const cfp8_tensor_desc* descs, int64_t n, void* stream) {
+    using namespace cfp8;
+    if (n < 0) return set_error(CFP8_EINVAL, "quant_tensorwise_static: bad tensor count");
+    if (n > kStaticMaxTensors)
+        return set_error(CFP8_EWORKSPACE,
+                         "quant_tensorwise_static: %lld tensors exceed the %d the library's own amax slots hold; "
+                         "split the call or use cfp8_quant_tensorwise_multi with a workspace",
+                         (long long)n, kStaticMaxTensors);
+    if (n == 0) return CFP8_OK;
+    if (!descs) return set_error(CFP8_EINVAL, "quant_tensorwise_static: null descriptor table");
+    if (int rc = check_device()) return rc;
+    u32* slots = nullptr;
+    if (int rc = static_slots(&slots)) return rc;
+    // the amax phase clears the n * kAmaxSlots slots it uses with a fill kernel before pass 1
+    return run_tensorwise(descs, n, reinterpret_cast<float*>(slots), stream, kPhaseAmax | kPhaseCast);
+}
 
 extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {
     return cfp8::run_tensorwise(descs, n, amax_ws, stream, cfp8::kPhaseAmax | cfp8::kPhaseCast);

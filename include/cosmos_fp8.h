@@ -106,6 +106,20 @@ int cfp8_tensorwise_amax_multi(const cfp8_tensor_desc* descs, int64_t n,
 int cfp8_tensorwise_cast_multi(const cfp8_tensor_desc* descs, int64_t n,
                                float* amax_ws, void* stream);
 
+/* cfp8_quant_tensorwise_multi without a workspace argument and without any allocation: the amax
+ * slots are a fixed array inside the library's device image (CFP8_TENSORWISE_STATIC_MAX_TENSORS *
+ * CFP8_TENSORWISE_AMAX_SLOTS * 4 bytes = 128 KiB, held on every GPU the library is used on until
+ * the process ends).  No counterpart in the reference: it is for callers that cannot allocate
+ * device memory - code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  The call makes no hipMalloc / hipFree and calls no allocating routine; inputs and
+ * outputs are still the caller's.  n > CFP8_TENSORWISE_STATIC_MAX_TENSORS returns
+ * CFP8_EWORKSPACE.  All calls on one GPU share the one array (each call clears the slots it
+ * uses first), so two calls that overlap on one GPU - different streams, or different threads -
+ * race; calls on one stream are ordered and safe.  Results are bit-identical to
+ * cfp8_quant_tensorwise_multi. */
+#define CFP8_TENSORWISE_STATIC_MAX_TENSORS 512
+int cfp8_quant_tensorwise_multi_static(const cfp8_tensor_desc* descs, int64_t n, void* stream);
+
 /* Single-tensor form of cfp8_quant_tensorwise_multi. */
 int cfp8_quant_tensorwise(const void* x, int64_t numel, void* q, float* scale,
                           float* amax_ws, void* stream);

@@ -36,6 +36,7 @@ def test_header_constants_match_binding():
     assert val("CFP8_OUT_BF16") == _lib.OUT_BF16 and val("CFP8_OUT_F32") == _lib.OUT_F32
     assert val("CFP8_GROUP_MODE_DIV") == _lib.GROUP_MODE_DIV and val("CFP8_GROUP_MODE_DEEPEP") == _lib.GROUP_MODE_DEEPEP
     assert val("CFP8_TENSORWISE_AMAX_SLOTS") == _lib.TENSORWISE_AMAX_SLOTS
+    assert val("CFP8_TENSORWISE_STATIC_MAX_TENSORS") == _lib.TENSORWISE_STATIC_MAX_TENSORS
     assert (val("CFP8_IN_BF16"), val("CFP8_IN_F16"), val("CFP8_IN_F32")) == (_lib.IN_BF16, _lib.IN_F16, _lib.IN_F32)
     assert (val("CFP8_COMBINE_BF16_STEPS"), val("CFP8_COMBINE_F32")) == (_lib.COMBINE_BF16_STEPS, _lib.COMBINE_F32)
     assert ctypes.sizeof(_lib.TensorDesc) == 32
@@ -59,6 +60,13 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert lib.cfp8_gemm_block128(None, 128, None, None, 128, None, 1, 1, None, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert lib.cfp8_quant_tensorwise_multi(None, 3, None, None) == _lib.EINVAL
+    # the entry point with the library's own amax slots: its capacity is checked before any device call
+    many = (_lib.TensorDesc * (_lib.TENSORWISE_STATIC_MAX_TENSORS + 1))()
+    assert lib.cfp8_quant_tensorwise_multi_static(many, _lib.TENSORWISE_STATIC_MAX_TENSORS + 1, None) == _lib.EWORKSPACE
+    assert "exceed" in _lib.last_error()
+    assert lib.cfp8_quant_tensorwise_multi_static(None, 0, None) == 0
+    assert lib.cfp8_quant_tensorwise_multi_static(None, 2, None) == _lib.EINVAL
+    assert lib.cfp8_quant_tensorwise_multi_static(None, -1, None) == _lib.EINVAL
     # shape checks come before any device access: host pointers are never dereferenced here
     buf = ctypes.create_string_buffer(4096)
     ptr = (ctypes.addressof(buf) + 255) & ~255
