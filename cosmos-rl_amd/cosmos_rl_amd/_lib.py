@@ -27,12 +27,18 @@ class TensorDesc(ctypes.Structure):
     _fields_ = [("x", c_void_p), ("q", c_void_p), ("scale", c_void_p), ("numel", c_int64)]
 
 
+class RowwiseDesc(ctypes.Structure):
+    _fields_ = [("x", c_void_p), ("q", c_void_p), ("scales", c_void_p), ("rows", c_int64), ("cols", c_int64),
+                ("ld_x", c_int64), ("ld_q", c_int64), ("x_dtype", c_int32), ("reserved", c_int32)]
+
+
 # name -> (restype, argtypes); must list every symbol the header declares
 SIGNATURES = {
     "cfp8_version": (c_int, []),
     "cfp8_last_error": (c_char_p, []),
     "cfp8_quant_rowwise": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_quant_rowwise_from": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "cfp8_quant_rowwise_multi": (c_int, [POINTER(RowwiseDesc), c_int64, c_void_p]),
     "cfp8_quant_tensorwise_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise_multi_static": (c_int, [POINTER(TensorDesc), c_int64, c_void_p]),
     "cfp8_tensorwise_amax_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),

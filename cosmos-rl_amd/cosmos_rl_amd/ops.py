@@ -106,12 +106,7 @@ def quant_rowwise_into(recv: torch.Tensor, q_out: torch.Tensor, scale_out: torch
     if q_out.dtype != FP8_DTYPE or scale_out.dtype != torch.float32:
         raise ValueError("q_out must be float8_e4m3fn and scale_out float32")
     rows, cols = recv.shape
-    if q_out.dim() == 2 and tuple(q_out.shape) == (rows, cols) and (q_out.stride(1) == 1 or cols == 1):
-        q_rm = q_out
-    elif q_out.dim() == 2 and tuple(q_out.shape) == (cols, rows) and (q_out.stride(0) == 1 or cols == 1):
-        q_rm = q_out.t()
-    else:
-        raise ValueError(f"q_out {tuple(q_out.shape)} strides {q_out.stride()} is not row-major storage for {tuple(recv.shape)}")
+    q_rm = _row_major_q(q_out, rows, cols)
     if scale_out.numel() != rows or not scale_out.is_contiguous():
         raise ValueError(f"scale_out must hold {rows} contiguous floats, got {tuple(scale_out.shape)}")
     if recv.stride(1) != 1 and cols > 1:
@@ -120,6 +115,58 @@ def quant_rowwise_into(recv: torch.Tensor, q_out: torch.Tensor, scale_out: torch
     ld_q = q_rm.stride(0) if rows > 1 else max(cols, 1)
     _lib.check(_lib.load().cfp8_quant_rowwise_from(recv.data_ptr(), _IN_DTYPE[recv.dtype], rows, cols, ld_x,
                                                   q_rm.data_ptr(), ld_q, scale_out.data_ptr(), _stream()))
+
+
+def _row_major_q(q_out: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """The [rows, cols] row-major view of fp8 storage given either that way or as the engine's
+    transposed parameter [cols, rows] with strides (1, pitch)."""
+    if q_out.dim() == 2 and tuple(q_out.shape) == (rows, cols) and (q_out.stride(1) == 1 or cols == 1):
+        return q_out
+    if q_out.dim() == 2 and tuple(q_out.shape) == (cols, rows) and (q_out.stride(0) == 1 or cols == 1):
+        return q_out.t()
+    raise ValueError(f"q_out {tuple(q_out.shape)} strides {q_out.stride()} is not row-major storage for {(rows, cols)}")
+
+
+def quant_rowwise_multi_into(recvs: Sequence[torch.Tensor], q_outs: Sequence[torch.Tensor],
+                             scale_outs: Sequence[torch.Tensor]) -> None:
+    """``quant_rowwise_into`` for a batch of weights in as few launches as their shapes allow (weights of one
+    row length and dtype share a launch): the completions a weight sync runs together once their shards have
+    landed (cosmos_rl/rollout/worker/rollout_control.py:1308-1319).  Same bits as per-weight calls."""
+    n = len(recvs)
+    if len(q_outs) != n or len(scale_outs) != n:
+        raise ValueError("one output and one scale tensor per weight")
+    if n == 0:
+        return
+    _need_gpu(*recvs, *q_outs, *scale_outs)
+    descs = (_lib.RowwiseDesc * n)()
+    keep = []
+    for i, (recv, q_out, scale_out) in enumerate(zip(recvs, q_outs, scale_outs)):
+        if recv.dim() != 2 or recv.dtype not in _IN_DTYPE:
+            raise ValueError(f"weight {i}: expected a 2-D bf16/fp16/fp32 tensor, got {tuple(recv.shape)} {recv.dtype}")
+        if q_out.dtype != FP8_DTYPE or scale_out.dtype != torch.float32:
+            raise ValueError(f"weight {i}: q_out must be float8_e4m3fn and scale_out float32")
+        rows, cols = recv.shape
+        q_rm = _row_major_q(q_out, rows, cols)
+        if scale_out.numel() != rows or not scale_out.is_contiguous():
+            raise ValueError(f"weight {i}: scale_out must hold {rows} contiguous floats, got {tuple(scale_out.shape)}")
+        if recv.stride(1) != 1 and cols > 1:
+            recv = recv.contiguous()
+        keep.append(recv)
+        d = descs[i]
+        d.x, d.q, d.scales = recv.data_ptr(), q_rm.data_ptr(), scale_out.data_ptr()
+        d.rows, d.cols = rows, cols
+        d.ld_x = recv.stride(0) if rows > 1 else max(cols, 1)
+        d.ld_q = q_rm.stride(0) if rows > 1 else max(cols, 1)
+        d.x_dtype = _IN_DTYPE[recv.dtype]
+    _lib.check(_lib.load().cfp8_quant_rowwise_multi(descs, n, _stream()))
+
+
+def quant_rowwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Tensor], List[torch.Tensor]]:
+    """Rowwise quantisation of a list of 2-D weights; returns (fp8 tensors [R, C], fp32 scales [R, 1])."""
+    qs = [torch.empty(t.shape, dtype=FP8_DTYPE, device=t.device) for t in tensors]
+    ss = [torch.empty((t.shape[0], 1), dtype=torch.float32, device=t.device) for t in tensors]
+    quant_rowwise_multi_into(tensors, qs, ss)
+    return qs, ss
 
 
 def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Tensor], torch.Tensor]:
@@ -470,12 +517,17 @@ def grouped_gemm_swiglu_quant(lhs: Tuple[torch.Tensor, torch.Tensor], rhs_interl
     return q, s
 
 
-def create_indices_from_offsets_nosync(m_offsets: torch.Tensor, total: Optional[int] = None) -> torch.Tensor:
+def create_indices_from_offsets_nosync(m_offsets: torch.Tensor, total: Optional[int] = None,
+                                       n_experts: Optional[int] = None) -> torch.Tensor:
     """``dsgemm_utils.create_indices_from_offsets_nosync`` (group_gemms.py:157): expert id per
     row from the inclusive cumulative group ends.  Pass ``total`` (the number of rows, which the
     caller already knows from its own slice at group_gemms.py:154) to stay free of a host sync;
-    without it the last offset is read back."""
+    without it the last offset is read back.  With ``n_experts`` given, ``total`` may be any bound on
+    the row count: rows past the last group get -1 (padding to the grouped GEMMs)."""
     if total is None:
         total = int(m_offsets[-1])
     rows = torch.arange(total, device=m_offsets.device, dtype=m_offsets.dtype)
-    return torch.searchsorted(m_offsets, rows, right=True).to(torch.int32)
+    idx = torch.searchsorted(m_offsets, rows, right=True).to(torch.int32)
+    if n_experts is not None:
+        idx = torch.where(idx < n_experts, idx, torch.full_like(idx, -1))
+    return idx

@@ -91,12 +91,22 @@ class DSGroupGEMM(GroupGEMMStrategy):
         fp8, scales = ops.prepare_fp8_weight(combined_weights)
         module.register_parameter(f"{submod_name}_fp8", nn.Parameter(fp8, requires_grad=False))
         module.register_parameter(f"{submod_name}_scales", nn.Parameter(scales, requires_grad=False))
+        self.invalidate_fused_weights(module)
         return combined_weights
 
     def _quant(self, x):
         return ops.groupwise_activation_quant(x) if self.use_triton_quant else ops.prepare_fp8_input(x)
 
     def execute(self, contig_tokens, m_sizes, m_offsets, module):
+        rows = contig_tokens.shape[0]
+        if rows % ops.BLOCK == 0 and contig_tokens.is_contiguous():
+            # The row count of the buffer already bounds the valid rows (group_gemms.py:154 slices it with
+            # m_offsets[-1], a host read-back): every row is quantised, rows past the last group get expert -1,
+            # which the GEMMs skip, and the down projection writes straight into ``contig_tokens`` - the rows the
+            # reference's final copy (:228) leaves alone stay untouched, and nothing waits for the device.
+            m_indices = ops.create_indices_from_offsets_nosync(m_offsets, rows, n_experts=m_offsets.numel())
+            self._run(self._quant(contig_tokens), m_indices, rows, module, contig_tokens.dtype, out=contig_tokens)
+            return contig_tokens
         total = int(m_offsets[-1])
         valid_tokens = contig_tokens[:total]
         m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
@@ -106,14 +116,38 @@ class DSGroupGEMM(GroupGEMMStrategy):
     def execute_from_tokens(self, tokens, row_tokens, m_sizes, m_offsets, module):
         """``execute`` on ``tokens[row_tokens]`` (zero rows for -1) without building that matrix: the gather and the
         1x128 quantisation of the first GEMM's input are one pass over the token matrix.  Returns the expert outputs
-        [rows, hidden] for the rows of the expert-grouped layout (``row_tokens``: token behind each row)."""
+        [rows, hidden] for the rows of the expert-grouped layout (``row_tokens``: token behind each row).  When
+        ``row_tokens`` has a multiple of 128 entries (a capacity bound, as ``route_tokens`` returns) nothing is read
+        back from the device: rows past the last group are padding to the GEMMs and come back as zeros."""
         from cosmos_rl_amd.policy.kernel.moe.indices import permute_quantize_tokens
+        rows = row_tokens.numel()
+        if rows % ops.BLOCK == 0:
+            m_indices = ops.create_indices_from_offsets_nosync(m_offsets, rows, n_experts=m_offsets.numel())
+            hidden_size = module.get_parameter("down_proj_weight").shape[1]
+            out = torch.zeros((rows, hidden_size), device=tokens.device, dtype=tokens.dtype)
+            return self._run(permute_quantize_tokens(tokens, row_tokens), m_indices, rows, module, tokens.dtype, out=out)
         total = int(m_offsets[-1])
         m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
         return self._run(permute_quantize_tokens(tokens, row_tokens[:total]), m_indices, total, module, tokens.dtype)
 
-    def _run(self, gate_up_input, m_indices, total, module, dt):
-        """gate/up GEMMs, activation, requantisation, down GEMM on the quantised expert-grouped rows"""
+    @staticmethod
+    def _weights_key(*tensors):
+        # address and in-place version of every tensor a fused copy was built from: an in-place update (copy_,
+        # load_state_dict) keeps the address and bumps the version.  A write through ``tensor.data`` bumps nothing:
+        # whoever updates the expert weights that way calls ``invalidate_fused_weights`` afterwards.
+        return tuple((t.data_ptr(), t._version) for t in tensors)
+
+    @staticmethod
+    def invalidate_fused_weights(module) -> None:
+        """Drop the fused / interleaved copies of the gate and up weights kept on ``module``; the next ``execute``
+        rebuilds them.  ``arrange_expert_weights`` calls it, so re-arranged weights are always picked up."""
+        for attr in ("_gate_up_fp8_interleaved", "_gate_up_fp8_fused"):
+            if hasattr(module, attr):
+                delattr(module, attr)
+
+    def _run(self, gate_up_input, m_indices, total, module, dt, out=None):
+        """gate/up GEMMs, activation, requantisation, down GEMM on the quantised expert-grouped rows; the result
+        goes to ``out`` ([total, hidden], rows of padding untouched) when given"""
 
         gate_fp8, gate_s = module.get_parameter("gate_proj_fp8"), module.get_parameter("gate_proj_scales")
         up_fp8, up_s = module.get_parameter("up_proj_fp8"), module.get_parameter("up_proj_scales")
@@ -123,21 +157,22 @@ class DSGroupGEMM(GroupGEMMStrategy):
         hidden_size = module.get_parameter("down_proj_weight").shape[1]
         dev = gate_up_input[0].device
 
-        down_out = torch.empty((total, hidden_size), device=dev, dtype=dt)
+        down_out = out if out is not None else torch.empty((total, hidden_size), device=dev, dtype=dt)
         # padding rows (m_indices < 0) are not written by the GEMMs: start from zeros so that what the
         # activation reads there is defined
         hidden_quantized = None
         if self.fuse_gate_up and self.fuse_swiglu and self.fuse_epilogue and intermediate_size % 128 == 0 and total % 128 == 0:
+            key = self._weights_key(gate_fp8, up_fp8, gate_s, up_s)
             inter = getattr(module, "_gate_up_fp8_interleaved", None)
-            if inter is None or inter[2] != (gate_fp8.data_ptr(), up_fp8.data_ptr()):
-                inter = (*ops.interleave_gate_up((gate_fp8, gate_s), (up_fp8, up_s)), (gate_fp8.data_ptr(), up_fp8.data_ptr()))
+            if inter is None or inter[2] != key:
+                inter = (*ops.interleave_gate_up((gate_fp8, gate_s), (up_fp8, up_s)), key)
                 module._gate_up_fp8_interleaved = inter
             hidden_quantized = ops.grouped_gemm_swiglu_quant(gate_up_input, (inter[0], inter[1]), m_indices)
         elif self.fuse_gate_up and intermediate_size % 128 == 0:
+            key = self._weights_key(gate_fp8, up_fp8, gate_s, up_s)
             fused = getattr(module, "_gate_up_fp8_fused", None)
-            if fused is None or fused[2] != (gate_fp8.data_ptr(), up_fp8.data_ptr()):
-                fused = (torch.cat([gate_fp8, up_fp8], dim=1), torch.cat([gate_s, up_s], dim=1),
-                         (gate_fp8.data_ptr(), up_fp8.data_ptr()))
+            if fused is None or fused[2] != key:
+                fused = (torch.cat([gate_fp8, up_fp8], dim=1), torch.cat([gate_s, up_s], dim=1), key)
                 module._gate_up_fp8_fused = fused
             gate_up_out = torch.zeros((total, 2 * intermediate_size), device=dev, dtype=dt)
             ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(gate_up_input, (fused[0], fused[1]), gate_up_out, m_indices)

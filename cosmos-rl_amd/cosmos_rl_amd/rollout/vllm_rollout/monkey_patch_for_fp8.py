@@ -27,13 +27,22 @@ class Fp8LinearOp:
             raise NotImplementedError("only the per-token (rowwise) FP8 linear is on this path")
         self.cutlass_fp8_supported = cutlass_fp8_supported
         self.use_per_token_if_dynamic = use_per_token_if_dynamic
+        # the scaled-mm kernel comes from the dispatch function, as in the engine the reference patches
+        self.w8a8_scaled_mm = _dispatch["dispatch_w8a8_scaled_mm"](cutlass_fp8_supported, True, use_per_token_if_dynamic)
 
     def apply(self, input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
               out_dtype: Optional[torch.dtype] = None, input_scale: Optional[torch.Tensor] = None,
               input_scale_ub: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         if input_scale is not None:
             raise NotImplementedError("static activation scales are not on this path")
-        return ops.fp8_linear(input, weight, weight_scale, bias=bias, out_dtype=out_dtype or input.dtype)
+        if self.w8a8_scaled_mm is torch_per_token_w8a8_scaled_mm:
+            # the per-token rowwise kernel: quantisation and GEMM as one library call
+            return ops.fp8_linear(input, weight, weight_scale, bias=bias, out_dtype=out_dtype or input.dtype)
+        x2 = input.reshape(-1, input.shape[-1])
+        qinput, x_scale = ops.scaled_fp8_quant(x2, scale=None, use_per_token_if_dynamic=True)
+        out = self.w8a8_scaled_mm(qinput=qinput, weight=weight, out_dtype=out_dtype or input.dtype, scale_a=x_scale,
+                                  scale_b=weight_scale, bias=bias)
+        return out.reshape(*input.shape[:-1], out.shape[-1])
 
 
 class Fp8LinearMethod:
@@ -58,11 +67,19 @@ def torch_per_token_w8a8_scaled_mm(*, qinput: torch.Tensor, weight: torch.Tensor
     return ops.scaled_mm(qinput, weight, scale_a, scale_b, out_dtype=out_dtype, bias=bias)
 
 
-_dispatch = {"w8a8_scaled_mm": torch_per_token_w8a8_scaled_mm}
+def dispatch_w8a8_scaled_mm(cutlass_fp8_supported: bool, per_tensor_weights: bool, per_tensor_activations: bool):
+    """The engine's kernel choice for an FP8 linear.  Only one kernel exists on this path, so the unpatched
+    choice is already the per-token rowwise mm; the name is kept because the reference replaces it."""
+    return torch_per_token_w8a8_scaled_mm
+
+
+# what ``Fp8LinearOp.__init__`` asks for its scaled-mm kernel; ``apply_patch_to_dispatch`` replaces the entry
+_dispatch = {"dispatch_w8a8_scaled_mm": dispatch_w8a8_scaled_mm}
 
 
 def apply_patch_to_dispatch():
-    """monkey_patch_for_fp8.py:26-34: every FP8 linear goes through the per-token rowwise mm."""
+    """monkey_patch_for_fp8.py:26-34: every FP8 linear constructed from now on goes through the per-token
+    rowwise mm, whatever the engine's own dispatch would have picked."""
     def dispatch_fp8_linear_kernel_to_torch_scaled_mm(*args, **kwargs):
         return torch_per_token_w8a8_scaled_mm
 

@@ -23,10 +23,41 @@ def fp8_quantization(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 class FP8RolloutMixin:
     """Methods a rollout backend mixes in to serve an FP8 engine: the quantiser and the two
     hooks of ``RolloutBase`` (cosmos_rl/rollout/rollout_base.py:138-185) as vLLMRollout fills
-    them for ``quantization_type == "fp8"``.  The host class provides ``get_underlying_model()``."""
+    them for ``quantization_type == "fp8"``, and the parameter map weight sync copies into
+    (rollout_base.py:186-230).  The host class provides ``get_underlying_model()`` and sets
+    ``_engine_initialized`` once its engine is up, as ``RolloutBase`` does."""
+
+    _engine_initialized: bool = False
+    _model_param_map = None  # key: compatible name, value: param
 
     def fp8_quantization(self, weight: torch.Tensor):
         return fp8_quantization(weight)
+
+    def is_engine_initialized(self) -> bool:
+        return self._engine_initialized
+
+    def get_quantized_tensors(self, weight_mapper) -> Dict[str, torch.Tensor]:
+        """rollout_base.py:211-230: quantised tensors that live outside the model's state dict.  For FP8 the
+        engine's fp8 weights and ``weight_scale`` tensors are ordinary parameters, so the map is empty (the
+        reference fills it for MXFP4 only, vllm_rollout.py:1088-1120)."""
+        if not self._engine_initialized:
+            raise RuntimeError("[Rollout] Engine is not initialized, please call init_engine first.")
+        return {}
+
+    def model_param_map(self, weight_mapper) -> Dict[str, torch.Tensor]:
+        """rollout_base.py:186-209: every parameter of the rollout model under its HF-compatible name, plus
+        the quantised tensors; built once and cached."""
+        if not self._engine_initialized:
+            raise RuntimeError("[Rollout] Engine is not initialized, please call init_engine first.")
+        if self._model_param_map:
+            return self._model_param_map
+        model = self.get_underlying_model()
+        param_map = {}
+        for name, param in model.state_dict().items():
+            param_map[weight_mapper.rollout_map_local_key_to_hf_key(name)] = param
+        param_map.update(self.get_quantized_tensors(weight_mapper))
+        self._model_param_map = param_map
+        return self._model_param_map
 
     def pre_get_params_for_sync_hook(self, quantization_type, weight_mapper, parallel_dims=None,
                                      promotion_dtype: torch.dtype = torch.bfloat16, **kwargs

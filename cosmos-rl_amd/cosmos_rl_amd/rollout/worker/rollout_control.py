@@ -86,6 +86,42 @@ class QuantizedWeightReceiver:
         scale_tensor.copy_(weight_scale)
         return True
 
+    # -- rollout_control.py:1308-1319: the completions of a flush group, run together ---------------------
+    def flush_completions(self, groups: Iterable[List[str]], do_weight_sync_check: bool = False) -> List[str]:
+        """Quantise the full weights of several instruction groups whose shards have all landed, as the
+        reference's ``flush_completions`` runs its queued completion lambdas together on the copy stream.
+        Without the first-sync check the weights of the batch that share a row length go through ONE launch
+        each way (``cfp8_quant_rowwise_multi``), straight from the staging parameters into the engine's fp8
+        parameters and ``weight_scale`` tensors - same bytes as one ``quantize_full_weight`` per group.
+        With the check every weight takes ``quantize_full_weight`` (the check compares old and new bytes).
+        Returns the full weight names that were quantised."""
+        from cosmos_rl_amd import ops
+
+        names: List[str] = []
+        for param_names in groups:
+            if self.quantization_type is None or self.check_inside_group(param_names, do_weight_sync_check):
+                continue
+            full = self.full_weight_name_of_group(param_names)
+            if self.quantization_type == "fp8" and full in self.hp_weight_map and full not in names:
+                names.append(full)
+        if do_weight_sync_check:
+            for name in names:
+                self.quantize_full_weight(name, True)
+            return names
+        model_param_map = self.rollout.model_param_map(self.weight_mapper)
+        weights, natives, scales = [], [], []
+        for name in names:
+            weight = self.hp_weight_map[name]                            # [out_dim, in_dim]
+            native = model_param_map[name]                               # [in_dim, out_dim], strides (1, in_dim)
+            scale_tensor = model_param_map[name.replace(".weight", ".weight_scale")]
+            assert tuple(scale_tensor.shape) == (weight.shape[0], 1), (
+                f"scale_tensor.shape: {scale_tensor.shape}, weight_scale.shape: {(weight.shape[0], 1)}")
+            weights.append(weight.data)
+            natives.append(native.data)
+            scales.append(scale_tensor.data)
+        ops.quant_rowwise_multi_into(weights, natives, scales)
+        return names
+
     # -- fused form of base.py:1053-1069 + rollout_control.py:856-898 --------------------------
     def quantize_received_rows(self, full_weight_name: str, recv_tensor: torch.Tensor, row_start: int = 0) -> bool:
         """Quantise a received shard that holds whole rows ``[row_start, row_start + n)`` of a weight

@@ -54,13 +54,23 @@ class FP8Config:
 
 def module_filter_fn(mod: nn.Module, fqn: str, filter_fqns: List[str]) -> bool:
     """fp8_util.py:62-87: convert only ``nn.Linear`` whose two dimensions are multiples of 16
-    and whose fully qualified name contains none of ``filter_fqns``."""
+    and whose fully qualified name contains none of ``filter_fqns``.
+
+    One condition is stricter here than in the reference: the FP8 MFMA GEMM consumes K in steps of
+    128, so ``in_features`` must be a multiple of 128 (the reference's torchao path takes any multiple
+    of 16).  A layer that fails it stays an ``nn.Linear`` and computes in its own dtype instead of
+    being converted and then failing in its first forward."""
     if not isinstance(mod, nn.Linear):
         return False
     out_features, in_features = mod.weight.shape
     if out_features % 16 or in_features % 16:
         return False
+    if in_features % FP8_GEMM_K_STEP:
+        return False
     return not any(f in fqn for f in filter_fqns)
+
+
+FP8_GEMM_K_STEP = 128  # K of one FP8 MFMA step: in_features of a converted layer is a multiple of it
 
 
 def is_gfx950_available() -> bool:
@@ -134,13 +144,13 @@ class FP8ModelConverter(ModelConverter):
             raise NotImplementedError("[FP8] Delayed scaling is not supported yet.")
         self.precompute_scale = False
 
-    def convert_model(self, model: torch.nn.Module) -> Optional[torch.nn.Module]:
+    def convert_model(self, model: torch.nn.Module) -> None:
+        """fp8_util.py:139-152: converts in place and returns nothing."""
         if not self.fp8_config.enable_fp8:
-            return None
+            return
         filter_fqns = model.fqn_filter_for_quantization() if hasattr(model, "fqn_filter_for_quantization") else []
         convert_to_float8_training(model, self.fp8_config.quant_recipe,
                                    module_filter_fn=partial(module_filter_fn, filter_fqns=filter_fqns))
-        return model
 
     def post_optimizer_hook(self, model: Union[nn.Module, List[nn.Module]]):
         # scales are dynamic (recomputed from the weights at every forward); nothing to refresh

@@ -72,15 +72,8 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     const int total = tiles_m * tiles_n;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = total >> 3, rem = total & 7;
-#ifdef CFP8_NO_XCD_REMAP
-    const int lin = pid;
-#else
     const int lin = xcd * base + (xcd < rem ? xcd : rem) + local;
-#endif
-#ifndef CFP8_GM
-#define CFP8_GM 8
-#endif
-    constexpr int GM = CFP8_GM;
+    constexpr int GM = 8;
     const int band = GM * tiles_n;
     const int g = lin / band, first = g * GM;
     const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;

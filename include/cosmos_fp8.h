@@ -75,6 +75,25 @@ int cfp8_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x,
 int cfp8_quant_rowwise_from(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld_x,
                             void* q, int64_t ld_q, float* scales, void* stream);
 
+/* Rowwise quantisation of many weights in as few launches as their shapes allow: what
+ * cfp8_quant_rowwise_from does for each descriptor, with the tensors of equal row-length class
+ * and source dtype sharing a launch (the table travels in the kernel arguments).  For the batch of
+ * completions that a weight sync runs together once their shards have landed,
+ * cosmos_rl/rollout/worker/rollout_control.py:1308-1319 (each completion quantises one full weight,
+ * :856-898); one launch per weight leaves every weight under ~50 MB bound by the ramp-up of its
+ * launch.  The descriptor array lives in HOST memory and is read before the call returns.
+ * Results are bit-identical to per-tensor calls.  Per descriptor: the contract of
+ * cfp8_quant_rowwise_from. */
+typedef struct cfp8_rowwise_desc {
+    const void* x;     /* [rows, cols] of x_dtype, row pitch ld_x elements, 16-byte aligned */
+    void* q;           /* fp8 out, row pitch ld_q bytes, 8-byte aligned                     */
+    float* scales;     /* device, rows floats out                                            */
+    int64_t rows, cols, ld_x, ld_q;
+    int32_t x_dtype;   /* CFP8_IN_*                                                          */
+    int32_t reserved;  /* 0                                                                  */
+} cfp8_rowwise_desc;
+int cfp8_quant_rowwise_multi(const cfp8_rowwise_desc* descs, int64_t n, void* stream);
+
 /* Tensorwise dynamic quantisation of many tensors in two passes (grid amax,
  * then cast), without a host round trip in between.
  * Replaces the torchao tensorwise recipe selected at

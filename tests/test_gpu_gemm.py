@@ -363,6 +363,34 @@ def test_grouped_cfg5_full_size_properties(dev):
     dn = torch.zeros(total, H, dtype=torch.bfloat16, device=dev)
     ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qh, sh), (qd, sd), dn, m_idx)
     check_bf16(dn[rows], ref_rows(qh, sh, qd, sd, rows).float().cpu(), "cfg5 down rows")
+    # the configuration the benchmark times: the gate_up GEMM on interleaved weights with the SwiGLU + 1x128
+    # requantisation as its epilogue, at this size in the form where a workgroup walks several tiles - bytes and
+    # scales equal the unfused chain's on every valid row, padding rows untouched
+    qgi, sgi = ops.interleave_gate_up((qgu[:, :I], sgu[:, :I // 128]), (qgu[:, I:], sgu[:, I // 128:]))
+    qf = torch.full((total, I), 0x55, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    sf = torch.full((total, I // 128), -1.0, dtype=torch.float32, device=dev)
+    from cosmos_rl_amd import _lib
+    _lib.check(_lib.load().cfp8_gemm_grouped_swiglu_quant(qx.data_ptr(), H, sx.data_ptr(), qgi.data_ptr(), sgi.data_ptr(), m_idx.data_ptr(),
+                                                         qf.data_ptr(), I, sf.data_ptr(), total, I, H, E,
+                                                         torch.cuda.current_stream().cuda_stream))
+    ok = ~pad
+    assert torch.equal(qf.view(torch.uint8)[ok], qh.view(torch.uint8)[ok]), "fused SwiGLU epilogue: bytes differ from the unfused chain"
+    assert torch.equal(sf[ok].view(torch.int32), sh[ok].view(torch.int32)), "fused SwiGLU epilogue: scales differ"
+    assert bool((qf.view(torch.uint8)[pad] == 0x55).all()) and bool((sf[pad] == -1.0).all()), "fused epilogue wrote padding rows"
+    # ... and the strategy object on top of it, straight from the token matrix (gather + quantise in one pass,
+    # fused gate_up + SwiGLU GEMM, down GEMM), against the chain above
+    import torch.nn as nn
+    from cosmos_rl_amd.policy.kernel.group_gemms import DSGroupGEMM
+    mod = nn.Module()
+    for name, qq, ss in (("gate_proj", qgu[:, :I].contiguous(), sgu[:, :I // 128].contiguous()),
+                         ("up_proj", qgu[:, I:].contiguous(), sgu[:, I // 128:].contiguous()), ("down_proj", qd, sd)):
+        mod.register_parameter(f"{name}_fp8", nn.Parameter(qq, requires_grad=False))
+        mod.register_parameter(f"{name}_scales", nn.Parameter(ss, requires_grad=False))
+    mod.register_parameter("gate_proj_weight", nn.Parameter(torch.empty(E, I, 0, device=dev), requires_grad=False))
+    mod.register_parameter("down_proj_weight", nn.Parameter(torch.empty(E, H, 0, device=dev), requires_grad=False))
+    out_ft = DSGroupGEMM(torch.nn.functional.silu, fuse_gate_up=True).execute_from_tokens(x, r.row_tokens, r.m_sizes, r.m_offsets, mod)
+    assert out_ft.shape[0] == r.row_tokens.numel() and torch.equal(out_ft[:total][ok], dn[ok])
+    assert bool((out_ft[:total][pad] == 0).all()) and bool((out_ft[total:] == 0).all())
     # permutation inside expert 3's group
     rows3 = (m_idx == 3).nonzero().flatten()
     perm = rows3[torch.randperm(rows3.numel(), generator=torch.Generator().manual_seed(1)).to(dev)]
@@ -450,6 +478,88 @@ def test_walking_kernels_repeatable(dev):
                     ops.gemm_fp8_fp8_bf16_nt((a, sx), (b, sw), o)
                     runs.append(o)
             assert all(torch.equal(runs[0], r) for r in runs[1:]), f"{mode} {M}x{N}x{K} {dt}: runs differ"
+
+
+def _grouped_problem(dev, T, E, K, topk, seed):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.rand(T, E, generator=g)
+    logits[:, 1] = -1.0                                   # an expert without tokens: a tile of padding to step over
+    token_of_row, m_indices, _, _ = O.route_topk_contiguous(logits, topk, 128)
+    x = O.make_activation(T, K, seed=seed + 1)
+    xs = torch.zeros(token_of_row.numel(), K, dtype=torch.bfloat16)
+    valid = token_of_row >= 0
+    xs[valid] = x[token_of_row[valid]]
+    qx, sx = ops.groupwise_activation_quant(xs.to(dev))
+    return qx, sx, m_indices.to(dev), valid.to(dev)
+
+
+def test_walking_grouped_kernels_repeatable_and_equal_to_sliced_calls(dev):
+    """The grouped kernel in which a workgroup walks several tiles, plain and with the SwiGLU + requantisation
+    epilogue: five runs give the same bits, and those bits equal what the same problem gives when it is cut along N
+    into calls small enough to take the one-tile-per-workgroup kernels (same arithmetic, other schedule)."""
+    E, topk = 7, 2
+    for K, I, T in ((1536, 1024, 3300), (2048, 768, 4500), (896, 1024, 3300)):
+        qx, sx, mi, valid = _grouped_problem(dev, T, E, K, topk, seed=K)
+        rows = qx.shape[0]
+        qg, sg = ops.per_block_cast_to_fp8(O.make_weight((E, I, K), seed=6, std=0.05).to(dev))
+        qu, su = ops.per_block_cast_to_fp8(O.make_weight((E, I, K), seed=7, std=0.05).to(dev))
+        qw, sw = torch.cat([qg, qu], 1).contiguous(), torch.cat([sg, su], 1).contiguous()
+        N = 2 * I
+        assert (rows // 128) * (N // 256) > 384, "shape must take the walking form"
+        runs = []
+        for _ in range(5):
+            o = torch.full((rows, N), 7.0, dtype=torch.bfloat16, device=dev)
+            ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qw, sw), o, mi)
+            runs.append(o)
+        assert all(torch.equal(runs[0], r) for r in runs[1:]), f"grouped K={K}: runs differ"
+        # the same product from calls of N / 4 columns (fewer than 384 tiles each: the generic kernel)
+        parts = []
+        for c in range(4):
+            n0, n1 = c * N // 4, (c + 1) * N // 4
+            o = torch.full((rows, n1 - n0), 7.0, dtype=torch.bfloat16, device=dev)
+            ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qw[:, n0:n1].contiguous(), sw[:, n0 // 128:n1 // 128].contiguous()), o, mi)
+            parts.append(o)
+        assert torch.equal(torch.cat(parts, 1), runs[0]), f"grouped K={K}: walking form differs from the sliced calls"
+        # SwiGLU epilogue
+        qi, si = ops.interleave_gate_up((qg, sg), (qu, su))
+        outs = [ops.grouped_gemm_swiglu_quant((qx, sx), (qi, si), mi) for _ in range(5)]
+        for q, sc in outs[1:]:
+            assert torch.equal(q.view(torch.uint8)[valid], outs[0][0].view(torch.uint8)[valid]) and torch.equal(sc[valid], outs[0][1][valid]), \
+                f"grouped SwiGLU K={K}: runs differ"
+        q0, s0 = ops.swiglu_quant(runs[0][:, :I], runs[0][:, I:])
+        assert torch.equal(outs[0][0].view(torch.uint8)[valid], q0.view(torch.uint8)[valid]) and torch.equal(outs[0][1][valid], s0[valid])
+
+
+def test_walking_kernels_equal_to_sliced_calls(dev):
+    """Rowwise and block-scaled: a problem with more tiles than CUs (the walking kernels) against the same problem cut
+    along N into calls that fit one round of workgroups (one tile per workgroup, or the generic kernel): same bits."""
+    g = torch.Generator(device=dev).manual_seed(9)
+    for mode, (M, N, K), cuts in (("row", (2304, 11520, 512), 3), ("row", (8192, 7680, 896), 6), ("blk", (1024, 12288, 1536), 2),
+                                  ("blk", (2048, 6400, 640), 2)):
+        qx = torch.randint(0, 256, (M, K), generator=g, device=dev, dtype=torch.uint8)
+        qw = torch.randint(0, 256, (N, K), generator=g, device=dev, dtype=torch.uint8)
+        qx[(qx & 0x7F) == 0x7F] = 0x30
+        qw[(qw & 0x7F) == 0x7F] = 0x30
+        a, b = qx.view(torch.float8_e4m3fn), qw.view(torch.float8_e4m3fn)
+        for dt in (torch.float32, torch.bfloat16):
+            if mode == "row":
+                sx = torch.rand(M, 1, generator=g, device=dev) + 0.5
+                sw = torch.rand(N, 1, generator=g, device=dev) + 0.5
+                whole = ops.scaled_mm(a, b.t(), sx, sw.t(), out_dtype=dt)
+                parts = [ops.scaled_mm(a, b[c * N // cuts:(c + 1) * N // cuts].t(), sx, sw[c * N // cuts:(c + 1) * N // cuts].t(), out_dtype=dt)
+                         for c in range(cuts)]
+            else:
+                sx = torch.rand(M, K // 128, generator=g, device=dev) + 0.5
+                sw = torch.rand(N // 128, K // 128, generator=g, device=dev) + 0.5
+                whole = torch.empty(M, N, dtype=dt, device=dev)
+                ops.gemm_fp8_fp8_bf16_nt((a, sx), (b, sw), whole)
+                parts = []
+                for c in range(cuts):
+                    n0, n1 = c * N // cuts, (c + 1) * N // cuts
+                    o = torch.empty(M, n1 - n0, dtype=dt, device=dev)
+                    ops.gemm_fp8_fp8_bf16_nt((a, sx), (b[n0:n1], sw[n0 // 128:n1 // 128].clone()), o)
+                    parts.append(o)
+            assert torch.equal(torch.cat(parts, 1), whole), f"{mode} {M}x{N}x{K} {dt}: walking form differs from the sliced calls"
 
 
 def test_random_shapes_all_dispatch_paths(dev):

@@ -47,16 +47,15 @@ class Mapper:
 class Rollout(FP8RolloutMixin):
     def __init__(self, model):
         self.model = model
+        self._engine_initialized = True
 
     def get_underlying_model(self):
         return self.model
 
-    def model_param_map(self, mapper):
-        d = {}
-        for name, m in self.model.named_children():
-            d[f"{name}.weight"] = m.weight
-            d[f"{name}.weight_scale"] = m.weight_scale
-        return d
+
+def recv_view_map(model, mapper):
+    # what cosmos_rollout_prepare_recv builds between the two hooks (rollout_control.py:382-384)
+    return {mapper.rollout_map_local_key_to_hf_key(k): v for k, v in model.state_dict().items()}
 
 
 def test_weight_sync_end_to_end(dev):
@@ -78,7 +77,7 @@ def test_weight_sync_end_to_end(dev):
 
     mapper, rollout = Mapper(), Rollout(model)
     hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
-    view = rollout.post_get_params_for_sync_hook("fp8", mapper, dict(rollout.model_param_map(mapper)), quantized)
+    view = rollout.post_get_params_for_sync_hook("fp8", mapper, recv_view_map(model, mapper), quantized)
     assert "qkv_proj.weight_scale" not in view
     recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
     # first sync: the policy sends the very weights the engine was loaded with -> self check passes
@@ -109,7 +108,7 @@ def test_fused_receive_quantises_row_shards_in_place(dev):
         m.quant_method.process_weights_after_loading(m)
     mapper, rollout = Mapper(), Rollout(model)
     hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
-    rollout.post_get_params_for_sync_hook("fp8", mapper, dict(rollout.model_param_map(mapper)), quantized)
+    rollout.post_get_params_for_sync_hook("fp8", mapper, recv_view_map(model, mapper), quantized)
     recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
     g = torch.Generator().manual_seed(11)
     w32 = torch.randn(4608, 3584, generator=g) * 0.03                       # transfer dtype fp32
@@ -126,6 +125,36 @@ def test_fused_receive_quantises_row_shards_in_place(dev):
     assert recv.quantize_received_rows("not_quantised.weight", w32[:8].to(dev)) is False
     with pytest.raises(ValueError, match="do not fit"):
         recv.quantize_received_rows("qkv_proj.weight", w32[:64].to(dev), row_start=4600)
+
+
+def test_flush_completions_quantises_a_batch_in_place(dev):
+    """The completions of a flush group run together: both weights go from their staging parameters into the
+    engine's fp8 parameters and weight_scale tensors through the table-driven quantiser; same bytes as one
+    quantize_full_weight per group, and the first-sync check still takes the per-weight path."""
+    model = Model(dev)
+    mp.simplify_process_weights_after_loading()
+    for m in model.children():
+        m.quant_method.process_weights_after_loading(m)
+    mapper, rollout = Mapper(), Rollout(model)
+    hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
+    rollout.post_get_params_for_sync_hook("fp8", mapper, recv_view_map(model, mapper), quantized)
+    recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
+    w_qkv = O.make_weight((4608, 3584), seed=21, std=0.03)
+    w_down = O.make_weight((3584, 2048), seed=22, std=0.01)
+    hp["qkv_proj.weight"].data.copy_(w_qkv.to(dev))
+    hp["down_proj.weight"].data.copy_(w_down.to(dev))
+    groups = [["q_proj.weight", "k_proj.weight", "v_proj.weight"], ["down_proj.weight"], ["norm.weight"]]
+    assert recv.flush_completions(groups) == ["qkv_proj.weight", "down_proj.weight"]
+    for lin, w in ((model.qkv_proj, w_qkv), (model.down_proj, w_down)):
+        qo, so = O.quant_rowwise(w)
+        assert torch.equal(lin.weight.t().contiguous().view(torch.uint8).cpu(), qo)
+        assert torch.equal(lin.weight_scale.cpu().view(torch.int32), so.view(torch.int32))
+        assert lin.weight.stride() == (1, w.shape[1])
+    # the engine now holds these weights: the first-sync check passes, and fails once the policy's differ
+    assert recv.flush_completions(groups, do_weight_sync_check=True) == ["qkv_proj.weight", "down_proj.weight"]
+    hp["down_proj.weight"].data.mul_(2.0).add_(0.01)
+    with pytest.raises(ValueError, match="FP8 weight doesn't match"):
+        recv.flush_completions(groups, do_weight_sync_check=True)
 
 
 def test_fp8_quantization_layout(dev):
@@ -223,3 +252,30 @@ def test_ds_group_gemm_strategy(dev):
     # can amplify to one e4m3 step on isolated entries: compare in Frobenius norm
     assert O.rel_frobenius(out[valid].float(), ref[valid].float()) <= 5e-3
     assert bool((out[~valid] == 0).all())               # zero tokens in, zeros out
+
+    # a buffer with more rows than the groups fill (a capacity bound): nothing is read back from the device, the
+    # rows of the groups equal the exact-size call and the rows past the last group keep what they held
+    cap = torch.full((tok.numel() + 256, H), 7.0, dtype=torch.bfloat16, device=dev)
+    cap[:tok.numel()] = xs.to(dev)
+    for kw in ({}, {"fuse_gate_up": True}, {"fuse_swiglu": False}):
+        want = group_gemms.DSGroupGEMM(act, **kw).execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod)
+        got = group_gemms.DSGroupGEMM(act, **kw).execute(cap.clone(), m_sizes.to(dev), m_offsets.to(dev), mod)
+        assert torch.equal(got[:tok.numel()], want) and bool((got[tok.numel():] == 7.0).all())
+    # a row count that is no multiple of 128 takes the reference's route (slice by m_offsets[-1])
+    odd = torch.cat([xs.to(dev), torch.full((40, H), 7.0, dtype=torch.bfloat16, device=dev)])
+    got = strat.execute(odd, m_sizes.to(dev), m_offsets.to(dev), mod)
+    assert torch.equal(got[:tok.numel()].cpu(), out) and bool((got[tok.numel():] == 7.0).all())
+
+    # the fused copies of the gate / up weights follow in-place updates of the parameters they were built from
+    for kw in ({"fuse_gate_up": True}, {"fuse_gate_up": True, "fuse_epilogue": False}):
+        st2 = group_gemms.DSGroupGEMM(act, **kw)
+        before = st2.execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod)
+        saved = mod.gate_proj_fp8.detach().clone()
+        with torch.no_grad():
+            mod.gate_proj_fp8.copy_(mod.up_proj_fp8)                       # same storage, new contents
+        after = st2.execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod)
+        fresh = group_gemms.DSGroupGEMM(act).execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod)
+        assert not torch.equal(after, before) and torch.equal(after, fresh)
+        mod.gate_proj_fp8.data.copy_(saved)                                # a write that no version counter sees ...
+        st2.invalidate_fused_weights(mod)                                  # ... is announced by the writer
+        assert torch.equal(st2.execute(xs.to(dev).clone(), m_sizes.to(dev), m_offsets.to(dev), mod), before)

@@ -48,9 +48,11 @@ def test_rowwise_cfg1(dev):
     assert_bytes(q, qo, "cfg1 bytes")
 
 
-@pytest.mark.parametrize("cols", [8, 64, 136, 512, 896, 1024, 2048, 3584, 4096, 4104, 8192, 18944, 32768, 32776, 40000])
+@pytest.mark.parametrize("cols", [8, 64, 136, 512, 896, 1024, 2048, 3584, 4096, 4104, 8192, 10248, 12288, 12296, 16384,
+                                  18944, 20480, 20488, 24576, 24584, 32768, 32776, 40000])
 def test_rowwise_widths(dev, cols):
-    """Every kernel variant: wave-per-row (V=1,2,4,8), block-per-row (V=4,8,16), streaming."""
+    """Every kernel variant: wave-per-row (V=1,2,4,8), block-per-row (V=4,5,6,8,10,12,16) on both sides of each
+    limit, streaming."""
     rows = 37 if cols < 20000 else 5
     g = torch.Generator().manual_seed(cols)
     w = (torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g) * 3)).to(torch.bfloat16)
@@ -194,6 +196,53 @@ def test_rowwise_from_into_engine_parameter(dev):
         ops.quant_rowwise_into(w.to(dev), param[:, a:b + 1], scale[a:b])
     with pytest.raises(ValueError):
         ops.quant_rowwise_into(w.to(dev).to(torch.float64), param[:, a:b], scale[a:b])
+
+
+def test_rowwise_multi_matches_single_calls_and_oracle(dev):
+    """cfp8_quant_rowwise_multi: a batch that mixes every kernel variant (row lengths 8 .. 40000), the three source
+    dtypes, empty tensors and more tensors of one class than a launch table holds - bytes and scales equal the
+    oracle's and those of one call per tensor."""
+    spec = [(37, 8, torch.bfloat16), (21, 136, torch.float32), (64, 896, torch.bfloat16), (33, 3584, torch.bfloat16),
+            (5, 3584, torch.float16), (12, 4104, torch.bfloat16), (9, 18944, torch.bfloat16), (3, 40000, torch.bfloat16),
+            (0, 64, torch.bfloat16), (7, 18944, torch.float32), (16, 1288, torch.bfloat16), (4, 2056, torch.bfloat16),
+            (6, 2568, torch.bfloat16), (2, 3080, torch.bfloat16)]
+    spec += [(4 + i % 7, 3584, torch.bfloat16) for i in range(45)]        # one class, more than one table
+    ws = [_recv(r, c, dt, seed=1000 + i) for i, (r, c, dt) in enumerate(spec)]
+    gs = [w.to(dev) for w in ws]
+    qs = [torch.full(w.shape, 0x55, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn) for w in ws]
+    ss = [torch.full((w.shape[0], 1), -1.0, dtype=torch.float32, device=dev) for w in ws]
+    ops.quant_rowwise_multi_into(gs, qs, ss)
+    for i, w in enumerate(ws):
+        if w.shape[0] == 0:
+            continue
+        qo, so = O.quant_rowwise_from(w)
+        assert_scales(ss[i], so, f"tensor {i} {tuple(w.shape)} {w.dtype} scales")
+        assert_bytes(qs[i], qo, f"tensor {i} {tuple(w.shape)} {w.dtype} bytes")
+        q1 = torch.empty_like(qs[i]); s1 = torch.empty_like(ss[i])
+        ops.quant_rowwise_into(gs[i], q1, s1)
+        assert torch.equal(q1.view(torch.uint8), qs[i].view(torch.uint8)) and torch.equal(bits(s1), bits(ss[i]))
+    q2, s2 = ops.quant_rowwise_multi(gs[:4])
+    assert all(torch.equal(a.view(torch.uint8), b.view(torch.uint8)) for a, b in zip(q2, qs[:4]))
+    assert tuple(s2[0].shape) == (37, 1)
+
+
+def test_rowwise_multi_into_engine_parameters(dev):
+    """Destinations are the engine's transposed fp8 parameters (strides (1, in_dim)), one of them a row range."""
+    shapes = [(96, 264), (64, 264), (48, 1024)]
+    ws = [_recv(r, c, torch.bfloat16, seed=50 + i) for i, (r, c) in enumerate(shapes)]
+    bufs = [torch.full((r + 8, c), 0x55, dtype=torch.uint8, device=dev) for r, c in shapes]
+    params = [b.view(torch.float8_e4m3fn).t()[:, 4:4 + r] for b, (r, c) in zip(bufs, shapes)]
+    scales = [torch.empty(r, 1, dtype=torch.float32, device=dev) for r, _ in shapes]
+    ops.quant_rowwise_multi_into([w.to(dev) for w in ws], params, scales)
+    for w, b, sc in zip(ws, bufs, scales):
+        qo, so = O.quant_rowwise(w)
+        assert_bytes(b[4:4 + w.shape[0]], qo, "rows in range")
+        assert_scales(sc, so, "scales")
+        assert (b[:4] == 0x55).all() and (b[4 + w.shape[0]:] == 0x55).all()
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_multi_into([ws[0].to(dev)], params[:1], [scales[0][:5]])
+    with pytest.raises(ValueError):
+        ops.quant_rowwise_multi_into([ws[0].to(dev)], params[:1], scales[:2])
 
 
 # ---------------------------------------------------------------------------- tensorwise

@@ -83,6 +83,7 @@ def test_process_weights_after_loading_and_patches(stub_quant):
     assert isinstance(lin.quant_method.fp8_linear, mp.Fp8LinearOp)
     assert lin.quant_method.fp8_linear.use_per_token_if_dynamic and not lin.quant_method.fp8_linear.cutlass_fp8_supported
     assert mp._dispatch["dispatch_w8a8_scaled_mm"]() is mp.torch_per_token_w8a8_scaled_mm
+    assert lin.quant_method.fp8_linear.w8a8_scaled_mm is mp.torch_per_token_w8a8_scaled_mm   # the op reads the dispatch
     with pytest.raises(NotImplementedError):
         mp.Fp8LinearOp(use_per_token_if_dynamic=False)
 
@@ -110,18 +111,33 @@ def test_cache_replace_and_view_map(stub_quant):
 class ToyRollout(vllm_rollout.FP8RolloutMixin):
     def __init__(self, model):
         self.model = model
+        self._engine_initialized = True
 
     def get_underlying_model(self):
         return self.model
 
-    def model_param_map(self, weight_mapper):
-        out = {}
-        for name, mod in self.model.named_modules():
-            if hasattr(mod, "weight") and isinstance(mod.weight, torch.Tensor):
-                out[weight_mapper.rollout_map_local_key_to_hf_key(name + ".weight")] = mod.weight
-            if hasattr(mod, "weight_scale"):
-                out[weight_mapper.rollout_map_local_key_to_hf_key(name + ".weight_scale")] = mod.weight_scale
-        return out
+
+def test_model_param_map_and_quantized_tensors(stub_quant):
+    """rollout_base.py:186-230: refuses before the engine is up, maps every state-dict entry to its HF name,
+    caches the map."""
+    model = ToyModel()
+    load_fp8(model)
+    mapper = Mapper()
+    rollout = ToyRollout(model)
+    rollout._engine_initialized = False
+    assert rollout.is_engine_initialized() is False
+    with pytest.raises(RuntimeError, match="Engine is not initialized, please call init_engine first"):
+        rollout.model_param_map(mapper)
+    with pytest.raises(RuntimeError, match="Engine is not initialized, please call init_engine first"):
+        rollout.get_quantized_tensors(mapper)
+    rollout._engine_initialized = True
+    assert rollout.get_quantized_tensors(mapper) == {}
+    pm = rollout.model_param_map(mapper)
+    assert set(pm) == {"model.qkv_proj.weight", "model.qkv_proj.weight_scale", "model.o_proj.weight",
+                       "model.o_proj.weight_scale", "model.norm.weight", "model.other.weight"}
+    assert pm["model.qkv_proj.weight"].data_ptr() == model.qkv_proj.weight.data_ptr()
+    assert pm["model.qkv_proj.weight"].stride() == (1, 32)
+    assert rollout.model_param_map(mapper) is pm                       # cached
 
 
 def test_sync_hooks_and_quantize_on_receive(stub_quant):
@@ -134,7 +150,9 @@ def test_sync_hooks_and_quantize_on_receive(stub_quant):
     rollout = ToyRollout(model)
     hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
     assert model.qkv_proj.weight is hp["model.qkv_proj.weight"]       # engine exposes hp buffers to the recv planner
-    view_map = {k: v for k, v in rollout.model_param_map(mapper).items()}
+    # (the recv view map is built from the model between the two hooks, as cosmos_rollout_prepare_recv does at
+    # rollout_control.py:382-384; model_param_map is first asked for by a completion, after the second hook)
+    view_map = {mapper.rollout_map_local_key_to_hf_key(k): v for k, v in model.state_dict().items()}
     view_map = rollout.post_get_params_for_sync_hook("fp8", mapper, view_map, quantized)
     assert not any("weight_scale" in k for k in view_map)
     assert model.qkv_proj.weight is quantized["model.qkv_proj.weight"]  # engine computes in fp8 again
@@ -167,10 +185,50 @@ def test_sync_hooks_and_quantize_on_receive(stub_quant):
     assert recv.check_inside_group(["model.norm.weight"], True) is True
     # scale shape assert (rollout_control.py:895)
     model.o_proj.weight_scale = nn.Parameter(torch.zeros(32), requires_grad=False)
+    rollout._model_param_map = None                                    # the map is cached: rebuild it for the new parameter
     with pytest.raises(AssertionError, match="scale_tensor.shape"):
         recv.quantize_full_weight("model.o_proj.weight")
     with pytest.raises(NotImplementedError):
         QuantizedWeightReceiver(rollout, mapper, hp, quantized, "mxfp4")
+
+
+def test_flush_completions_batches_the_groups(stub_quant, monkeypatch):
+    """rollout_control.py:1308-1319: the completions of a flush group run together - here as one table-driven
+    quantiser call over the quantised weights of the batch, written into the engine's own parameters."""
+    torch.manual_seed(4)
+    model = ToyModel()
+    load_fp8(model)
+    mapper, rollout = Mapper(), ToyRollout(model)
+    hp, quantized = rollout.pre_get_params_for_sync_hook("fp8", mapper, None)
+    view_map = {mapper.rollout_map_local_key_to_hf_key(k): v for k, v in model.state_dict().items()}
+    rollout.post_get_params_for_sync_hook("fp8", mapper, view_map, quantized)
+    recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
+    batches = []
+
+    def fake_multi(weights, q_outs, scale_outs):
+        batches.append([tuple(w.shape) for w in weights])
+        for w, q, sc in zip(weights, q_outs, scale_outs):
+            qo, so = O.quant_rowwise(w)
+            assert tuple(q.shape) == (w.shape[1], w.shape[0]) and q.stride() == (1, w.shape[1])   # the engine's layout
+            q.copy_(qo.view(torch.float8_e4m3fn).t())
+            sc.copy_(so)
+
+    monkeypatch.setattr(ops, "quant_rowwise_multi_into", fake_multi)
+    new_qkv = (torch.randn(48, 32) * 0.05).to(torch.bfloat16)
+    new_o = (torch.randn(32, 32) * 0.02).to(torch.bfloat16)
+    hp["model.qkv_proj.weight"].data.copy_(new_qkv)
+    hp["model.o_proj.weight"].data.copy_(new_o)
+    groups = [["model.q_proj.weight", "model.k_proj.weight", "model.v_proj.weight"], ["model.o_proj.weight"],
+              ["model.norm.weight"], ["model.o_proj.weight"]]
+    assert recv.flush_completions(groups) == ["model.qkv_proj.weight", "model.o_proj.weight"]
+    assert batches == [[(48, 32), (32, 32)]] and stub_quant == []       # one batch, no per-weight call
+    for lin, w in ((model.qkv_proj, new_qkv), (model.o_proj, new_o)):
+        qo, so = O.quant_rowwise(w)
+        assert torch.equal(lin.weight.t().contiguous().view(torch.uint8), qo) and torch.equal(lin.weight_scale, so)
+    # with the first-sync check every weight takes the per-weight path (the check compares old and new bytes)
+    assert recv.flush_completions(groups, do_weight_sync_check=True) == ["model.qkv_proj.weight", "model.o_proj.weight"]
+    assert stub_quant == [(48, 32), (32, 32)] and len(batches) == 1
+    assert QuantizedWeightReceiver(rollout, mapper, hp, quantized, None).flush_completions(groups) == []
 
 
 def test_fp8_quantization_returns_transposed_view(stub_quant):
@@ -186,9 +244,12 @@ def test_recipes_filter_and_converter(monkeypatch):
     assert not fp8_util.is_valid_fp8_quant_recipe("blockwise")
     assert fp8_util.FP8QuantRecipe.ROWWISE == "rowwise" and str(fp8_util.FP8Recipe.DYNAMIC_SCALING) == "dynamic_scaling"
     f = fp8_util.module_filter_fn
-    assert f(nn.Linear(32, 64), "model.layers.0.mlp.up_proj", ["lm_head"])
-    assert not f(nn.Linear(32, 64), "lm_head", ["lm_head"])
-    assert not f(nn.Linear(24, 64), "x", []) and not f(nn.Linear(32, 40), "x", [])
+    assert f(nn.Linear(128, 64), "model.layers.0.mlp.up_proj", ["lm_head"])
+    assert not f(nn.Linear(128, 64), "lm_head", ["lm_head"])
+    assert not f(nn.Linear(120, 64), "x", []) and not f(nn.Linear(128, 40), "x", [])
+    # multiples of 16 that the FP8 GEMM cannot take (K must be a multiple of 128) stay nn.Linear instead of
+    # converting and then failing in their first forward
+    assert not f(nn.Linear(80, 64), "x", []) and not f(nn.Linear(1200, 64), "x", []) and f(nn.Linear(1280, 48), "x", [])
     assert not f(nn.LayerNorm(32), "x", [])
 
     def cfg(**kw):
@@ -207,8 +268,8 @@ def test_recipes_filter_and_converter(monkeypatch):
     class Net(nn.Module):
         def __init__(self):
             super().__init__()
-            self.body = nn.Sequential(nn.Linear(32, 64), nn.ReLU(), nn.Linear(64, 24))
-            self.lm_head = nn.Linear(32, 128)
+            self.body = nn.Sequential(nn.Linear(128, 256), nn.ReLU(), nn.Linear(256, 24), nn.Linear(80, 64))
+            self.lm_head = nn.Linear(128, 128)
 
         def fqn_filter_for_quantization(self):
             return ["lm_head"]
@@ -222,10 +283,11 @@ def test_recipes_filter_and_converter(monkeypatch):
     assert isinstance(net.body[0], fp8_util.Float8Linear) and net.body[0].quant_recipe == "tensorwise"
     assert net.body[0].weight is w_before
     assert type(net.body[2]) is nn.Linear            # 24 is not a multiple of 16
+    assert type(net.body[3]) is nn.Linear            # in_features 80: a multiple of 16 but not of the GEMM's K step
     assert type(net.lm_head) is nn.Linear            # filtered by FQN
     assert conv.post_optimizer_hook(net) is None
     with pytest.raises(NotImplementedError):         # forward direction only
-        net.body[0](torch.randn(2, 32, requires_grad=True))
+        net.body[0](torch.randn(2, 128, requires_grad=True))
 
 
 def test_group_gemm_strategies_on_cpu():
@@ -261,3 +323,6 @@ def test_create_indices_from_offsets():
     assert idx.dtype == torch.int32 and idx.numel() == 384
     assert bool((idx[:128] == 0).all()) and bool((idx[128:] == 2).all())
     assert torch.equal(idx, ops.create_indices_from_offsets_nosync(offs))
+    # a row bound instead of the exact count: rows past the last group are padding (-1), nothing is read back
+    cap = ops.create_indices_from_offsets_nosync(offs, 640, n_experts=3)
+    assert torch.equal(cap[:384], idx) and bool((cap[384:] == -1).all())
