@@ -203,6 +203,7 @@ def test_flush_completions_batches_the_groups(stub_quant, monkeypatch):
     view_map = {mapper.rollout_map_local_key_to_hf_key(k): v for k, v in model.state_dict().items()}
     rollout.post_get_params_for_sync_hook("fp8", mapper, view_map, quantized)
     recv = QuantizedWeightReceiver(rollout, mapper, hp, quantized, "fp8")
+    stub_quant.clear()
     batches = []
 
     def fake_multi(weights, q_outs, scale_outs):
