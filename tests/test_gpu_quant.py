@@ -435,6 +435,27 @@ def test_swiglu_quant_bit_exact(dev, M, I):
     assert_bytes(q, qo, f"swiglu {M}x{I} bytes")
 
 
+def test_swiglu_every_gate_pattern(dev):
+    """All 65536 bf16 gate patterns, one 1x128 group each (the whole group holds the pattern, up = 1 except one
+    element of 0.5): the group's scale is |bf16(silu(g))| / 448, which is injective in that bf16 value, and the
+    bytes carry its sign - so equal scales and bytes mean the kernel's SiLU equals the defining fp32 sequence
+    of the C restatement after rounding to bf16 for every input, including those that take the hardware
+    exponential / reciprocal path."""
+    import numpy as np
+    from oracle import c_oracle as C
+    gate = all_bf16_patterns().reshape(65536, 1).expand(65536, 128).contiguous()
+    up = torch.ones(65536, 128, dtype=torch.bfloat16)
+    up[:, 5] = 0.5
+    q, s = ops.swiglu_quant(gate.to(dev), up.to(dev))
+    qo, so = C.swiglu_quant_group128(_np16(gate), _np16(up))
+    qo, so = torch.from_numpy(qo), torch.from_numpy(so)
+    nan = torch.isnan(so).reshape(-1)
+    assert int(nan.sum()) < 600                                         # NaN patterns and -inf
+    assert_scales(s.cpu().reshape(-1)[~nan], so.reshape(-1)[~nan], "silu of every bf16 pattern: scales")
+    assert bool(torch.isnan(s.cpu().reshape(-1)[nan]).all())
+    assert_bytes(q, qo, "silu of every bf16 pattern: bytes")
+
+
 def test_swiglu_quant_fused_gate_up_layout_and_torch_semantics(dev):
     """gate and up as the two column halves of one [M, 2I] GEMM output (row pitch 2I), and the result
     against torch's own silu(g) * u followed by the 1x128 quantiser: dequantised values within fp8
