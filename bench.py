@@ -9,9 +9,14 @@ already resident in HBM).  One step = one `cfp8_quant_tensorwise_multi` call ove
 `value` = algorithmic bytes of the two-pass algorithm (5 B/element: 2 read by the amax pass,
 2 read + 1 written by the cast pass) per second over the timed steps.
 `roofline` is for the dominant kernel (the cast pass, 3 B/element), timed per launch with
-events on the launch stream.  `extra` carries the other kernels of the path (rowwise / block /
-group quantisers in GB/s, the FP8 GEMMs in TFLOP/s).  `cpu_baseline` times the torch CPU oracle
-on one tensor of each distinct shape and scales by multiplicity.
+events on the launch stream.  The GEMM half of the metric has rooflines of its own at the top level
+(`roofline_gemm` = config 3 at 8192 tokens, `roofline_gemm_cfg4`, `roofline_gemm_cfg5`, against the
+5.0 PFLOP/s dense FP8 peak; `roofline_decode` = config 3 at 1 and 64 tokens against HBM, with a plain
+copy of the same bytes beside them; `roofline_rowwise_sync` = the rowwise quantisation of one full
+weight sync as the table-driven launch).  `extra` carries every other kernel of the path.
+`cpu_baseline` times the torch CPU oracle on one tensor of each distinct shape of the headline workload
+and scales by multiplicity; `cpu_baseline_cfg1/3/4/5` time the CPU path of the other configs (config 1 in
+full, config 3 at every M, configs 4 and 5 once), medians of >= 5 runs after one warm-up where stated.
 
 Prints ONE JSON line.
 """
@@ -140,6 +145,8 @@ def main() -> int:
         "unit": "GB/s",
         "frac": round(cast_bytes / (cast_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "traffic": CAST_TRAFFIC_BYTES_PER_LAUNCH if (n == 197 and launches == 5) else None,
+        "traffic_source": "profiles/tensorwise_qwen25_7b_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
+                          "command, calibrated on a 1 GiB copy; a constant of that profile, not measured in this run)",
         "bytes_per_launch": cast_bytes // launches,
         "launches_per_step": launches,
         "avg_launch_ms": round(cast_med / launches, 4),
@@ -164,9 +171,12 @@ def main() -> int:
     torch.cuda.empty_cache()
 
     cpu = None
+    cpu_other = {}
     if not args.no_cpu:
         cpu = cpu_baseline(torch)
+        cpu_other = cpu_baseline_other_configs(torch)
 
+    top = summarise_top_level(extra)
     line = {
         "metric": "weight-quant HBM GB/s + fp8 scaled-GEMM TFLOP/s, Qwen2.5-7B shapes, 1 GPU",
         "value": round(value, 1),
@@ -180,7 +190,9 @@ def main() -> int:
                    "elements": numel, "tensors": n,
                    "single_read_lower_bound_GBps": round((3 * numel) / (ms_per_step * 1e-3) / 1e9, 1)},
         "roofline": roofline,
+        **top,
         "cpu_baseline": cpu,
+        **cpu_other,
         "extra": extra,
     }
     print(json.dumps(line))
@@ -188,6 +200,71 @@ def main() -> int:
 
 
 WARM_SECONDS = 0.15
+
+
+def summarise_top_level(extra):
+    """Flat top-level records for the GEMM half of the metric and the other graded lines, taken from `extra`."""
+    top = {}
+
+    def gemm(key, name, kernel, workload, also=None):
+        e = extra.get(name)
+        if not e or "ms" not in e:
+            return
+        rec = {"kernel": kernel, "workload": workload, "bound": "mfma", "flops": e.get("flops"), "median_ms": e["ms"],
+               "achieved": e["TFLOP/s"], "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": e["frac_mfma"]}
+        for k, nm in (also or {}).items():
+            if nm in extra and "ms" in extra[nm]:
+                rec[k + "_ms"] = extra[nm]["ms"]
+                rec[k + "_frac"] = extra[nm]["frac_mfma"]
+        top[key] = rec
+
+    gemm("roofline_gemm", "linear_rowwise_cfg3_M8192", "gemm_rowwise_256p_kernel (+ per-token quantiser, + tail launch)",
+         "configs[2] M=8192: bf16 [8192,3584] quantised per token in the call, x fp8 [18944,3584]^T -> bf16",
+         {"gemm_only": "scaled_mm_rowwise_cfg3_M8192_gemm_only", "M1024": "linear_rowwise_cfg3_M1024",
+          "vendor_scaled_mm": "vendor_torch_scaled_mm_rowwise_cfg3_M8192",
+          "qkv_M2048": "linear_rowwise_qkv_4608x3584_M2048", "o_M2048": "linear_rowwise_o_3584x3584_M2048",
+          "gate_up_M2048": "linear_rowwise_gate_up_37888x3584_M2048", "down_M2048": "linear_rowwise_down_3584x18944_M2048"})
+    gemm("roofline_gemm_cfg4", "gemm_block128_cfg4_4096x18432x7168_incl_act_quant", "gemm_block_w8_kernel<256,128> (+ 1x128 quantiser)",
+         "configs[3]: [4096,7168] x [7168,18432], 128x128 weight blocks, 1x128 activation groups",
+         {"short_k_1536": "gemm_block128_short_k_4096x24576x1536_gemm_only"})
+    gemm("roofline_gemm_cfg5", "grouped_cfg5_mlp_quant_gateup_swiglu_down", "gemm_block_w8p_kernel<128,256,grouped,SwiGLU> + gemm_block_w8_kernel<128,256,grouped>",
+         "configs[4]: 128 experts, 8192 tokens top-8: 1x128 quant, gate_up GEMM + SwiGLU + requant, down GEMM",
+         {"swiglu_separate": "grouped_cfg5_mlp_swiglu_as_separate_launch"})
+    dec = {}
+    for M in (1, 64):
+        e = extra.get(f"linear_rowwise_cfg3_M{M}")
+        if e and "ms" in e:
+            dec[f"M{M}_ms"], dec[f"M{M}_GBps"], dec[f"M{M}_frac_hbm"] = e["ms"], e["GB/s"], e["frac_hbm"]
+    c = extra.get("plain_copy_same_bytes_as_cfg3_weight")
+    if c:
+        dec["copy_same_bytes_ms"], dec["copy_GBps"], dec["copy_frac_hbm"] = c["ms"], c["GB/s"], c["frac_hbm"]
+    if dec:
+        dec.update({"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "workload": "configs[2] M=1 and M=64: the 68 MB fp8 weight streamed once; beside them a plain device copy moving the same 68 MB"})
+        top["roofline_decode"] = dec
+    r = extra.get("rowwise_multi_qwen25_7b_sync_112_weights")
+    if r:
+        top["roofline_rowwise_sync"] = {"kernel": "rowwise_wave_multi_kernel<8> + rowwise_block_multi_kernel<10>", "bound": "hbm",
+                                        "workload": "rowwise quantisation of the 112 packed linear weights of one Qwen2.5-7B sync (28 x qkv, o, gate_up, down) as one table-driven call",
+                                        "median_ms": r["ms"], "achieved": r["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": r["frac_hbm"],
+                                        "one_launch_per_weight_ms": extra.get("rowwise_single_calls_qwen25_7b_sync_112_weights", {}).get("ms")}
+    # the quantisers that are short enough for the ramp-up of a launch to matter, each with the fraction a plain
+    # device copy of the same number of bytes reaches (`*_copy`): the ceiling for a kernel of that size on this GPU
+    q = {}
+    for k, nm, exact in (("rowwise_cfg1", "rowwise_cfg1_4864x896", True), ("rowwise_qkv", "rowwise_qkv_4608x3584", True),
+                         ("rowwise_down", "rowwise_down_3584x18944", True), ("block128", "block128_cfg4_7168x18432", True),
+                         ("block128_T", "block128_cfg4_7168x18432_T", True), ("group128", "group128_cfg4_4096x7168", True),
+                         ("swiglu_quant", "swiglu_quant_cfg5", False), ("gather_quant", "gather_quant_cfg5", False)):
+        for name, e in extra.items():
+            if (name == nm if exact else name.startswith(nm)) and "frac_hbm" in e:
+                q[k] = e["frac_hbm"]
+                if "copy_frac_hbm" in e:
+                    q[k + "_copy"] = e["copy_frac_hbm"]
+                break
+    if q:
+        q["unit"] = "fraction of 8 TB/s (algorithmic bytes / median time); *_copy = torch device copy moving the same bytes"
+        top["quantiser_fracs"] = q
+    return top
 
 
 def _time_events(torch, fn, warmup, iters, flush=None):
@@ -222,12 +299,21 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     flush = torch.zeros(128 * 1024 * 1024, dtype=torch.float32, device=dev)
     out = {}
 
-    def hbm(name, bytes_, fn, iters=50):
+    def hbm(name, bytes_, fn, iters=50, copy_ceiling=False):
         if only and only not in name:
             return
         med, mn = _time_events(torch, fn, 10, iters, flush)
         out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "GB/s": round(bytes_ / (med * 1e-3) / 1e9, 1),
                      "frac_hbm": round(bytes_ / (med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        if copy_ceiling:
+            # a plain device copy that moves the same number of bytes (half in, half out), same flush and warm-up
+            half = (int(bytes_) // 2 + 255) & ~255
+            src = torch.empty(half, dtype=torch.uint8, device=dev).fill_(1)
+            dst = torch.empty_like(src)
+            cmed, _ = _time_events(torch, lambda: dst.copy_(src), 10, iters, flush)
+            out[name]["copy_ms"] = round(cmed, 4)
+            out[name]["copy_frac_hbm"] = round(2 * half / (cmed * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+            del src, dst
 
     def mfma(name, flops, bytes_, fn, iters=50, cold=True):
         if only and only not in name:
@@ -236,7 +322,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         tf = flops / (med * 1e-3) / 1e12
         gbs = bytes_ / (med * 1e-3) / 1e9
         bound = "mfma" if flops / bytes_ > FP8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9) else "hbm"
-        out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
+        out[name] = {"ms": round(med, 4), "min_ms": round(mn, 4), "flops": flops, "TFLOP/s": round(tf, 1), "GB/s": round(gbs, 1), "bound": bound,
                      "frac": round(tf / FP8_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS, 4),
                      "frac_mfma": round(tf / FP8_PEAK_TFLOPS, 4), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)}
 
@@ -248,8 +334,29 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         q = torch.empty(r, c, dtype=torch.float8_e4m3fn, device=dev)
         s = torch.empty(r, 1, dtype=torch.float32, device=dev)
         hbm(nm, 3 * r * c + 4 * r,
-            lambda: check(lib.cfp8_quant_rowwise(x.data_ptr(), r, c, c, q.data_ptr(), c, s.data_ptr(), stream)))
+            lambda: check(lib.cfp8_quant_rowwise(x.data_ptr(), r, c, c, q.data_ptr(), c, s.data_ptr(), stream)), copy_ceiling=r * c < 3e8)
         del x, q, s
+
+    # the rowwise quantisation of one whole Qwen2.5-7B weight sync (vLLM's packed layers x 28): one table-driven call
+    # against one launch per weight
+    if not only or "rowwise_multi" in only or "rowwise_single" in only:
+        ws = [torch.empty(r, c, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
+              for _ in range(28) for (r, c) in ((4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944))]
+        qs = [torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=dev) for w in ws]
+        ss = [torch.empty(w.shape[0], 1, dtype=torch.float32, device=dev) for w in ws]
+        nd = len(ws)
+        rd = (_lib.RowwiseDesc * nd)()
+        for i, (w, q, sc) in enumerate(zip(ws, qs, ss)):
+            rd[i].x, rd[i].q, rd[i].scales = w.data_ptr(), q.data_ptr(), sc.data_ptr()
+            rd[i].rows, rd[i].cols, rd[i].ld_x, rd[i].ld_q, rd[i].x_dtype = w.shape[0], w.shape[1], w.shape[1], w.shape[1], 0
+        sync_bytes = sum(3 * w.numel() + 4 * w.shape[0] for w in ws)
+        hbm("rowwise_multi_qwen25_7b_sync_112_weights", sync_bytes, lambda: check(lib.cfp8_quant_rowwise_multi(rd, nd, stream)), iters=10)
+
+        def singles():
+            for w, q, sc in zip(ws, qs, ss):
+                check(lib.cfp8_quant_rowwise(w.data_ptr(), w.shape[0], w.shape[1], w.shape[1], q.data_ptr(), w.shape[1], sc.data_ptr(), stream))
+        hbm("rowwise_single_calls_qwen25_7b_sync_112_weights", sync_bytes, singles, iters=10)
+        del ws, qs, ss, rd
 
     # quantise-on-receive straight from an fp32 transfer buffer (cast + quantise + store in one kernel)
     r, c = 37888, 3584
@@ -266,10 +373,10 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     q4 = torch.empty(N4, K4, dtype=torch.float8_e4m3fn, device=dev)
     s4 = torch.empty(K4 // 128, N4 // 128, dtype=torch.float32, device=dev)
     hbm("block128_cfg4_7168x18432_T", 3 * K4 * N4 + 4 * s4.numel(),
-        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4.data_ptr(), s4.data_ptr(), 1, stream)))
+        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4.data_ptr(), s4.data_ptr(), 1, stream)), copy_ceiling=True)
     q4n = torch.empty(K4, N4, dtype=torch.float8_e4m3fn, device=dev)
     hbm("block128_cfg4_7168x18432", 3 * K4 * N4 + 4 * s4.numel(),
-        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4n.data_ptr(), s4.data_ptr(), 0, stream)))
+        lambda: check(lib.cfp8_quant_block128(w4.data_ptr(), 1, K4, N4, q4n.data_ptr(), s4.data_ptr(), 0, stream)), copy_ceiling=True)
     # the inverse: block dequantisation of the same matrix to bf16 (1 B read, 2 B written per element)
     hbm("dequant_block128_cfg4_7168x18432_bf16", 3 * K4 * N4 + 4 * s4.numel(),
         lambda: check(lib.cfp8_dequant_block128(q4n.data_ptr(), s4.data_ptr(), K4, N4, w4.data_ptr(), 0, stream)))
@@ -278,7 +385,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     qx4 = torch.empty(M4, K4, dtype=torch.float8_e4m3fn, device=dev)
     sx4 = torch.empty(M4, K4 // 128, dtype=torch.float32, device=dev)
     hbm("group128_cfg4_4096x7168", 3 * M4 * K4 + 4 * sx4.numel(),
-        lambda: check(lib.cfp8_quant_group128(x4.data_ptr(), M4, K4, K4, qx4.data_ptr(), K4, sx4.data_ptr(), 0, stream)))
+        lambda: check(lib.cfp8_quant_group128(x4.data_ptr(), M4, K4, K4, qx4.data_ptr(), K4, sx4.data_ptr(), 0, stream)), copy_ceiling=True)
     o4 = torch.empty(M4, N4, dtype=torch.bfloat16, device=dev)
 
     def gemm4():
@@ -304,6 +411,12 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     w3 = torch.empty(N3, K3, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
     qw3, sw3 = ops.quant_rowwise(w3)
     del w3
+    # a plain device copy that moves as many bytes as the decode shapes read (34 MB in, 34 MB out = the 68 MB weight):
+    # what a kernel of that size and duration reaches here, beside the M = 1 and M = 64 lines
+    csrc = torch.empty(N3 * K3 // 2, dtype=torch.uint8, device=dev).fill_(1)
+    cdst = torch.empty_like(csrc)
+    hbm("plain_copy_same_bytes_as_cfg3_weight", N3 * K3, lambda: cdst.copy_(csrc))
+    del csrc, cdst
     for M in (1, 64, 1024, 8192):
         x = torch.randn(M, K3, generator=gen, device=dev)
         chan = torch.rand(K3, generator=gen, device=dev) < 0.005
@@ -426,7 +539,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     moe()
     hbm("swiglu_quant_cfg5_%dx%d" % (total, I), 5 * total * I + 4 * sh.numel(),
         lambda: check(lib.cfp8_swiglu_quant_group128(gu.data_ptr(), 2 * I, gu.data_ptr() + I * 2, 2 * I, total, I,
-                                                     qh.data_ptr(), I, sh.data_ptr(), stream)))
+                                                     qh.data_ptr(), I, sh.data_ptr(), stream)), copy_ceiling=True)
     flops5 = 2.0 * routed * (H * 2 * I + I * H)
     mfma("grouped_cfg5_mlp_quant_gateup_swiglu_down", flops5,
          qgu.numel() + qd.numel() + routed * (H * 2 + I + H * 2), moe_fused, iters=50)
@@ -448,7 +561,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         check(lib.cfp8_gather_rows(tok.data_ptr(), H * 2, src.data_ptr(), total, H * 2, gath.data_ptr(), H * 2, stream))
         check(lib.cfp8_quant_group128(gath.data_ptr(), total, H, H, qxs.data_ptr(), H, sxs.data_ptr(), 0, stream))
     hbm("gather_quant_cfg5_%dx%d" % (total, H), T * H * 2 + total * H + 4 * sxs.numel() + 4 * total,
-        lambda: check(lib.cfp8_gather_quant_group128(tok.data_ptr(), H, src.data_ptr(), total, H, qxs.data_ptr(), H, sxs.data_ptr(), stream)))
+        lambda: check(lib.cfp8_gather_quant_group128(tok.data_ptr(), H, src.data_ptr(), total, H, qxs.data_ptr(), H, sxs.data_ptr(), stream)), copy_ceiling=True)
     hbm("gather_then_quant_cfg5_two_launches", T * H * 2 + total * H + 4 * sxs.numel() + 4 * total, gather_then_quant)
     # weighted combine of the expert rows back into token order (bf16 rounding at every step)
     e_sorted, order = torch.sort(topi, stable=True)
@@ -468,13 +581,36 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     return out
 
 
-def cpu_baseline(torch):
-    """The torch CPU oracle (a port of the reference's torch-op path) on one tensor of each
-    distinct Qwen2.5-7B shape, median of 3, scaled by multiplicity to a full pass."""
-    from oracle import fp8_oracle as O
+def _cpu_info(torch):
+    model = "unknown"
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.lower().startswith("model name"):
+                model = ln.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
+    return {"cores": cores, "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(), "cpu_model": model}
+
+
+def _median_after_warmup(fn, runs=5):
+    fn()                                  # warm-up
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts), min(ts)
+
+
+def cpu_baseline(torch):
+    """The torch CPU oracle (a port of the reference's torch-op path) on one tensor of each
+    distinct Qwen2.5-7B shape, median of 5 after one warm-up, scaled by multiplicity to a full pass."""
+    from oracle import fp8_oracle as O
+    info = _cpu_info(torch)
     shapes = {}
     for _, shp, mult in QWEN25_7B:
         shapes[shp] = shapes.get(shp, 0) + mult
@@ -482,19 +618,84 @@ def cpu_baseline(torch):
     g = torch.Generator().manual_seed(1)
     for shp, mult in shapes.items():
         w = (torch.randn(*shp, generator=g) * 0.02).to(torch.bfloat16)
-        ts = []
-        for _ in range(3 if w.numel() < 2e8 else 2):
-            t0 = time.perf_counter()
-            O.quant_tensorwise(w)
-            ts.append(time.perf_counter() - t0)
-        total_s += statistics.median(ts) * mult
+        med, _ = _median_after_warmup(lambda: O.quant_tensorwise(w), 5)
+        total_s += med * mult
         numel += w.numel() * mult
         del w
     return {"value": round(5 * numel / total_s / 1e9, 2),
-            "unit": "GB/s (same 5 B/element accounting)", "cores": cores, "kind": "port",
+            "unit": "GB/s (same 5 B/element accounting)", "cores": info["cores"], "kind": "port",
             "sample": "torch CPU oracle quant_tensorwise on one tensor of each of the 5 distinct shapes "
-                      "(median of 2-3 runs), scaled by multiplicity to the 197-tensor pass",
-            "estimated_full_pass_s": round(total_s, 2)}
+                      "(median of 5 runs after a warm-up), scaled by multiplicity to the 197-tensor pass",
+            "estimated_full_pass_s": round(total_s, 2), **info}
+
+
+def cpu_baseline_other_configs(torch):
+    """CPU legs of the other configs: the oracle's restatement of the reference's torch path on the host cores.
+    Config 1 in full (rowwise quantisation of [4864, 896]); config 3 at every M (per-token quantisation, then the
+    dequantised fp32 matmul - torch's CPU _scaled_mm has no rowwise form); configs 4 and 5 once each."""
+    from oracle import fp8_oracle as O
+    info = _cpu_info(torch)
+    out = {}
+    # config 1
+    w1 = O.make_weight((4864, 896), seed=1235, outlier_frac=1e-3, outlier_mul=20.0)
+    med, mn = _median_after_warmup(lambda: O.quant_rowwise(w1), 7)
+    b1 = 3 * w1.numel() + 4 * w1.shape[0]
+    out["cpu_baseline_cfg1"] = {"value": round(b1 / med / 1e9, 3), "unit": "GB/s (3 B/element + 4 B/row)", "median_ms": round(med * 1e3, 3),
+                                "min_ms": round(mn * 1e3, 3), "kind": "port", "runs": "median of 7 after 1 warm-up",
+                                "sample": "configs[0] in full: oracle quant_rowwise of bf16 [4864, 896], N(0,0.02) with 0.1% x20 outliers, seed 1235", **info}
+    # config 3
+    N3, K3 = 18944, 3584
+    w3 = O.make_weight((N3, K3), seed=3)
+    qw3, sw3 = O.quant_rowwise(w3)
+    del w3
+    rec = {"unit": "TFLOP/s", "kind": "port", "runs": "median of 5 after 1 warm-up (3 at M=8192)",
+           "sample": "configs[2]: oracle fp8_linear_rowwise = per-token quantisation + dequantisation of both operands + fp32 torch.matmul, "
+                     "weight [18944, 3584] quantised outside the timed region", **info}
+    for M in (1, 64, 1024, 8192):
+        x = O.make_activation(M, K3, seed=30 + M, chan_outlier_frac=0.005, outlier_mul=30.0)
+        med, _ = _median_after_warmup(lambda: O.fp8_linear_rowwise(x, qw3, sw3), 5 if M < 8192 else 3)
+        rec[f"M{M}_ms"] = round(med * 1e3, 2)
+        rec[f"M{M}_TFLOPs"] = round(2.0 * M * N3 * K3 / med / 1e12, 4)
+    rec["value"] = rec["M8192_TFLOPs"]
+    out["cpu_baseline_cfg3"] = rec
+    del qw3, sw3
+    # config 4, once
+    M4, K4, N4 = 4096, 7168, 18432
+    g = torch.Generator().manual_seed(4)
+    x4 = torch.randn(M4, K4, generator=g).to(torch.bfloat16)
+    w4 = (torch.randn(N4, K4, generator=g) * 0.02).to(torch.bfloat16)
+    t0 = time.perf_counter()
+    qw4, s4 = O.quant_block128(w4)
+    tq = time.perf_counter() - t0
+    del w4
+    t0 = time.perf_counter()
+    qx4, sx4 = O.quant_group128(x4)
+    O.scaled_mm_block128(qx4, sx4, qw4, s4)
+    tg = time.perf_counter() - t0
+    out["cpu_baseline_cfg4"] = {"value": round(2.0 * M4 * N4 * K4 / tg / 1e12, 4), "unit": "TFLOP/s", "gemm_incl_act_quant_s": round(tg, 3),
+                                "block_quant_s": round(tq, 3), "block_quant_GBps": round(3 * N4 * K4 / tq / 1e9, 3), "kind": "port", "runs": "once",
+                                "sample": "configs[3]: oracle quant_block128 of the [18432, 7168] weight; quant_group128 + dequantised fp32 matmul at 4096 tokens", **info}
+    del x4, qw4, s4, qx4, sx4
+    # config 5, once: the expert MLP on routed rows
+    E, H, I, T, TOPK = 128, 2048, 768, 8192, 8
+    logits = torch.rand(T, E, generator=g)
+    tok, m_idx, _, _ = O.route_topk_contiguous(logits, TOPK, 128)
+    x5 = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    xs = torch.zeros(tok.numel(), H, dtype=torch.bfloat16)
+    xs[tok >= 0] = x5[tok[tok >= 0]]
+    qgu, sgu = O.quant_block128((torch.randn(E, 2 * I, H, generator=g) * 0.02).to(torch.bfloat16))
+    qd, sd = O.quant_block128((torch.randn(E, H, I, generator=g) * 0.02).to(torch.bfloat16))
+    t0 = time.perf_counter()
+    qx, sx = O.quant_group128(xs)
+    gu = O.grouped_mm_block128(qx, sx, qgu, sgu, m_idx).to(torch.bfloat16)
+    qh, sh = O.swiglu_quant_group128(gu[:, :I], gu[:, I:])
+    O.grouped_mm_block128(qh, sh, qd, sd, m_idx)
+    t5 = time.perf_counter() - t0
+    routed = int((tok >= 0).sum())
+    out["cpu_baseline_cfg5"] = {"value": round(2.0 * routed * (H * 2 * I + I * H) / t5 / 1e12, 4), "unit": "TFLOP/s", "mlp_s": round(t5, 3),
+                                "kind": "port", "runs": "once", "routed_rows": routed,
+                                "sample": "configs[4]: oracle 1x128 quant, grouped gate_up matmul (loop over 128 experts, fp32), silu*up + requant, grouped down matmul", **info}
+    return out
 
 
 if __name__ == "__main__":
