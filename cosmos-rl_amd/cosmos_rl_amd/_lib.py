@@ -64,6 +64,7 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "cfp8_gemm_block128": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_int64,
                                    c_void_p, c_int64, c_int, c_int64, c_int64, c_int64, c_void_p]),
+    "cfp8_gemm_dispatch_info": (c_int, [c_int, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
     "cfp8_gemm_grouped_block128": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p]),
 }
@@ -87,6 +88,17 @@ def load() -> ctypes.CDLL:
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+DISPATCH_ROWWISE, DISPATCH_LINEAR, DISPATCH_BLOCK, DISPATCH_GROUPED, DISPATCH_GROUPED_SWIGLU = range(5)
+
+
+def gemm_dispatch_info(kind: int, M: int, N: int, K: int, out_dtype: int = OUT_BF16, cus: int = 256,
+                       with_split_workspace: bool = False) -> str:
+    """The kernels a GEMM entry point would launch for a problem ("name grid=.. block=.. lds=..; ..."); needs no GPU."""
+    buf = ctypes.create_string_buffer(1024)
+    check(load().cfp8_gemm_dispatch_info(kind, M, N, K, out_dtype, cus, int(with_split_workspace), buf, len(buf)))
+    return buf.value.decode()
 
 
 def last_error() -> str:

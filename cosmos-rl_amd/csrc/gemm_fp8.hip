@@ -23,6 +23,7 @@
 //   block:    every K step is one 128-block; its MFMA result is folded into the
 //             running sum as acc += part * (sa[m, kb] * sb[n / 128, kb]).
 #include <atomic>
+#include <stdio.h>
 #include <type_traits>
 
 #include "cfp8_common.h"
@@ -1397,22 +1398,47 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
 }
 
+// ---------------------------------------------------------------------------
+// Launch record.  cfp8_gemm_dispatch_info walks the very dispatch code below with launching switched off and
+// gets back which kernels a problem would run, with grid, workgroup size and LDS bytes - so a test can pin, on
+// a machine without a GPU, that a shape still takes the kernel form its parity tests cover.
+// ---------------------------------------------------------------------------
+struct LaunchRecord {
+    bool dry = false;   // record only: no HIP call is made
+    int cus = 256;      // compute units assumed while dry
+    char text[768];
+    size_t len = 0;
+};
+static thread_local LaunchRecord g_rec;
+static bool dry_run() { return g_rec.dry; }
+// returns true when the kernel is to be launched for real
+static bool note_launch(const char* kernel, unsigned grid, unsigned block, size_t lds) {
+    if (!g_rec.dry) return true;
+    const int n = snprintf(g_rec.text + g_rec.len, sizeof(g_rec.text) - g_rec.len, "%s%s grid=%u block=%u lds=%zu", g_rec.len ? "; " : "",
+                           kernel, grid, block, lds);
+    if (n > 0) g_rec.len = g_rec.len + (size_t)n < sizeof(g_rec.text) ? g_rec.len + (size_t)n : sizeof(g_rec.text) - 1;
+    return false;
+}
+static int launched(const char* what) { return dry_run() ? CFP8_OK : check_launch(what); }
+
 // Kernels that use more than 64 KiB of LDS need the limit raised once per device and function.
 // `flag` is that (device, function) pair's once-flag; a race on the first call raises it twice, harmlessly.
 static int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag) {
-    if (flag.load(std::memory_order_relaxed)) return CFP8_OK;
+    if (dry_run() || flag.load(std::memory_order_relaxed)) return CFP8_OK;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
     flag.store(true, std::memory_order_relaxed);
     return CFP8_OK;
 }
 static int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached) beyond
+    if (dry_run()) return 64;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 64;
     return dev >= 0 && dev < 64 ? dev : 64;
 }
 
 static int cu_count() {  // compute units of the current device
+    if (dry_run()) return g_rec.cus;
     static std::atomic<int> cached[64];  // zero-initialised
     const int slot = device_slot();
     if (slot < 64) {
@@ -1441,6 +1467,7 @@ static int launch_rowwise_256p(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (!note_launch("gemm_rowwise_256p", (unsigned)blocks, 256, lds)) return CFP8_OK;
     if (v) hipLaunchKernelGGL(gemm_rowwise_256p_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_256p_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm");
@@ -1458,6 +1485,7 @@ static int launch_rowwise_256x128(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (!note_launch("gemm_rowwise_256x128", (unsigned)blocks, 256, lds)) return CFP8_OK;
     if (v) hipLaunchKernelGGL(gemm_rowwise_256x128_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_256x128_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm");
@@ -1478,6 +1506,7 @@ static int launch_rowwise_256(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    if (!note_launch("gemm_rowwise_256", (unsigned)blocks, 256, lds)) return CFP8_OK;
     if (v) hipLaunchKernelGGL(gemm_rowwise_256_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_256_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm");
@@ -1808,6 +1837,7 @@ template <int MR>
 static int launch_linear_gemv_fused_mr(const void* x, int64_t ld_x, GemmArgs& p, int out_dtype, hipStream_t st) {
     const int64_t blocks = (p.N + 15) / 16;
     const size_t lds = (size_t)p.M * (size_t)p.K;  // <= 16 KiB
+    if (!note_launch("linear_gemv_fused", (unsigned)blocks, 256, lds)) return CFP8_OK;
     if (out_dtype == CFP8_OUT_F32)
         hipLaunchKernelGGL((linear_gemv_fused_kernel<MR, true>), dim3((unsigned)blocks), dim3(256), lds, st, static_cast<const uint4*>(x), ld_x / 8, p);
     else
@@ -1822,6 +1852,7 @@ static int launch_linear_gemv_fused(const void* x, int64_t ld_x, GemmArgs& p, in
 
 static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int64_t blocks = (p.N + 15) / 16;
+    if (!note_launch("gemm_rowwise_gemv", (unsigned)blocks, 256, 0)) return CFP8_OK;
     if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(gemm_rowwise_gemv_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_gemv_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, p);
     return check_launch("gemm");
@@ -1864,6 +1895,13 @@ static int launch_rowwise_skinny_cfg(GemmArgs& p, int out_dtype, hipStream_t st)
     const int slot = device_slot();
     if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    {
+        char name[64];
+        snprintf(name, sizeof(name), "gemm_rowwise_skinny<%d,%d> k_slices=%d", TM, NTL, p.k_slices > 1 ? p.k_slices : 1);
+        const bool real = note_launch(name, (unsigned)blocks, NTL * 128, lds);
+        if (p.k_slices > 1) note_launch("splitk_reduce", (unsigned)(((int64_t)p.M * (p.N >> 2) + 255) / 256), 256, 0);
+        if (!real) return CFP8_OK;
+    }
     if (v) hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, true>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
     else hipLaunchKernelGGL((gemm_rowwise_skinny_kernel<TM, NTL, KS, false>), dim3((unsigned)blocks), dim3(NTL * 128), lds, st, p);
     if (p.k_slices > 1) {
@@ -1934,6 +1972,11 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
         const int slot = device_slot();
         if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
         if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds, done[slot][vec][f32])) return rc;
+    }
+    {
+        char name[64];
+        snprintf(name, sizeof(name), "gemm_kernel<%d,%d,%d,%d,%s>", BM, BN, WM, WN, MODE == kRowwise ? "rowwise" : MODE == kBlock ? "block" : "grouped");
+        if (!note_launch(name, (unsigned)blocks, NT, lds)) return CFP8_OK;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(NT), lds, st, p);
     return check_launch("gemm");
@@ -2381,6 +2424,7 @@ static int launch_block_w8p(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) done[64][f32].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][f32])) return rc;
+    if (!note_launch(MODE == kGrouped ? "gemm_block_w8p<128,256,grouped>" : "gemm_block_w8p<256,128,block>", (unsigned)blocks, 512, lds)) return CFP8_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
     return check_launch("gemm");
 }
@@ -2405,6 +2449,7 @@ static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec][f32])) return rc;
+    if (!note_launch(MODE == kGrouped ? "gemm_block_w8<128,256,grouped>" : "gemm_block_w8<256,128,block>", (unsigned)blocks, 512, lds)) return CFP8_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
     return check_launch("gemm");
 }
@@ -2429,6 +2474,7 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
         const int slot = device_slot();
         if (slot == 64) done[64].store(false, std::memory_order_relaxed);
         if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), 160 * 1024, done[slot])) return rc;
+        if (!note_launch("gemm_block_w8p<128,256,grouped,swiglu>", (unsigned)(blocks < cus ? blocks : cus), 512, lds)) return CFP8_OK;
         hipLaunchKernelGGL(kern, dim3((unsigned)(blocks < cus ? blocks : cus)), dim3(512), lds, st, p);
         return check_launch("gemm");
     }
@@ -2442,6 +2488,7 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) done[64][vec].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec])) return rc;
+    if (!note_launch("gemm_block_w8<128,256,grouped,swiglu>", (unsigned)blocks, 512, lds)) return CFP8_OK;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
     return check_launch("gemm");
 }
@@ -2564,6 +2611,72 @@ int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x
                          float* scales, bool streaming_out, hipStream_t st);
 
 }  // namespace cfp8
+
+extern "C" int cfp8_gemm_dispatch_info(int kind, int64_t M, int64_t N, int64_t K, int out_dtype, int cus, int with_split_workspace,
+                                       char* buf, size_t buf_bytes) {
+    using namespace cfp8;
+    if (!buf || buf_bytes == 0) return set_error(CFP8_EINVAL, "gemm_dispatch_info: no buffer");
+    buf[0] = 0;
+    if (M <= 0 || N <= 0 || K <= 0 || K % 128 || N % 16 || M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || cus <= 0)
+        return set_error(CFP8_EINVAL, "gemm_dispatch_info: bad shape or compute-unit count");
+    if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "gemm_dispatch_info: unknown out_dtype %d", out_dtype);
+    // operands that pass every alignment test; nothing dereferences them
+    static const uintptr_t fake = 0x100000;
+    GemmArgs p{};
+    p.a = reinterpret_cast<const uint8_t*>(fake);
+    p.b = reinterpret_cast<const uint8_t*>(fake);
+    p.sa = reinterpret_cast<const float*>(fake);
+    p.sb = reinterpret_cast<const float*>(fake);
+    p.m_indices = reinterpret_cast<const int32_t*>(fake);
+    p.out = reinterpret_cast<void*>(fake);
+    p.h_scales = reinterpret_cast<float*>(fake);
+    p.ld_a = K; p.ld_b = K; p.ld_out = N;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    g_rec.dry = true;
+    g_rec.cus = cus;
+    g_rec.len = 0;
+    g_rec.text[0] = 0;
+    int rc = CFP8_OK;
+    const int64_t kb = K / 128, nb = (N + 127) / 128;
+    switch (kind) {
+        case CFP8_DISPATCH_ROWWISE:
+            rc = launch_gemm<kRowwise>(p, out_dtype, nullptr);
+            break;
+        case CFP8_DISPATCH_LINEAR:
+            if (fused_gemv_applies(M, K, reinterpret_cast<const void*>(fake), K)) {
+                rc = launch_linear_gemv_fused(reinterpret_cast<const void*>(fake), K, p, out_dtype, nullptr);
+            } else {
+                note_launch("quant_rowwise", 0, 256, 0);
+                if (with_split_workspace) {
+                    p.partial = reinterpret_cast<float*>(fake);
+                    p.partial_bytes = cfp8_linear_workspace_bytes_split(M, N, K) - cfp8_linear_workspace_bytes(M, K);
+                }
+                rc = launch_gemm<kRowwise>(p, out_dtype, nullptr);
+            }
+            break;
+        case CFP8_DISPATCH_BLOCK:
+            p.sb_stride_n = kb; p.sb_stride_k = 1;
+            rc = launch_gemm<kBlock>(p, out_dtype, nullptr);
+            break;
+        case CFP8_DISPATCH_GROUPED:
+            p.sb_stride_n = kb; p.sb_stride_k = 1; p.sb_stride_e = nb * kb;
+            rc = M % 128 ? set_error(CFP8_EINVAL, "gemm_dispatch_info: grouped M must be a multiple of 128") : launch_gemm<kGrouped>(p, out_dtype, nullptr);
+            break;
+        case CFP8_DISPATCH_GROUPED_SWIGLU:  // N = 2 I; the quantised product has N / 2 columns
+            p.sb_stride_n = kb; p.sb_stride_k = 1; p.sb_stride_e = nb * kb;
+            p.ld_out = N / 2; p.ld_hs = N / 256;
+            rc = (M % 128 || N % 256 || out_dtype != CFP8_OUT_BF16)
+                     ? set_error(CFP8_EINVAL, "gemm_dispatch_info: grouped SwiGLU needs M %% 128 == 0, N %% 256 == 0 and the bf16 form")
+                     : launch_grouped_swiglu(p, nullptr);
+            break;
+        default:
+            rc = set_error(CFP8_EINVAL, "gemm_dispatch_info: unknown kind %d", kind);
+    }
+    g_rec.dry = false;
+    if (rc) return rc;
+    snprintf(buf, buf_bytes, "%s", g_rec.text);
+    return CFP8_OK;
+}
 
 extern "C" int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* sa, const void* b, int64_t ld_b,
                                       const float* sb, void* out, int64_t ld_out, int out_dtype, int64_t M,

@@ -308,6 +308,22 @@ int cfp8_gemm_grouped_block128(const void* a, int64_t ld_a, const float* sa,
                                void* out, int64_t ld_out, int out_dtype,
                                int64_t M, int64_t N, int64_t K, int64_t E, void* stream);
 
+/* Which kernels a GEMM call would launch, without launching anything and without a device: the
+ * dispatch code of the entry point named by `kind` runs with launches switched off and writes, for
+ * each kernel in order, "<kernel> grid=<workgroups> block=<threads> lds=<bytes>" separated by "; "
+ * into buf.  `cus` stands in for the device's compute-unit count (256 on MI355X), which several
+ * choices depend on; with_split_workspace says whether CFP8_DISPATCH_LINEAR is given the larger
+ * workspace of cfp8_linear_workspace_bytes_split.  No counterpart in the reference: it exists so
+ * that a test can pin, on any machine, that a shape still takes the kernel form its parity tests
+ * cover.  CFP8_DISPATCH_GROUPED_SWIGLU takes N = 2 I. */
+#define CFP8_DISPATCH_ROWWISE 0        /* cfp8_scaled_mm_rowwise          */
+#define CFP8_DISPATCH_LINEAR 1         /* cfp8_linear_rowwise             */
+#define CFP8_DISPATCH_BLOCK 2          /* cfp8_gemm_block128              */
+#define CFP8_DISPATCH_GROUPED 3        /* cfp8_gemm_grouped_block128      */
+#define CFP8_DISPATCH_GROUPED_SWIGLU 4 /* cfp8_gemm_grouped_swiglu_quant  */
+int cfp8_gemm_dispatch_info(int kind, int64_t M, int64_t N, int64_t K, int out_dtype, int cus,
+                            int with_split_workspace, char* buf, size_t buf_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,85 @@
+"""Which kernel form each benchmark and parity shape is dispatched to, with its launch geometry and LDS bytes.
+
+The kernels in which one workgroup walks several tiles keep loads in flight across barriers that are written with
+hand-counted wait counts; what guards them is the parity and repeatability tests at the shapes listed here.  A change
+of a dispatch threshold that silently moved one of these shapes to another kernel form would leave that form untested
+at its benchmark shape - this file fails instead.  Runs without a GPU: the library walks its dispatch code with
+launching switched off (cfp8_gemm_dispatch_info)."""
+import pytest
+
+from cosmos_rl_amd import _lib as L
+
+ROW, LIN, BLK, GRP, SWI = L.DISPATCH_ROWWISE, L.DISPATCH_LINEAR, L.DISPATCH_BLOCK, L.DISPATCH_GROUPED, L.DISPATCH_GROUPED_SWIGLU
+LDS_ROW = (2 + 3) * 256 * 128            # two activation + three weight stages of the 256 x 256 rowwise kernels
+
+
+def w8p_lds(bm, bn, kt):
+    return (2 * bm + 3 * bn) * 128 + 2 * 8 * bm * 4 + 8 * 16 * 144 + 2 * 128 * 4 + 2 * ((kt * (bn // 128) + 63) & ~63) * 4
+
+
+def w8_lds(bm, bn, kt):
+    return (2 * bm + 3 * bn) * 128 + 2 * 8 * bm * 4 + kt * (bn // 128) * 4
+
+
+CASES = [
+    # benchmark config 3 (rowwise linear, N = 18944, K = 3584)
+    ("cfg3 M=8192", (ROW, 8192, 18944, 3584),
+     f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
+    ("cfg3 M=8192 linear", (LIN, 8192, 18944, 3584),
+     f"quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}; "
+     "gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
+    ("cfg3 M=1024", (ROW, 1024, 18944, 3584),
+     f"gemm_rowwise_256 grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=160 block=256 lds=65536"),
+    ("cfg3 M=64", (LIN, 64, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_skinny<4,5> k_slices=1 grid=237 block=640 lds=131072"),
+    ("cfg3 M=1", (LIN, 1, 18944, 3584), "linear_gemv_fused grid=1184 block=256 lds=3584"),
+    ("cfg3 M=16", (LIN, 16, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_gemv grid=1184 block=256 lds=0"),
+    ("down projection M=64, split-K workspace", (LIN, 64, 3584, 18944, L.OUT_BF16, 256, True),
+     "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_skinny<4,4> k_slices=4 grid=224 block=512 lds=131072; splitk_reduce grid=224 block=256 lds=0"),
+    # benchmark config 4 and the short-K block shape
+    ("cfg4", (BLK, 4096, 18432, 7168), f"gemm_block_w8<256,128,block> grid=2304 block=512 lds={w8_lds(256, 128, 56)}"),
+    ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 12)}"),
+    # benchmark config 5 (73600 padded rows)
+    ("cfg5 gate_up", (GRP, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
+    ("cfg5 gate_up + SwiGLU", (SWI, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped,swiglu> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
+    ("cfg5 down", (GRP, 73600, 2048, 768), f"gemm_block_w8<128,256,grouped> grid=4600 block=512 lds={w8_lds(128, 256, 6)}"),
+    # the shapes of the walking-kernel parity tests (tests/test_gpu_gemm.py): each must take the walking form
+    ("walk rowwise 2304x11520x512", (ROW, 2304, 11520, 512), f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}"),
+    ("walk rowwise 8192x7680x896", (ROW, 8192, 7680, 896), f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}"),
+    ("walk block 1024x12288x1536", (BLK, 1024, 12288, 1536), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 12)}"),
+    ("walk block 2048x6400x640", (BLK, 2048, 6400, 640), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 5)}"),
+    ("walk grouped K=1536", (GRP, 7168, 2048, 1536), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 12)}"),
+    ("walk grouped K=896", (GRP, 7168, 2048, 896), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 7)}"),
+    ("walk grouped SwiGLU K=2176", (SWI, 7168, 2048, 2176), f"gemm_block_w8p<128,256,grouped,swiglu> grid=256 block=512 lds={w8p_lds(128, 256, 17)}"),
+    # ... and their sliced counterparts must not
+    ("sliced rowwise", (ROW, 2304, 3840, 512), f"gemm_rowwise_256 grid=135 block=256 lds={LDS_ROW}"),
+    ("sliced grouped", (GRP, 7168, 512, 1536), "gemm_kernel<128,128,2,2,grouped> grid=224 block=256 lds=73728"),
+]
+
+
+@pytest.mark.parametrize("name,args,want", CASES, ids=[c[0] for c in CASES])
+def test_dispatch_is_pinned(name, args, want):
+    assert L.gemm_dispatch_info(*args) == want
+
+
+def test_dispatch_limits_of_the_walking_forms():
+    """K range of the walking forms and the tile count above which they apply."""
+    info = L.gemm_dispatch_info
+    assert "w8p" in info(GRP, 73600, 2048, 896) and "w8p" not in info(GRP, 73600, 2048, 768)          # grouped: from 7 K steps
+    assert "w8p" in info(GRP, 73600, 2048, 4096) and "w8p" not in info(GRP, 73600, 2048, 4224)        # ... to 32
+    assert "w8p" in info(BLK, 4096, 24576, 384) and "w8p" not in info(BLK, 4096, 24576, 256)          # block: from 3
+    assert "256p" in info(ROW, 8192, 18944, 384) and "256p" not in info(ROW, 8192, 18944, 256)        # rowwise: K >= 384
+    assert "256p" not in info(ROW, 2048, 4608, 3584)                                                  # no more tiles than CUs
+    assert "256p" in info(ROW, 2048, 4608, 3584, L.OUT_BF16, 64)                                      # ... unless the GPU is smaller
+    assert "swiglu" in info(SWI, 256, 512, 256)
+
+
+def test_dispatch_info_rejects_bad_arguments():
+    lib = L.load()
+    import ctypes
+    buf = ctypes.create_string_buffer(64)
+    assert lib.cfp8_gemm_dispatch_info(ROW, 128, 128, 100, 0, 256, 0, buf, 64) == L.EINVAL      # K % 128
+    assert lib.cfp8_gemm_dispatch_info(9, 128, 128, 128, 0, 256, 0, buf, 64) == L.EINVAL        # kind
+    assert lib.cfp8_gemm_dispatch_info(GRP, 100, 256, 128, 0, 256, 0, buf, 64) == L.EINVAL      # grouped M % 128
+    assert lib.cfp8_gemm_dispatch_info(ROW, 128, 128, 128, 0, 256, 0, None, 0) == L.EINVAL
+    # a short buffer truncates, it does not overflow
+    assert lib.cfp8_gemm_dispatch_info(ROW, 8192, 18944, 3584, 0, 256, 0, buf, 16) == 0 and len(buf.value) == 15
