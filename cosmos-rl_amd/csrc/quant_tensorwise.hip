@@ -1,13 +1,17 @@
 // Tensorwise dynamic FP8 quantisation of many tensors: two launches per batch of
 // up to 48 tensors (and a bounded number of bytes), no host round trip between them.
 //
-//   pass 1 (amax)  reads 2 B/element.  Every workgroup reduces one contiguous
-//                  chunk of one tensor and publishes its maximum with one
+//   pass 1 (amax)  reads 2 B/element.  Every workgroup reduces a few contiguous
+//                  chunks of one tensor and publishes its maximum with one
 //                  fire-and-forget atomic max on the bit pattern (valid because
 //                  |x| >= 0, and NaN patterns sort above infinity, so NaN
 //                  propagates).  A tensor owns kAmaxSlots slots and a workgroup
 //                  picks one by its index: thousands of co-resident workgroups
-//                  hitting a single address serialise at the memory side.
+//                  hitting a single address serialise at the memory side.  Even
+//                  so the 64 slots are two cache lines, and one atomic per 32 KiB
+//                  holds a 1 GB tensor at 5.2 TB/s where the same loads without
+//                  the atomic reach 6.9: a large launch therefore gives every
+//                  workgroup up to 8 chunks (one atomic per 256 KiB).
 //   pass 2 (cast)  reads 2 B and writes 1 B per element; every workgroup folds
 //                  the tensor's slots and forms the scale on its own.
 // The table of tensors travels in the kernel arguments (scalar loads), so the
@@ -31,7 +35,14 @@ struct TensorTable {
     u32* amax[kMaxBatch];  // kAmaxSlots slots each
     unsigned first_block[kMaxBatch + 1];  // exclusive prefix of workgroups per tensor
     int n;
+    int per;  // chunks per workgroup (pass 1 only; pass 2 is one chunk per workgroup)
 };
+
+// Chunks per workgroup of pass 1 for a launch of `chunks` chunks in all: one while the launch is small (every
+// chunk its own workgroup fills the GPU best), more once there are plenty.
+static inline int amax_chunks_per_block(uint64_t chunks) {
+    return chunks >= 32768 ? 8 : chunks >= 16384 ? 4 : chunks >= 8192 ? 2 : 1;
+}
 
 __device__ __forceinline__ int find_tensor(const TensorTable& tb, unsigned b) {
     int lo = 0, hi = tb.n - 1;
@@ -53,29 +64,32 @@ __global__ __launch_bounds__(256) void tensorwise_amax_kernel(const TensorTable 
     __shared__ u32 red[4];
     const int t = find_tensor(tb, blockIdx.x);
     const unsigned local = blockIdx.x - tb.first_block[t];
-    const int64_t base = (int64_t)local * kChunkVecs;
     const int64_t nvec = tb.nvec[t];
-    const uint4* x = tb.x[t] + base;
-    const int64_t left = nvec - base;
-    uint4 v[8];
-    if (left >= kChunkVecs) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = ld16<LDNT>(x + threadIdx.x + 256 * i);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int idx = threadIdx.x + 256 * i;
-            v[i] = idx < left ? ld16<LDNT>(x + idx) : make_uint4(0, 0, 0, 0);
-        }
-    }
     u32 m = 0;
+    for (int c = 0; c < tb.per; ++c) {
+        const int64_t base = ((int64_t)local * tb.per + c) * kChunkVecs;
+        const int64_t left = nvec - base;
+        if (left <= 0) break;  // uniform
+        const uint4* x = tb.x[t] + base;
+        uint4 v[8];
+        if (left >= kChunkVecs) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) m = absmax8(m, v[i]);
+            for (int i = 0; i < 8; ++i) v[i] = ld16<LDNT>(x + threadIdx.x + 256 * i);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int idx = threadIdx.x + 256 * i;
+                v[i] = idx < left ? ld16<LDNT>(x + idx) : make_uint4(0, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = absmax8(m, v[i]);
+    }
     m = wave_max(pk_fold(m));
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-        m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;  // fp32 bit pattern of the chunk amax
+        m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;  // fp32 bit pattern of the workgroup's amax
         if (m) atomicMax(tb.amax[t] + (local & (kAmaxSlots - 1)), m);  // result unused: the wave does not wait
     }
 }
@@ -139,29 +153,42 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
     // because every launch pays a ramp-up and a tail.
     int64_t i = 0;
     while (i < n) {
-        TensorTable tb;
-        tb.n = 0;
-        unsigned blocks = 0;
-        while (i < n && tb.n < kMaxBatch) {
-            const cfp8_tensor_desc& d = descs[i];
-            int64_t nvec = d.numel / 8;
-            // a tensor with no element still owns one workgroup: it writes the scale
-            unsigned nb = (unsigned)((nvec + kChunkVecs - 1) / kChunkVecs);
-            if (nb == 0) nb = 1;
-            if (tb.n > 0 && (uint64_t)blocks + nb > 0x7FFFFFFFull) break;
-            tb.x[tb.n] = static_cast<const uint4*>(d.x);
-            tb.q[tb.n] = static_cast<uint2*>(d.q);
-            tb.scale[tb.n] = d.scale;
-            tb.nvec[tb.n] = nvec;
-            tb.amax[tb.n] = slots + i * kAmaxSlots;
-            tb.first_block[tb.n] = blocks;
-            blocks += nb;
-            ++tb.n;
+        // the tensors of this batch: at most kMaxBatch, and few enough chunks for one grid
+        const int64_t first = i;
+        uint64_t chunks = 0;
+        int count = 0;
+        while (i < n && count < kMaxBatch) {
+            uint64_t nc = (uint64_t)((descs[i].numel / 8 + kChunkVecs - 1) / kChunkVecs);
+            if (nc == 0) nc = 1;  // a tensor with no element still owns one workgroup: it writes the scale
+            if (count > 0 && chunks + nc > 0x7FFFFFFFull) break;
+            chunks += nc;
+            ++count;
             ++i;
         }
-        tb.first_block[tb.n] = blocks;
-        if (phases & kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
-        if (phases & kPhaseCast) hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
+        // pass 1 gives a workgroup `per` chunks, pass 2 one: two tables that differ in the workgroup prefix
+        for (int phase = kPhaseAmax; phase <= kPhaseCast; phase <<= 1) {
+            if (!(phases & phase)) continue;
+            TensorTable tb;
+            tb.n = count;
+            tb.per = phase == kPhaseAmax ? amax_chunks_per_block(chunks) : 1;
+            unsigned blocks = 0;
+            for (int k = 0; k < count; ++k) {
+                const cfp8_tensor_desc& d = descs[first + k];
+                const int64_t nvec = d.numel / 8;
+                uint64_t nc = (uint64_t)((nvec + kChunkVecs - 1) / kChunkVecs);
+                if (nc == 0) nc = 1;
+                tb.x[k] = static_cast<const uint4*>(d.x);
+                tb.q[k] = static_cast<uint2*>(d.q);
+                tb.scale[k] = d.scale;
+                tb.nvec[k] = nvec;
+                tb.amax[k] = slots + (first + k) * kAmaxSlots;
+                tb.first_block[k] = blocks;
+                blocks += (unsigned)((nc + tb.per - 1) / tb.per);
+            }
+            tb.first_block[count] = blocks;
+            if (phase == kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
+            else hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
+        }
     }
     return check_launch("quant_tensorwise");
 }
