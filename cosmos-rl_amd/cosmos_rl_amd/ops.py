@@ -481,14 +481,15 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs: Tuple[torch.Tensor, torch.Ten
 
 def interleave_gate_up(gate: Tuple[torch.Tensor, torch.Tensor], up: Tuple[torch.Tensor, torch.Tensor]
                        ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Gate and up expert weights (fp8 [E, I, K], block scales [E, I/128, K/128] each) as one [E, 2I, K] weight
-    whose 128-row blocks alternate gate, up, gate, up ... - the layout ``grouped_gemm_swiglu_quant`` takes.
-    Done once, when the weights are arranged."""
+    """Gate and up expert weights (fp8 [E, I, K], block scales [E, I/128, K/128] each) as one [E, 2I, K] weight in
+    the layout ``grouped_gemm_swiglu_quant`` takes: rows alternate in units of 16 - 16 gate rows, the 16 up rows of
+    the same intermediate features, the next 16 gate rows ... - so every 256 rows hold one 128-feature block of both
+    projections; scale rows alternate per block: gate block j, up block j.  Done once, when the weights are arranged."""
     (qg, sg), (qu, su) = gate, up
     E, I, K = qg.shape
     if I % BLOCK or qu.shape != qg.shape or sg.shape != su.shape:
         raise ValueError("gate and up must have the same shape with I a multiple of 128")
-    q = torch.stack([qg.view(torch.uint8).view(E, I // BLOCK, BLOCK, K), qu.view(torch.uint8).view(E, I // BLOCK, BLOCK, K)], dim=2)
+    q = torch.stack([qg.view(torch.uint8).view(E, I // 16, 16, K), qu.view(torch.uint8).view(E, I // 16, 16, K)], dim=2)
     s = torch.stack([sg, su], dim=2)
     return q.reshape(E, 2 * I, K).view(FP8_DTYPE), s.reshape(E, 2 * I // BLOCK, K // BLOCK).contiguous()
 

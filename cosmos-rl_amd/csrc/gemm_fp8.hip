@@ -1056,6 +1056,83 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 }
 
 // ---------------------------------------------------------------------------
+// SwiGLU + 1x128 requantisation of a grouped gate_up tile, in registers.
+// The interleaved weight puts gate and up rows side by side in units of 16 (one MFMA tile): of a wave's four weight
+// tiles, 0 and 2 are gate rows and 1 and 3 the up rows of the same hidden columns, so a lane that holds gate[m][c .. c+3]
+// in acc[2 pp][j] holds up[m][c .. c+3] in acc[2 pp + 1][j] and forms h = bf16(bf16(silu(gate)) * up) without moving
+// anything - both rounded to bf16 first, as the GEMM would have written them, so the result is bit for bit that of the
+// grouped GEMM followed by the SwiGLU quantiser.  A wave covers 32 of the 128 hidden columns of the tile's 1x128 group;
+// the four waves that share token rows exchange their maxima through 2 KiB of LDS (`xch`: [128 rows][4] bf16 bit
+// patterns; one barrier), every lane derives the scale of its rows and casts its own values.  Per wave: 8 byte stores
+// (4 bytes per lane) and 4 scale stores, issued unconditionally: a row that does not belong to the tile's expert gets an
+// offset past the end of the buffer descriptor and the hardware drops it (the walking kernel counts stores between two
+// tiles).  LDS is touched by instructions written out: in front of an LDS access it knows of, the compiler waits for
+// every direct-to-LDS load in flight.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ u32 quarters_max(u32 v) {  // max over the four lanes l, l + 16, l + 32, l + 48; all get it
+    typedef u32 u32x2s __attribute__((ext_vector_type(2)));
+    const u32x2s a = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    v = umax(a[0], a[1]);
+    const u32x2s b = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return umax(b[0], b[1]);
+}
+// four bf16 (two packed words, element order preserved) -> four fp8 bytes
+__device__ __forceinline__ u32 cast4(u32 w0, u32 w1, const Divider& d) {
+    if (d.finite) {
+        const u32 lo = cvt2<false>(d.fast(bf16_lo(w0)), d.fast(bf16_hi(w0)), 0u);
+        return cvt2<true>(d.fast(bf16_lo(w1)), d.fast(bf16_hi(w1)), lo);
+    }
+    return slow_byte(bf16_lo(w0), d.s) | (slow_byte(bf16_hi(w0), d.s) << 8) | (slow_byte(bf16_lo(w1), d.s) << 16) |
+           (slow_byte(bf16_hi(w1), d.s) << 24);
+}
+// acc: [weight tile][token tile] of the wave's 64 x 64 block; row_keep[j]: the wave's token row j * 16 + lrow belongs to
+// the tile's expert; rq / rh: buffer descriptors of the tile's first row of the fp8 output and of its scales
+__device__ __forceinline__ void swiglu_quant_epilogue(const f32x4 (&acc)[4][4], uint8_t* xch, int wm, int wn, int lrow, int quarter,
+                                                      const bool (&row_keep)[4], __amdgpu_buffer_rsrc_t rq, __amdgpu_buffer_rsrc_t rh,
+                                                      int ld_out, int ld_hs, int tn) {
+    typedef __attribute__((address_space(3))) void lds_void;
+    u32 h[4][2][2];  // [token tile][pair][two packed bf16 words] of h
+    u32 mx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        u32 m = 0;
+#pragma unroll
+        for (int pp = 0; pp < 2; ++pp) {
+            const f32x4 g = acc[2 * pp][j], u = acc[2 * pp + 1][j];
+            h[j][pp][0] = swiglu_pair(pack_bf16x2(g[0], g[1]), pack_bf16x2(u[0], u[1]));
+            h[j][pp][1] = swiglu_pair(pack_bf16x2(g[2], g[3]), pack_bf16x2(u[2], u[3]));
+            m = pk_absmax(pk_absmax(m, h[j][pp][0]), h[j][pp][1]);
+        }
+        mx[j] = quarters_max(pk_fold(m));
+    }
+    const uint32_t xw = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(xch + ((wm * 64 + lrow) * 4 + wn) * 4));
+    const uint32_t xr = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(xch + (wm * 64 + lrow) * 16));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) asm volatile("ds_write_b32 %0, %1 offset:%2" ::"v"(xw), "v"(mx[j]), "n"(j * 256) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    u32x4 all[4];
+    asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:256\n\tds_read_b128 %2, %4 offset:512\n\t"
+                 "ds_read_b128 %3, %4 offset:768\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&v"(all[0]), "=&v"(all[1]), "=&v"(all[2]), "=&v"(all[3])
+                 : "v"(xr)
+                 : "memory");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32 amax_bits = umax(umax(all[j][0], all[j][1]), umax(all[j][2], all[j][3]));
+        const float scale = scale_from_amax(amax_from_bits(amax_bits));
+        const Divider d(scale);
+        const int r = wm * 64 + j * 16 + lrow;  // row of the tile
+#pragma unroll
+        for (int pp = 0; pp < 2; ++pp) {
+            const u32 bytes = cast4(h[j][pp][0], h[j][pp][1], d);
+            __builtin_amdgcn_raw_buffer_store_b32(bytes, rq, row_keep[j] ? (uint32_t)(r * ld_out + tn * 128 + wn * 32 + pp * 16 + quarter * 4) : 0xFFFFFFF0u, 0, 0);
+        }
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(scale), rh,
+                                              row_keep[j] && wn == 0 && quarter == 0 ? (uint32_t)((r * ld_hs + tn) * 4) : 0xFFFFFFF0u, 0, 0);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Block-scaled and grouped GEMM, full tiles: 256 x 128 (block) or 128 x 256 (grouped, whose groups are
 // 128 rows) x 128 per workgroup, eight wavefronts (two per SIMD), each a 64 x 64 block = 4 x tiles
 // times 4 w tiles.  Operand tiles go straight from global memory into LDS as in gemm_rowwise_256_kernel
@@ -1186,13 +1263,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         return r;
     };
     i32x8 W[4], X[4];
-    float sm[4], s_n;
+    float sm[4], s_n, s_nu = 0.f;  // s_nu: with the SwiGLU epilogue, the scale of the wave's up rows (s_n: of its gate rows)
     auto read_scales = [&](int kt) {  // s_m of this wave's four x tiles and s_n of its weight block for K step kt
         const int k = kt < last ? kt : last;
         const float* const sgk = sg_buf + (((k >> 3) & 1) * 8 + (k & 7)) * BM + wm * 64 + lrow;
 #pragma unroll
         for (int j = 0; j < 4; ++j) sm[j] = sgk[j * 16];
-        s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
+        if (SWIGLU) {
+            s_n = sn_lds[k * NB];
+            s_nu = sn_lds[k * NB + 1];
+        } else {
+            s_n = sn_lds[k * NB + (NB == 2 ? wn >> 1 : 0)];
+        }
     };
 
     // prologue: (activation tiles 0 and 1 are under way) weight tiles 0, 1, 2 into their stages, and the scales.  (The compiler waits
@@ -1224,6 +1306,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     read_scales(0);
     CFP8_PHASE_END();
     float sc2p = 0.f, sc3p = 0.f;  // scales of the products still waiting in P from the previous step
+    float sc2pu = 0.f, sc3pu = 0.f;  // SwiGLU: those of the up tiles (weight tiles 1 and 3)
+// the scale of weight tile i: with the SwiGLU epilogue odd tiles are up rows, which have a block scale of their own
+#define CFP8_SC(x, i) ((SWIGLU && ((i)&1)) ? x##u : x)
 
 // (the empty statement pins the four FMAs to this place: their results are not needed before the next step, and the
 // compiler would otherwise sink them past the branches of the tail, half of them to just behind the barrier)
@@ -1247,7 +1332,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         X[2] = frag(xs_cur, x_off, x_off2, 2);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            CFP8_RESCALE(i, 2, 0, sc2p);
+            CFP8_RESCALE(i, 2, 0, CFP8_SC(sc2p, i));
             CFP8_PRODUCT(i, 0, 0);
         }
         CFP8_PHASE_END();
@@ -1255,7 +1340,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         X[3] = frag(xs_cur, x_off, x_off2, 3);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            CFP8_RESCALE(i, 3, 1, sc3p);
+            CFP8_RESCALE(i, 3, 1, CFP8_SC(sc3p, i));
             CFP8_PRODUCT(i, 1, 1);
         }
         CFP8_PHASE_END();
@@ -1268,8 +1353,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         // were fetched a step earlier and are first read two barriers later, at the end of step 8 g + 7.
         if ((kt & 7) == 6) sg_store((kt >> 3) + 1);
         const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
+        const float sc0u = sm[0] * s_nu, sc1u = sm[1] * s_nu;
         sc2p = sm[2] * s_n;
         sc3p = sm[3] * s_n;
+        sc2pu = sm[2] * s_nu;
+        sc3pu = sm[3] * s_nu;
         X[0] = frag(xs_nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) dma_x(kx, kt & 1, i);
@@ -1277,8 +1365,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         CFP8_PHASE_END();
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            CFP8_RESCALE(i, 0, 0, sc0);
-            CFP8_RESCALE(i, 1, 1, sc1);
+            CFP8_RESCALE(i, 0, 0, CFP8_SC(sc0, i));
+            CFP8_RESCALE(i, 1, 1, CFP8_SC(sc1, i));
             CFP8_PRODUCT(i, 2, 0);
             CFP8_PRODUCT(i, 3, 1);
             CFP8_PHASE_END();
@@ -1294,55 +1382,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in the stages: the epilogues reuse them
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        CFP8_RESCALE(i, 2, 0, sc2p);
-        CFP8_RESCALE(i, 3, 1, sc3p);
+        CFP8_RESCALE(i, 2, 0, CFP8_SC(sc2p, i));
+        CFP8_RESCALE(i, 3, 1, CFP8_SC(sc3p, i));
     }
 #undef CFP8_RESCALE
 #undef CFP8_PRODUCT
+#undef CFP8_SC
 
     // epilogue: lane holds out[m][n .. n+3] for every (i, j)
     if constexpr (SWIGLU) {
-        // The tile's 256 weight rows are 128 gate rows followed by the 128 up rows of the same hidden columns
-        // (the caller interleaves the two projections in blocks of 128), so the tile holds everything one 1x128
-        // group of h = silu(gate) * up needs.  Both halves go to LDS rounded to bf16, as the GEMM would have
-        // written them; then four threads per token row form h, its group maximum and scale, and the fp8 bytes:
-        // the arithmetic of the separate SwiGLU quantiser, bit for bit, without the bf16 round trip through memory.
-        constexpr int GST = 272;                       // LDS row stride in bytes (128 bf16 + 16)
-        __syncthreads();                               // all waves are done reading the operand stages
-        uint8_t* const side = smem + (wn >> 1) * (128 * GST);
+        bool row_keep[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const f32x4 v = acc[i][j];
-                *reinterpret_cast<uint2*>(side + (wm * 64 + j * 16 + lrow) * GST + ((wn & 1) * 64 + i * 16 + quarter * 4) * 2) =
-                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-            }
-        __syncthreads();
-        const int r = t >> 2, c4 = t & 3;              // token row of the tile, 32-column part of the group
-        const uint8_t* const gp = smem + r * GST + c4 * 64;
-        const uint8_t* const up = gp + 128 * GST;
-        uint4 h[4];
-        u32 mx = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint4 g = *reinterpret_cast<const uint4*>(gp + e * 16), u = *reinterpret_cast<const uint4*>(up + e * 16);
-            h[e] = make_uint4(swiglu_pair(g.x, u.x), swiglu_pair(g.y, u.y), swiglu_pair(g.z, u.z), swiglu_pair(g.w, u.w));
-            mx = absmax8(mx, h[e]);
-        }
-        mx = pk_fold(mx);
-        mx = umax(mx, dpp<0xB1>(mx));                  // the four threads of a row are one DPP quad
-        mx = umax(mx, dpp<0x4E>(mx));
-        const float scale = scale_from_amax(amax_from_bits(mx));
-        const Divider d(scale);
-        const int m = m0 + r;
-        if (p.m_indices[m] == expert) {
-            uint8_t* const q = static_cast<uint8_t*>(p.out) + (int64_t)m * p.ld_out + tn * 128 + c4 * 32;
-            const uint2 b0 = cast8(h[0], d), b1 = cast8(h[1], d), b2 = cast8(h[2], d), b3 = cast8(h[3], d);
-            *reinterpret_cast<uint4*>(q) = make_uint4(b0.x, b0.y, b1.x, b1.y);
-            *reinterpret_cast<uint4*>(q + 16) = make_uint4(b2.x, b2.y, b3.x, b3.y);
-            if (c4 == 0) p.h_scales[(int64_t)m * p.ld_hs + tn] = scale;
-        }
+        for (int j = 0; j < 4; ++j) row_keep[j] = p.m_indices[m0 + wm * 64 + j * 16 + lrow] == expert;
+        __syncthreads();  // all waves are done reading the operand stages: their first bytes serve the exchange of maxima
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(static_cast<uint8_t*>(p.out) + (int64_t)m0 * p.ld_out, 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(p.h_scales + (int64_t)m0 * p.ld_hs, 0, 0x80000000u, 0x00020000);
+        swiglu_quant_epilogue(acc, smem, wm, wn, lrow, quarter, row_keep, rq, rh, (int)p.ld_out, (int)p.ld_hs, tn);
         return;
     }
     if (OUT_F32) {
@@ -2122,12 +2177,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         return r;
     };
     i32x8 W[4], X[4];
-    float sm[4], s_n;
+    float sm[4], s_n, s_nu = 0.f;  // s_nu: with the SwiGLU epilogue, the scale of the wave's up rows (s_n: of its gate rows)
     auto read_scales = [&](int gpar_, int snpar_, int k) {  // s_m of the wave's four x tiles and s_n of its weight block for step k
         const float* const sgk = sg_buf + (((gpar_ + (k >> 3)) & 1) * 8 + (k & 7)) * BM + wm * 64 + lrow;
 #pragma unroll
         for (int j = 0; j < 4; ++j) sm[j] = sgk[j * 16];
-        s_n = sn_lds[snpar_ * KTP + k * NB + (NB == 2 ? wn >> 1 : 0)];
+        if (SWIGLU) {
+            s_n = sn_lds[snpar_ * KTP + k * NB];
+            s_nu = sn_lds[snpar_ * KTP + k * NB + 1];
+        } else {
+            s_n = sn_lds[snpar_ * KTP + k * NB + (NB == 2 ? wn >> 1 : 0)];
+        }
     };
 
     int pid = blockIdx.x;
@@ -2169,6 +2229,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         P[1][i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     float sc2p = 0.f, sc3p = 0.f;  // scales of the products still waiting in P from the previous step
+    float sc2pu = 0.f, sc3pu = 0.f;  // SwiGLU: those of the up tiles (weight tiles 1 and 3)
+// the scale of weight tile i: with the SwiGLU epilogue odd tiles are up rows, which have a block scale of their own
+#define CFP8_SC(x, i) ((SWIGLU && ((i)&1)) ? x##u : x)
     int xs = 0, ws = 0;            // stages of the stream's current step: activation stage (0 or XS bytes), weight stage 0..2
     int gpar = 0, snpar = 0;       // scale buffers of the current tile: first group of activation scales, weight scales
 
@@ -2203,7 +2266,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             X[2] = frag(xs, x_off, x_off2, 2);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                CFP8_RESCALE(i, 2, 0, sc2p);
+                CFP8_RESCALE(i, 2, 0, CFP8_SC(sc2p, i));
                 CFP8_PRODUCT(i, 0, 0);
             }
             CFP8_PHASE_END();
@@ -2211,7 +2274,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             X[3] = frag(xs, x_off, x_off2, 3);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                CFP8_RESCALE(i, 3, 1, sc3p);
+                CFP8_RESCALE(i, 3, 1, CFP8_SC(sc3p, i));
                 CFP8_PRODUCT(i, 1, 1);
             }
             CFP8_PHASE_END();
@@ -2224,7 +2287,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
                 if constexpr (OUT_F32) CFP8_WAIT_BARRIER(18);
                 else CFP8_WAIT_BARRIER(10);
             } else {
-                if constexpr (OUT_F32) CFP8_WAIT_BARRIER(20);
+                if constexpr (SWIGLU) CFP8_WAIT_BARRIER(16);  // 8 byte stores + 4 scale stores per wave
+                else if constexpr (OUT_F32) CFP8_WAIT_BARRIER(20);
                 else CFP8_WAIT_BARRIER(12);
             }
             CFP8_PHASE_END();
@@ -2234,8 +2298,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             if ((kt & 7) == 6 && kt + 2 <= last) sg_store(gpar + (kt >> 3) + 1);
             if (kt == last - 1) sg_store(gpar + G);
             const float sc0 = sm[0] * s_n, sc1 = sm[1] * s_n;
+            const float sc0u = sm[0] * s_nu, sc1u = sm[1] * s_nu;
             sc2p = sm[2] * s_n;
             sc3p = sm[3] * s_n;
+            sc2pu = sm[2] * s_nu;
+            sc3pu = sm[3] * s_nu;
             X[0] = frag(xs_nxt, x_off, x_off2, 0);
             if (kt == last - 1) dma_sn(m0n, n0n, expert_n, snpar ^ 1);  // older than this step's weight loads: landed at the next barrier
 #pragma unroll
@@ -2245,8 +2312,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
             CFP8_PHASE_END();
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                CFP8_RESCALE(i, 0, 0, sc0);
-                CFP8_RESCALE(i, 1, 1, sc1);
+                CFP8_RESCALE(i, 0, 0, CFP8_SC(sc0, i));
+                CFP8_RESCALE(i, 1, 1, CFP8_SC(sc1, i));
                 CFP8_PRODUCT(i, 2, 0);
                 CFP8_PRODUCT(i, 3, 1);
                 CFP8_PHASE_END();
@@ -2265,11 +2332,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         for (int kt = 1; kt < KT; ++kt) step(kt, std::integral_constant<int, 0>{});
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            CFP8_RESCALE(i, 2, 0, sc2p);
-            CFP8_RESCALE(i, 3, 1, sc3p);
+            CFP8_RESCALE(i, 2, 0, CFP8_SC(sc2p, i));
+            CFP8_RESCALE(i, 3, 1, CFP8_SC(sc3p, i));
         }
         sc2p = 0.f;  // the products left in P belong to this tile
         sc3p = 0.f;
+        sc2pu = 0.f;
+        sc3pu = 0.f;
 
         // epilogue: lane holds out[m][n .. n+3] for every (i, j).  Its per-lane addresses are derived here, from a
         // lane number the compiler cannot see through: hoisted out of the tile loop they would occupy registers
@@ -2281,58 +2350,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
         // with an offset past the end of the buffer descriptor (the hardware drops them): the barrier of the next tile's
         // first step counts on a fixed number of stores in front of the loads it lets pass.
         if constexpr (SWIGLU) {
-            // The tile's 256 weight rows are 128 gate rows followed by the 128 up rows of the same hidden columns, so the
-            // tile holds everything one 1x128 group of h = silu(gate) * up needs.  32 token rows at a time (the epilogue
-            // buffers hold no more): the four waves that own them put both halves into LDS rounded to bf16, as the GEMM
-            // would have written them; then sixteen threads per row form h, its group maximum and scale, and the fp8
-            // bytes - the arithmetic of the separate SwiGLU quantiser, bit for bit.  Two stores per wave and pass.
-            constexpr int GST = 272;  // LDS row stride in bytes (128 bf16 + 16)
-            uint8_t* const sw = smem + EBASE;  // [gate, up][32 rows][GST]
-            const int32_t* const tile_expert_of_row = reinterpret_cast<const int32_t*>(smem + IBASE) + snpar * 128;
+            // (which of the wave's rows belong to the tile's expert: read by an instruction of its own, see swiglu_quant_epilogue)
+            const uint32_t ie = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(smem + IBASE + (snpar * 128 + wm * 64 + lrow_e) * 4));
+            int re[4];
+            asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %4 offset:64\n\tds_read_b32 %2, %4 offset:128\n\t"
+                         "ds_read_b32 %3, %4 offset:192\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(re[0]), "=&v"(re[1]), "=&v"(re[2]), "=&v"(re[3])
+                         : "v"(ie)
+                         : "memory");
+            const bool row_keep[4] = {re[0] == expert, re[1] == expert, re[2] == expert, re[3] == expert};
             const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
                 static_cast<uint8_t*>(p.out) + (int64_t)m0 * p.ld_out, 0, 0x80000000u, 0x00020000);
             const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(
                 p.h_scales + (int64_t)m0 * p.ld_hs, 0, 0x80000000u, 0x00020000);
-            const int tn = n0 >> 8;
-            int te = t;
-            asm volatile("" : "+v"(te));
-            const int r32 = te >> 4, c16 = te & 15;
-            const uint32_t sw_wr = (uint32_t) reinterpret_cast<uintptr_t>(
-                (lds_void*)(sw + (wn >> 1) * (32 * GST) + lrow_e * GST + ((wn & 1) * 64 + quarter_e * 4) * 2));
-            const uint32_t sw_rd = (uint32_t) reinterpret_cast<uintptr_t>((lds_void*)(sw + r32 * GST + c16 * 16));
-#pragma unroll
-            for (int qp = 0; qp < 4; ++qp) {
-                if (qp) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // the previous pass has been read
-                if (wm == (qp >> 1)) {
-#pragma unroll
-                    for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const f32x4 v = acc[i][(qp & 1) * 2 + jj];
-                            const uint64_t two = (uint64_t)pack_bf16x2(v[0], v[1]) | ((uint64_t)pack_bf16x2(v[2], v[3]) << 32);
-                            asm volatile("ds_write_b64 %0, %1 offset:%2" ::"v"(sw_wr), "v"(two), "n"(jj * 16 * GST + i * 32) : "memory");
-                        }
-                }
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                // (read by instructions of its own: in front of an LDS read it knows of, the compiler waits for the
-                // next tile's loads that are on their way into other parts of LDS)
-                u32x4 gv, uv;
-                asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
-                             : "=&v"(gv), "=&v"(uv)
-                             : "v"(sw_rd), "n"(32 * GST)
-                             : "memory");
-                const uint4 g = make_uint4(gv[0], gv[1], gv[2], gv[3]), u = make_uint4(uv[0], uv[1], uv[2], uv[3]);
-                const uint4 h = make_uint4(swiglu_pair(g.x, u.x), swiglu_pair(g.y, u.y), swiglu_pair(g.z, u.z), swiglu_pair(g.w, u.w));
-                const u32 mx = row16_max(pk_fold(absmax8(0u, h)));  // the sixteen threads of a row are one DPP row
-                const float scale = scale_from_amax(amax_from_bits(mx));
-                const Divider d(scale);
-                const int r = qp * 32 + r32;  // row of the tile
-                const bool keep = tile_expert_of_row[r] == expert;
-                const uint2 b = cast8(h, d);
-                __builtin_amdgcn_raw_buffer_store_b64(u32x2{b.x, b.y}, rq, keep ? (uint32_t)(r * (int)p.ld_out + tn * 128 + c16 * 8) : 0xFFFFFFF0u, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(scale), rh, keep && c16 == 0 ? (uint32_t)((r * (int)p.ld_hs + tn) * 4) : 0xFFFFFFF0u, 0, 0);
-            }
-            // (the first barrier of the next tile's K loop separates its first pass from this tile's last reads)
+            // the exchange buffer is the first 2 KiB of the epilogue buffers; the K loop of the next tile (many barriers)
+            // lies between this tile's reads of it and the next tile's writes
+            swiglu_quant_epilogue(acc, smem + EBASE, wm, wn, lrow_e, quarter_e, row_keep, rq, rh, (int)p.ld_out, (int)p.ld_hs, n0 >> 8);
         } else {
         const int32_t* const row_expert = reinterpret_cast<const int32_t*>(smem + IBASE) + snpar * 128 + wm * 64;
         const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
@@ -2400,6 +2433,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
     }
 #undef CFP8_RESCALE
 #undef CFP8_PRODUCT
+#undef CFP8_SC
     // the loads past the last tile (they fetched its first steps once more) land before the workgroup gives up its LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }

@@ -181,11 +181,13 @@ int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up
  * cfp8_gemm_grouped_block128 (on the concatenated gate and up weights) followed by
  * cfp8_swiglu_quant_group128 compute, bit for bit, without writing the bf16 [M, 2 I] product to memory
  * and reading it back.  Replaces cosmos_rl/policy/kernel/group_gemms.py:194-218 as one launch.
- * b fp8 [E, 2 I, K] and sb fp32 [E, 2 I / 128, K / 128] hold gate and up interleaved in blocks of 128
- * rows: rows [256 j, 256 j + 128) = gate rows [128 j, 128 j + 128), rows [256 j + 128, 256 j + 256) = up rows
- * [128 j, 128 j + 128) (scale rows 2 j and 2 j + 1 likewise), so that one 128 x 256 tile holds both halves
- * of a 1x128 group of h = silu(gate) * up.  q fp8 [M, I] (pitch ld_q bytes), scales fp32 [M, I / 128];
- * rows with m_indices < 0 are left untouched.  M % 128 == 0, I % 128 == 0, K % 128 == 0. */
+ * b fp8 [E, 2 I, K] holds gate and up rows interleaved in units of 16 (one MFMA tile): for every block j of 128
+ * intermediate features and p = 0 .. 7, rows [256 j + 32 p, + 16) = gate rows [128 j + 16 p, + 16) and rows
+ * [256 j + 32 p + 16, + 16) = the up rows of the same features - a lane of the GEMM then holds a gate value and the up
+ * value it is multiplied with, and the SwiGLU needs no exchange.  sb fp32 [E, 2 I / 128, K / 128]: scale row 2 j = the
+ * block scales of gate block j, row 2 j + 1 those of up block j (ops.interleave_gate_up builds both).  One 128 x 256
+ * tile holds both halves of a 1x128 group of h = silu(gate) * up.  q fp8 [M, I] (pitch ld_q bytes), scales fp32
+ * [M, I / 128]; rows with m_indices < 0 are left untouched.  M % 128 == 0, I % 128 == 0, K % 128 == 0. */
 int cfp8_gemm_grouped_swiglu_quant(const void* a, int64_t ld_a, const float* sa, const void* b, const float* sb,
                                    const int32_t* m_indices, void* q, int64_t ld_q, float* scales,
                                    int64_t M, int64_t I, int64_t K, int64_t E, void* stream);

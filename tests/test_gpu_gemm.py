@@ -302,7 +302,9 @@ def test_grouped_swiglu_epilogue_bit_exact(dev, T, E, K, I, topk):
     ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (torch.cat([qg, qu], 1), torch.cat([sg, su], 1)), gu, mi)
     q0, s0 = ops.swiglu_quant(gu[:, :I], gu[:, I:])
     qi, si = ops.interleave_gate_up((qg, sg), (qu, su))
-    assert torch.equal(qi.view(torch.uint8)[:, 128:256], qu.view(torch.uint8)[:, :128]) and torch.equal(si[:, 1], su[:, 0])
+    # rows alternate in units of 16: gate 0-15, up 0-15, gate 16-31, ...; scale rows alternate per block of 128
+    assert torch.equal(qi.view(torch.uint8)[:, 16:32], qu.view(torch.uint8)[:, :16]) and torch.equal(qi.view(torch.uint8)[:, 32:48], qg.view(torch.uint8)[:, 16:32])
+    assert torch.equal(si[:, 0], sg[:, 0]) and torch.equal(si[:, 1], su[:, 0])
     q1 = torch.full((xs.shape[0], I), 0x55, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
     s1 = torch.full((xs.shape[0], I // 128), -1.0, dtype=torch.float32, device=dev)
     from cosmos_rl_amd import _lib
