@@ -60,6 +60,31 @@ def test_graph_weight_quantisers(dev):
     _replay_matches_eager(dev, inputs, fn)
 
 
+def test_graph_batch_quantisers_without_allocation(dev):
+    """The table-driven rowwise quantiser and the tensorwise entry point whose amax slots live inside the library,
+    captured with caller-owned outputs: nothing inside the captured region allocates."""
+    shapes = [(512, 896), (300, 256), (64, 3584), (16, 18944)]
+    qs = [torch.empty(sh, dtype=torch.float8_e4m3fn, device=dev) for sh in shapes]
+    ss = [torch.empty(sh[0], 1, dtype=torch.float32, device=dev) for sh in shapes]
+    qt = [torch.empty(sh, dtype=torch.float8_e4m3fn, device=dev) for sh in shapes]
+    st = torch.empty(len(shapes), dtype=torch.float32, device=dev)
+
+    def inputs(seed):
+        return [_bf16(dev, seed + 10 * i, *sh, std=0.02 * (i + 1)) for i, sh in enumerate(shapes)]
+
+    def fn(*ws):
+        ops.quant_rowwise_multi_into(list(ws), qs, ss)
+        ops.quant_tensorwise_multi_static(list(ws), qt, st)
+        return (*qs, *ss, *qt, st)
+
+    _replay_matches_eager(dev, inputs, fn)
+    # and the captured results are the per-tensor ones
+    ws = inputs(13)
+    for w, q, sc in zip(ws, qs, ss):
+        q1, s1 = ops.quant_rowwise(w)
+        assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(sc, s1)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 3584), (64, 2048, 3584), (48, 1024, 7168), (1024, 2048, 3584), (2304, 8448, 256)])
 def test_graph_fp8_linear(dev, M, N, K):
     """single-token and 64-token kernels, the split-K pair of launches, 256x256 tiles, and the head + tail pair"""
