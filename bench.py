@@ -254,7 +254,8 @@ def summarise_top_level(extra):
     for k, nm, exact in (("rowwise_cfg1", "rowwise_cfg1_4864x896", True), ("rowwise_qkv", "rowwise_qkv_4608x3584", True),
                          ("rowwise_down", "rowwise_down_3584x18944", True), ("block128", "block128_cfg4_7168x18432", True),
                          ("block128_T", "block128_cfg4_7168x18432_T", True), ("group128", "group128_cfg4_4096x7168", True),
-                         ("swiglu_quant", "swiglu_quant_cfg5", False), ("gather_quant", "gather_quant_cfg5", False)):
+                         ("swiglu_quant", "swiglu_quant_cfg5", False), ("gather_quant", "gather_quant_cfg5", False),
+                         ("scatter_quant", "scatter_quant_cfg5", False)):
         for name, e in extra.items():
             if (name == nm if exact else name.startswith(nm)) and "frac_hbm" in e:
                 q[k] = e["frac_hbm"]
@@ -570,6 +571,10 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     row_of_slot[order] = start[e_sorted] + torch.arange(T * TOPK, device=dev) - first[e_sorted]
     slot_order = torch.argsort(topi.view(T, TOPK), dim=1, stable=True)
     row_map = torch.gather(row_of_slot.view(T, TOPK), 1, slot_order).to(torch.int32).contiguous()
+    # the same rows written from the token side: every token read and quantised once, stored to its TOPK rows
+    hbm("scatter_quant_cfg5_%dx%d" % (total, H), T * H * 2 + total * H + 4 * sxs.numel() + 4 * total + 4 * T * TOPK,
+        lambda: check(lib.cfp8_scatter_quant_group128(tok.data_ptr(), H, T, H, row_map.data_ptr(), TOPK, src.data_ptr(), total,
+                                                      qxs.data_ptr(), H, sxs.data_ptr(), stream)), copy_ceiling=True)
     probs = torch.rand(T, TOPK, generator=gen, device=dev).to(torch.bfloat16)
     yt = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
     hbm("combine_rows_cfg5_%dx%d_top%d" % (T, H, TOPK), T * TOPK * (2 * H + 6) + T * H * 2,

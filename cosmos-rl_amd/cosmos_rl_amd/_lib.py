@@ -55,6 +55,8 @@ SIGNATURES = {
                                   c_void_p, c_int64, c_void_p]),
     "cfp8_quant_mxfp4": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "cfp8_gather_quant_group128": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    "cfp8_scatter_quant_group128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                            c_void_p, c_void_p]),
     "cfp8_dequant_block128": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "cfp8_scaled_mm_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                        c_int, c_int64, c_int64, c_int64, c_void_p]),

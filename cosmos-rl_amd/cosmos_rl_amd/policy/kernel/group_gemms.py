@@ -113,22 +113,25 @@ class DSGroupGEMM(GroupGEMMStrategy):
         contig_tokens[:total] = self._run(self._quant(valid_tokens), m_indices, total, module, contig_tokens.dtype)
         return contig_tokens
 
-    def execute_from_tokens(self, tokens, row_tokens, m_sizes, m_offsets, module):
+    def execute_from_tokens(self, tokens, row_tokens, m_sizes, m_offsets, module, row_map=None):
         """``execute`` on ``tokens[row_tokens]`` (zero rows for -1) without building that matrix: the gather and the
         1x128 quantisation of the first GEMM's input are one pass over the token matrix.  Returns the expert outputs
         [rows, hidden] for the rows of the expert-grouped layout (``row_tokens``: token behind each row).  When
         ``row_tokens`` has a multiple of 128 entries (a capacity bound, as ``route_tokens`` returns) nothing is read
-        back from the device: rows past the last group are padding to the GEMMs and come back as zeros."""
+        back from the device: rows past the last group are padding to the GEMMs and come back as zeros.
+        ``row_map`` (``TokenRouting.row_map``: the rows of every token) lets the pass quantise each token once and
+        store it to all its rows instead of once per row; same bits."""
         from cosmos_rl_amd.policy.kernel.moe.indices import permute_quantize_tokens
         rows = row_tokens.numel()
         if rows % ops.BLOCK == 0:
             m_indices = ops.create_indices_from_offsets_nosync(m_offsets, rows, n_experts=m_offsets.numel())
             hidden_size = module.get_parameter("down_proj_weight").shape[1]
             out = torch.zeros((rows, hidden_size), device=tokens.device, dtype=tokens.dtype)
-            return self._run(permute_quantize_tokens(tokens, row_tokens), m_indices, rows, module, tokens.dtype, out=out)
+            return self._run(permute_quantize_tokens(tokens, row_tokens, row_map), m_indices, rows, module, tokens.dtype, out=out)
         total = int(m_offsets[-1])
         m_indices = ops.create_indices_from_offsets_nosync(m_offsets, total)
-        return self._run(permute_quantize_tokens(tokens, row_tokens[:total]), m_indices, total, module, tokens.dtype)
+        # (rows of row_map at or past `total` would be padding; the scatter form skips rows beyond its output)
+        return self._run(permute_quantize_tokens(tokens, row_tokens[:total], row_map), m_indices, total, module, tokens.dtype)
 
     @staticmethod
     def _weights_key(*tensors):

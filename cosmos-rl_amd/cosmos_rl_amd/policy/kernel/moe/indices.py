@@ -66,16 +66,29 @@ def permute_tokens(tokens: torch.Tensor, permuted_indices: torch.Tensor) -> torc
     return out
 
 
-def permute_quantize_tokens(tokens: torch.Tensor, permuted_indices: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+def permute_quantize_tokens(tokens: torch.Tensor, permuted_indices: torch.Tensor,
+                            row_map: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """``groupwise_activation_quant(tokens[permuted_indices])`` (zero rows for -1) in one pass: the 1x128-quantised
     input of the first grouped GEMM (group_gemms.py:188-191) straight from the token matrix, without the gathered
-    bf16 copy.  Returns (fp8 [rows, H], fp32 [rows, ceil(H/128)])."""
+    bf16 copy.  Returns (fp8 [rows, H], fp32 [rows, ceil(H/128)]).
+
+    ``row_map`` (int32 [tokens, topk], the rows each token feeds, -1 for none: ``TokenRouting.row_map``) selects the
+    scatter form, which quantises every token once and stores the result to all of its rows - same bits, an eighth
+    of the reads and of the arithmetic at top-8.  It must describe the same layout as ``permuted_indices``."""
     if not tokens.is_cuda or tokens.dim() != 2 or tokens.stride(1) != 1 or tokens.dtype != torch.bfloat16:
         raise ValueError("expected a 2-D bf16 GPU tensor with unit column stride")
     H = tokens.shape[1]
     idx = permuted_indices.to(torch.int32).contiguous()
     q = torch.empty((idx.numel(), H), dtype=torch.float8_e4m3fn, device=tokens.device)
     s = torch.empty((idx.numel(), (H + 127) // 128), dtype=torch.float32, device=tokens.device)
+    if row_map is not None:
+        if row_map.dim() != 2 or row_map.shape[0] != tokens.shape[0] or row_map.dtype != torch.int32 or not row_map.is_cuda:
+            raise ValueError(f"row_map must be an int32 GPU tensor [tokens, topk], got {tuple(row_map.shape)} {row_map.dtype}")
+        rm = row_map.contiguous()
+        _lib.check(_lib.load().cfp8_scatter_quant_group128(tokens.data_ptr(), tokens.stride(0), tokens.shape[0], H, rm.data_ptr(),
+                                                          rm.shape[1], idx.data_ptr(), idx.numel(), q.data_ptr(), H, s.data_ptr(),
+                                                          _stream()))
+        return q, s
     _lib.check(_lib.load().cfp8_gather_quant_group128(tokens.data_ptr(), tokens.stride(0), idx.data_ptr(), idx.numel(), H,
                                                      q.data_ptr(), H, s.data_ptr(), _stream()))
     return q, s

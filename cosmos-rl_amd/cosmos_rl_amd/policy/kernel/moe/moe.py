@@ -99,7 +99,7 @@ def grouped_experts_forward(x: torch.Tensor, token_mask: Optional[torch.Tensor],
     routing = route_tokens(indices, token_mask, n_experts, alignment)
     if hasattr(strategy, "execute_from_tokens") and x.dtype == torch.bfloat16:
         # the FP8 strategy quantises while it gathers: the expert-grouped bf16 copy of the tokens is never built
-        out = strategy.execute_from_tokens(x, routing.row_tokens, routing.m_sizes, routing.m_offsets, module)
+        out = strategy.execute_from_tokens(x, routing.row_tokens, routing.m_sizes, routing.m_offsets, module, row_map=routing.row_map)
     else:
         contig = permute_tokens(x, routing.row_tokens)
         out = strategy.execute(contig, routing.m_sizes, routing.m_offsets, module)

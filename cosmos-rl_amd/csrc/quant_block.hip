@@ -255,6 +255,80 @@ __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __res
     }
 }
 
+// The gather-and-quantise pass turned round for a token matrix whose rows each feed several rows of the grouped
+// matrix (top-k routing): a token's 1x128 groups are quantised once and the eight bytes a lane holds are stored to
+// every row the token goes to, instead of reading and quantising the token once per destination.  The first
+// blocks_tokens workgroups take the tokens (16 lanes per group of 128 columns, four groups per lane set as in
+// group128_kernel), the rest write the rows of padding: zero bytes and the scale of an all-zero group.
+__global__ __launch_bounds__(256) void scatter_group128_kernel(const uint4* __restrict__ x, int nvec, u32 ngroups, int64_t ldx,
+                                                               u32 tokens, u32 token_groups, const int32_t* __restrict__ row_map,
+                                                               int topk, const int32_t* __restrict__ src_rows, u32 rows_out,
+                                                               uint2* __restrict__ q, int64_t ldq, float* __restrict__ scales,
+                                                               u32 blocks_tokens) {
+    const int sub = threadIdx.x & 15;
+    if (blockIdx.x >= blocks_tokens) {
+        // padding: one lane set per (row, group), four at a time
+        const u32 total = rows_out * ngroups;
+        const u32 g0 = ((blockIdx.x - blocks_tokens) * 16u + (threadIdx.x >> 4)) * 4u;
+        u32 r = g0 / ngroups, c = g0 - r * ngroups;
+        const float floor_scale = scale_from_amax(0.0f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (g0 + i < total && src_rows[r] < 0) {
+                const int vec = (int)c * 16 + sub;
+                if (vec < nvec) q[(int64_t)r * ldq + vec] = make_uint2(0u, 0u);
+                if (sub == 0) scales[(int64_t)r * ngroups + c] = floor_scale;
+            }
+            if (++c == ngroups) c = 0, ++r;
+        }
+        return;
+    }
+    const u32 g0 = (blockIdx.x * 16u + (threadIdx.x >> 4)) * 4u;
+    uint4 v[4];
+    u32 tok[4], gcol[4];
+    bool ok[4];
+    {
+        u32 r = g0 / ngroups, c = g0 - r * ngroups;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            tok[i] = r;
+            gcol[i] = c;
+            if (++c == ngroups) c = 0, ++r;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int vec = (int)gcol[i] * 16 + sub;
+        ok[i] = g0 + i < token_groups && vec < nvec;
+        const u32 rc = tok[i] < tokens ? tok[i] : tokens - 1;
+        const int vc = vec < nvec ? vec : nvec - 1;
+        v[i] = ld16<true>(x + (int64_t)rc * ldx + vc);  // read once: streaming
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (!ok[i]) v[i] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u32 m = row16_max(pk_fold(absmax8(0u, v[i])));
+        const float scale = scale_from_amax(amax_from_bits(m));
+        const Divider d(scale);
+        const uint2 out = cast8(v[i], d);
+        if (g0 + i >= token_groups) continue;
+        const int32_t* const dst = row_map + (int64_t)tok[i] * topk;
+        for (int k0 = 0; k0 < topk; k0 += 8) {
+            int32_t r[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) r[k] = k0 + k < topk ? dst[k0 + k] : -1;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (r[k] < 0 || (u32)r[k] >= rows_out) continue;
+                if (ok[i]) st8<false>(q + (int64_t)r[k] * ldq + gcol[i] * 16 + sub, out);
+                if (sub == 0) scales[(int64_t)r[k] * ngroups + gcol[i]] = scale;
+            }
+        }
+    }
+}
+
 // Groups are numbered in 32 bits, and a block's first group index must not wrap.
 constexpr int64_t kMaxGroups = 0xFFFFFF00ll;
 
@@ -333,6 +407,32 @@ extern "C" int cfp8_gather_quant_group128(const void* x, int64_t ld_x, const int
                        static_cast<hipStream_t>(stream), static_cast<const uint4*>(x), (int)(cols / 8), (u32)ngroups, ld_x / 8,
                        static_cast<uint2*>(q), ld_q / 8, scales, (u32)rows_out, (u32)total, src_rows);
     return check_launch("gather_quant_group128");
+}
+
+extern "C" int cfp8_scatter_quant_group128(const void* x, int64_t ld_x, int64_t tokens, int64_t cols, const int32_t* row_map,
+                                           int64_t topk, const int32_t* src_rows, int64_t rows_out, void* q, int64_t ld_q,
+                                           float* scales, void* stream) {
+    using namespace cfp8;
+    if (tokens < 0 || cols < 0 || rows_out < 0 || topk < 0) return set_error(CFP8_EINVAL, "scatter_quant_group128: negative shape");
+    if (rows_out == 0 || cols == 0) return CFP8_OK;
+    if (!src_rows || !q || !scales || (tokens > 0 && topk > 0 && (!x || !row_map)))
+        return set_error(CFP8_EINVAL, "scatter_quant_group128: null pointer");
+    if (topk > 64) return set_error(CFP8_EINVAL, "scatter_quant_group128: topk=%lld is out of range (0..64)", (long long)topk);
+    if (cols % 8 || ld_x % 8 || ld_q % 8 || ld_x < cols || ld_q < cols)
+        return set_error(CFP8_EINVAL, "scatter_quant_group128: cols=%lld ld_x=%lld ld_q=%lld must be multiples of 8 with ld >= cols",
+                         (long long)cols, (long long)ld_x, (long long)ld_q);
+    if ((x && !aligned16(x)) || (reinterpret_cast<uintptr_t>(q) & 7u)) return set_error(CFP8_EINVAL, "scatter_quant_group128: misaligned pointer");
+    const int64_t ngroups = (cols + 127) / 128;
+    const int64_t token_groups = (topk > 0 ? tokens : 0) * ngroups, row_groups = rows_out * ngroups;
+    if (token_groups > kMaxGroups || row_groups > kMaxGroups || tokens > 0x7FFFFFFFll || rows_out > 0x7FFFFFFFll)
+        return set_error(CFP8_EINVAL, "scatter_quant_group128: too many groups for one launch");
+    const int64_t blocks_tokens = (token_groups + 63) / 64, blocks_rows = (row_groups + 63) / 64;
+    if (blocks_tokens + blocks_rows > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "scatter_quant_group128: too many groups for one launch");
+    if (int rc = check_device()) return rc;
+    hipLaunchKernelGGL(scatter_group128_kernel, dim3((unsigned)(blocks_tokens + blocks_rows)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(x), (int)(cols / 8), (u32)ngroups, ld_x / 8, (u32)tokens, (u32)token_groups, row_map, (int)topk,
+                       src_rows, (u32)rows_out, static_cast<uint2*>(q), ld_q / 8, scales, (u32)blocks_tokens);
+    return check_launch("scatter_quant_group128");
 }
 
 extern "C" int cfp8_swiglu_quant_group128(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, int64_t rows,

@@ -253,6 +253,17 @@ int cfp8_quant_mxfp4(const void* x, int64_t rows, int64_t cols, int64_t ld_x, vo
 int cfp8_gather_quant_group128(const void* x, int64_t ld_x, const int32_t* src_rows, int64_t rows_out, int64_t cols,
                                void* q, int64_t ld_q, float* scales, void* stream);
 
+/* The same result as cfp8_gather_quant_group128, computed from the token side: every row of x (bf16 [tokens, cols])
+ * is quantised once and its bytes and scales are stored to the rows row_map[t, 0 .. topk) of the output (int32, device;
+ * negative or >= rows_out = no row), and the rows r with src_rows[r] < 0 are written as zero rows.  For top-k routing
+ * this reads and quantises a token once instead of once per expert it goes to.  row_map and src_rows must describe
+ * the same layout (src_rows[r] == t exactly for the rows r listed in row_map[t, :]); rows that neither names are
+ * left untouched.  topk <= 64.  Same reference lines as cfp8_gather_quant_group128 (the torch indexing in front of
+ * cosmos_rl/policy/kernel/group_gemms.py:188-191, with the layout cosmos_rl/policy/kernel/moe/moe.py:244-263 implies). */
+int cfp8_scatter_quant_group128(const void* x, int64_t ld_x, int64_t tokens, int64_t cols, const int32_t* row_map,
+                                int64_t topk, const int32_t* src_rows, int64_t rows_out, void* q, int64_t ld_q,
+                                float* scales, void* stream);
+
 /* Block dequantisation y = fp8 * s[i/128, j/128]; out_dtype CFP8_OUT_BF16 or
  * CFP8_OUT_F32.  Replaces weight_dequant at
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */

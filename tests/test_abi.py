@@ -94,6 +94,11 @@ def test_argument_errors_need_no_device():
     assert lib.cfp8_gather_quant_group128(ptr, 60, ptr, 4, 60, ptr, 64, ptr, None) == _lib.EINVAL
     assert lib.cfp8_gather_quant_group128(None, 64, None, 4, 64, None, 64, None, None) == _lib.EINVAL
     assert lib.cfp8_gather_quant_group128(None, 64, None, 0, 64, None, 64, None, None) == 0
+    assert lib.cfp8_scatter_quant_group128(ptr, 64, 4, 60, ptr, 2, ptr, 8, ptr, 64, ptr, None) == _lib.EINVAL      # cols % 8
+    assert lib.cfp8_scatter_quant_group128(ptr, 64, 4, 64, ptr, 65, ptr, 8, ptr, 64, ptr, None) == _lib.EINVAL     # topk
+    assert "topk" in _lib.last_error()
+    assert lib.cfp8_scatter_quant_group128(None, 64, 4, 64, None, 2, ptr, 8, ptr, 64, ptr, None) == _lib.EINVAL
+    assert lib.cfp8_scatter_quant_group128(None, 64, 4, 64, None, 2, None, 0, None, 64, None, None) == 0
     # empty problems succeed without pointers
     assert lib.cfp8_quant_rowwise(None, 0, 16, 16, None, 16, None, None) == 0
     assert lib.cfp8_scaled_mm_rowwise(None, 128, None, None, 128, None, None, 64, 0, 0, 64, 128, None) == 0

@@ -294,3 +294,50 @@ def test_permute_quantize_tokens_is_gather_then_quant(dev, T, H, R):
     xs[idx >= 0] = x[idx[idx >= 0].long()]
     qo, so = O.quant_group128(xs)
     assert torch.equal(q1.view(torch.uint8).cpu(), qo) and torch.equal(s1.cpu().view(torch.int32), so.view(torch.int32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,H,E,K,masked", [(512, 2048, 16, 8, False), (300, 264, 7, 3, True), (64, 128, 40, 12, True), (1000, 7168, 8, 2, False),
+                                            (5, 1024, 4, 1, False)])
+def test_scatter_quantize_equals_gather_quantize(dev, T, H, E, K, masked):
+    """The token-side form (every token quantised once, stored to all its rows) against the row-side form and the
+    oracle: same bytes and scales on every row, padding rows included; untouched where neither index names a row."""
+    from cosmos_rl_amd import _lib
+    from cosmos_rl_amd.policy.kernel.moe.indices import permute_quantize_tokens
+    from cosmos_rl_amd.policy.kernel.moe.moe import route_tokens
+    from oracle import fp8_oracle as O
+    g = torch.Generator().manual_seed(T * 7 + H + K)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    x[T // 2, 3] = 250.0
+    x[0] = 0
+    indices = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    mask = (torch.rand(T, generator=g) > 0.2) if masked else None
+    routing = route_tokens(indices.to(dev), None if mask is None else mask.to(dev), E)
+    xd = torch.zeros(T, H + 16, dtype=torch.bfloat16, device=dev)[:, :H]
+    xd.copy_(x)
+    q1, s1 = permute_quantize_tokens(xd, routing.row_tokens, routing.row_map)
+    q0, s0 = permute_quantize_tokens(xd, routing.row_tokens)
+    assert torch.equal(q1.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(s1.view(torch.int32), s0.view(torch.int32))
+    rt = routing.row_tokens.cpu()
+    xs = torch.zeros(rt.numel(), H, dtype=torch.bfloat16)
+    xs[rt >= 0] = x[rt[rt >= 0].long()]
+    qo, so = O.quant_group128(xs)
+    assert torch.equal(q1.view(torch.uint8).cpu(), qo) and torch.equal(s1.cpu().view(torch.int32), so.view(torch.int32))
+    assert int((rt >= 0).sum()) == (T * K if mask is None else int(mask.sum()) * K)
+    # straight through the C ABI with an output pitch of its own and rows that no index names: they keep their bytes
+    lib = _lib.load()
+    rows = rt.numel()
+    src = routing.row_tokens.clone()
+    rm = routing.row_map.clone()
+    victim = int(torch.nonzero(rt >= 0)[0])                 # drop one routed row from both indices
+    tok = int(rt[victim])
+    rm[tok][rm[tok] == victim] = -1
+    src[victim] = 10 ** 6                                   # neither padding nor listed by its token
+    qb = torch.full((rows, H + 8), 0x5A, dtype=torch.uint8, device=dev)
+    sb = torch.full((rows, (H + 127) // 128), -3.0, device=dev)
+    _lib.check(lib.cfp8_scatter_quant_group128(xd.data_ptr(), xd.stride(0), T, H, rm.data_ptr(), K, src.data_ptr(), rows,
+                                               qb.data_ptr(), H + 8, sb.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    keep = torch.ones(rows, dtype=torch.bool)
+    keep[victim] = False
+    assert torch.equal(qb[:, :H].cpu()[keep], qo[keep]) and torch.equal(sb.cpu().view(torch.int32)[keep], so.view(torch.int32)[keep])
+    assert bool((qb[victim] == 0x5A).all()) and bool((sb[victim] == -3.0).all()) and bool((qb[:, H:] == 0x5A).all())
