@@ -41,6 +41,7 @@ SIGNATURES = {
     "cfp8_quant_rowwise_multi": (c_int, [POINTER(RowwiseDesc), c_int64, c_void_p]),
     "cfp8_quant_tensorwise_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise_multi_static": (c_int, [POINTER(TensorDesc), c_int64, c_void_p]),
+    "cfp8_tensorwise_resident": (c_int, [c_int]),
     "cfp8_tensorwise_amax_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_tensorwise_cast_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),

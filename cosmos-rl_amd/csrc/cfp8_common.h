@@ -148,6 +148,39 @@ __device__ __forceinline__ u32 slow_byte(float x, float s) {
     return cvt2<false>(y, 0.0f, 0u) & 0xFFu;
 }
 
+// cast8 below for a finite scale only
+__device__ __forceinline__ uint2 cast8_finite(const uint4& v, const Divider& d) {
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+    u32 o[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        u32 p = cvt2<false>(d.fast(bf16_lo(w[2 * i])), d.fast(bf16_hi(w[2 * i])), 0u);
+        o[i] = cvt2<true>(d.fast(bf16_lo(w[2 * i + 1])), d.fast(bf16_hi(w[2 * i + 1])), p);
+    }
+    return make_uint2(o[0], o[1]);
+}
+
+// cast8 below for a scale that is +infinity or NaN, in integer arithmetic: x / NaN, NaN / s and inf / inf are NaN
+// (byte 0x7F), a finite x over infinity is a zero with the sign of x
+__device__ __forceinline__ uint2 cast8_nonfinite_scale(const uint4& v, float s) {
+    const bool s_nan = s != s;
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+    u32 o[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        u32 bytes = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const u32 h = (w[2 * i + (e >> 1)] >> ((e & 1) * 16)) & 0xFFFFu;  // bf16 bits
+            const bool x_nonfinite = (h & 0x7F80u) == 0x7F80u;
+            const u32 b = (s_nan || x_nonfinite) ? 0x7Fu : ((h >> 8) & 0x80u);
+            bytes |= b << (8 * e);
+        }
+        o[i] = bytes;
+    }
+    return make_uint2(o[0], o[1]);
+}
+
 // 8 bf16 (one 16-byte vector) -> 8 fp8 bytes (uint2), element order preserved
 __device__ __forceinline__ uint2 cast8(const uint4& v, const Divider& d) {
     const u32 w[4] = {v.x, v.y, v.z, v.w};

@@ -17,6 +17,7 @@
 // The table of tensors travels in the kernel arguments (scalar loads), so the
 // library needs no device-side descriptor buffer.
 
+#include <atomic>
 #include <mutex>
 
 #include "cfp8_common.h"
@@ -26,6 +27,7 @@ namespace cfp8 {
 constexpr int kMaxBatch = 48;
 constexpr int kChunkVecs = 256 * 8;  // 16-byte vectors per workgroup: 32 KiB of bf16
 constexpr int kAmaxSlots = CFP8_TENSORWISE_AMAX_SLOTS;  // one wavefront reads them in one load
+constexpr int kMaxDevices = 64;  // device ordinals with per-device state of their own
 
 struct TensorTable {
     const uint4* x[kMaxBatch];
@@ -123,7 +125,294 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
     }
 }
 
+// ---------------------------------------------------------------------------
+// Both passes in one launch, with the tensor kept on the chip in between (tensors of 106-141 MB: the MLP
+// weights of a 7-8 B model).  One workgroup of twelve waves per CU (three per SIMD, 168 registers each, all of
+// the CU's LDS): a lane keeps kResRegVecs 16-byte vectors in registers and kResLdsVecs in LDS, 256 CUs x 768
+// lanes x 45 x 16 B = 141 MB.  Per tensor every wave loads its 1 KiB chunks (chunk c of the tensor goes to wave
+// c mod waves, so that at any moment the GPU reads one compact window that moves through the tensor),
+// reduces |x|, the workgroup publishes its maximum with one atomic max, the workgroups meet at a counter in
+// device memory, and every wave casts what it holds with the tensor's scale and stores it: 2 B read and 1 B
+// written per element instead of 2 + 2 + 1.  A workgroup that is done storing goes on to load the next tensor
+// while others still store.  Every kept vector has its own registers, hence its own instructions: the code a
+// wave runs per tensor is 30 KB of straight line, shared by the CU's twelve waves and small enough to stay in
+// the instruction cache from one tensor to the next (with one wave per SIMD and all 512 registers it was 350 KB
+// and the kernel spent its time fetching it).
+// The wait at the counter is bounded by the wall clock, so every wave leaves the kernel whatever happens; a
+// workgroup that gives up poisons the tensor's scale and bytes with NaN.  The launch needs all its workgroups
+// resident at once: the grid is one workgroup per CU and a workgroup takes a whole CU, so on a GPU that no
+// other grid holds they are.  Two such launches on different streams of one GPU could each hold part of the
+// CUs and wait for the rest until the bound expires: callers that run this path from several streams at once
+// switch it off (cfp8_tensorwise_resident).
+// ---------------------------------------------------------------------------
+static std::atomic<int> g_resident_enabled{1};
+
+constexpr int kResWaves = 12;     // per workgroup
+constexpr int kResRegVecs = 32;
+constexpr int kResLdsVecs = 13;
+constexpr int kResVecs = kResRegVecs + kResLdsVecs;
+static_assert(kResLdsVecs <= kResRegVecs, "the LDS part passes through registers");
+constexpr size_t kResLdsBytes = (size_t)kResWaves * kResLdsVecs * 64 * 16 + 64;
+static_assert(kResLdsBytes <= 160 * 1024, "LDS of one CU");
+
+struct ResidentTable {
+    const uint4* x[kMaxBatch];
+    uint2* q[kMaxBatch];
+    float* scale[kMaxBatch];
+    unsigned nchunks[kMaxBatch];  // 64-vector chunks (the tensor is a whole number of them)
+    u32* amax[kMaxBatch];         // slot 0: arrival counter, slots 1 .. 63: maxima of the workgroups
+    int n;
+    unsigned wait_ticks;  // bound of the wait at the counter, in ticks of the 100 MHz wall clock
+};
+
+// atomic max that has been performed when the function returns (the wave waits for the value it returns)
+__device__ __forceinline__ void publish_max(u32* slot, u32 bits) {
+    const u32 old = __hip_atomic_fetch_max(slot, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("" ::"v"(old));
+}
+
+__global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tensorwise_resident_kernel(const ResidentTable tb) {
+    extern __shared__ __attribute__((aligned(16))) uint4 res_lds[];  // [waves][kResLdsVecs][64 lanes], then the give-up flag
+    u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);
+    u32* const red = gave_up + 1;  // [kResWaves]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned gw = blockIdx.x * (unsigned)kResWaves + (unsigned)wave;
+    const unsigned nw = gridDim.x * (unsigned)kResWaves;
+    uint4* const my_lds = res_lds + wave * (kResLdsVecs * 64) + lane;
+    if (threadIdx.x == 0) *gave_up = 0u;
+    // Chunk i of the wave is chunk gw + i * nw of the tensor: at any moment the waves of the whole GPU read one compact
+    // window that moves through the tensor, as a streaming kernel's workgroups do.  Every wave issues the same loads
+    // and stores whatever its share: slots past its last chunk repeat that chunk (a wave without any repeats a chunk
+    // of another wave), which changes neither the maximum nor a stored byte - branches around the loads would make
+    // the compiler wait for every load in flight at each use of one.
+    // Addresses are a scalar base (the tensor), a scalar offset (the slot's chunk) and one per-lane offset that is the
+    // same for every slot of a tensor: buffer loads and stores, so that no slot needs address registers of its own.
+    struct Geo {
+        u32 lane_vec;  // vector index of the wave's chunk 0, plus the lane
+        int lastc;     // index of the wave's last chunk
+    };
+    auto geo = [&](int t) {
+        const unsigned nchunks = tb.nchunks[t];
+        const int cnt = nchunks > gw ? (int)((nchunks - gw + nw - 1) / nw) : 0;
+        const unsigned cb = gw < nchunks ? gw : gw % nchunks;
+        return Geo{cb * 64u + (u32)lane, cnt > 0 ? cnt - 1 : 0};
+    };
+    const u32 stride = nw * 64u;  // vectors between two chunks of a wave
+    auto slot_vec = [&](const Geo& g, int i) { return (u32)(i < g.lastc ? i : g.lastc) * stride; };  // scalar
+    auto load = [&](__amdgpu_buffer_rsrc_t rx, const Geo& g, int i) {  // streaming 16-byte load of the wave's chunk i
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, g.lane_vec * 16u, slot_vec(g, i) * 16u, 2);
+        return make_uint4(v[0], v[1], v[2], v[3]);
+    };
+    auto store = [&](__amdgpu_buffer_rsrc_t rq, const Geo& g, int i, uint2 o) {
+        u32x2 v;
+        v[0] = o.x;
+        v[1] = o.y;
+        __builtin_amdgcn_raw_buffer_store_b64(v, rq, g.lane_vec * 8u, slot_vec(g, i) * 8u, 2);
+    };
+    auto rsrc = [&](const void* base) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xFFFFFFFF, 0x00020000);
+    };
+    // Chunks 0 .. kResLdsVecs - 1 of the wave live in LDS and pass through the first register slots; chunk
+    // kResLdsVecs + r lives in register slot r.
+    uint4 keep[kResRegVecs];
+    for (int t = 0; t < tb.n; ++t) {
+        const Geo g = geo(t);
+        // ---- pass 1: kResDepth loads in flight per wave, issued in chunk order, straight into the registers that
+        // keep them
+        {
+            constexpr int kResDepth = 8;
+            const __amdgpu_buffer_rsrc_t rx = rsrc(tb.x[t]);
+            u32 m = 0;
+#pragma unroll
+            for (int l = 0; l < kResDepth; ++l) keep[l] = load(rx, g, l);
+#pragma unroll
+            for (int l = 0; l < kResLdsVecs; ++l) {
+                m = absmax8(m, keep[l]);
+                my_lds[l * 64] = keep[l];
+                if (l + kResDepth < kResLdsVecs) keep[l + kResDepth] = load(rx, g, l + kResDepth);
+            }
+#pragma unroll
+            for (int r = 0; r < kResDepth; ++r) keep[r] = load(rx, g, kResLdsVecs + r);
+#pragma unroll
+            for (int r = 0; r < kResRegVecs; ++r) {
+                m = absmax8(m, keep[r]);
+                if (r + kResDepth < kResRegVecs) keep[r + kResDepth] = load(rx, g, kResLdsVecs + r + kResDepth);
+            }
+            const u32 w = wave_max(pk_fold(m));
+            if (lane == 0) red[wave] = w;
+        }
+        // ---- the workgroup's maximum goes to one of the tensor's slots 1 .. 63 with one atomic (thousands of atomics on
+        // one address serialise at the memory side: one per wave cost 30 us per tensor); slot 0 counts the workgroups
+        // that have done so.  A workgroup is counted once its atomic max has been performed (thread 0 has waited for
+        // the value it returns); counter and maxima are only ever touched by device-scope atomics, which act at the
+        // memory side of the XCDs' L2s, so no cache needs writing back or invalidating here (a release or acquire
+        // fence at device scope does both, tens of microseconds each).
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            u32 w = 0;
+#pragma unroll
+            for (int k = 0; k < kResWaves; ++k) w = umax(w, red[k]);
+            if (w) publish_max(tb.amax[t] + 1 + blockIdx.x % (kAmaxSlots - 1), w << 16);  // fp32 bit pattern
+            u32* const counter = tb.amax[t];
+            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t since = __builtin_amdgcn_s_memrealtime();
+            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x) {
+                if (__builtin_amdgcn_s_memrealtime() - since > (uint64_t)tb.wait_ticks) {
+                    *gave_up = 1u;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+        }
+        __syncthreads();
+        // ---- pass 2: cast what is held and store it
+        static_assert(kAmaxSlots == 64, "one slot per lane");
+        const float amax = __uint_as_float(wave_max(lane ? __hip_atomic_load(tb.amax[t] + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u));
+        const float scale = *gave_up != 0u ? __uint_as_float(kCanonNaN) : scale_from_amax(amax);
+        if (gw == 0 && lane == 0) *tb.scale[t] = scale;
+        const Divider d(scale);
+        const __amdgpu_buffer_rsrc_t rq = rsrc(tb.q[t]);
+        // (slots past the wave's last chunk hold copies of it: skipped here, where a branch costs nothing - a wave with
+        // no chunk of its own stores the one it copied once more, the same bytes)
+        if (d.finite) {  // (one branch per tensor: the code of the other case is never fetched)
+#pragma unroll
+            for (int l = 0; l < kResLdsVecs; ++l)
+                if (l <= g.lastc) store(rq, g, l, cast8_finite(my_lds[l * 64], d));
+#pragma unroll
+            for (int r = 0; r < kResRegVecs; ++r)
+                if (kResLdsVecs + r <= g.lastc) store(rq, g, kResLdsVecs + r, cast8_finite(keep[r], d));
+        } else {
+#pragma unroll
+            for (int l = 0; l < kResLdsVecs; ++l)
+                if (l <= g.lastc) store(rq, g, l, cast8_nonfinite_scale(my_lds[l * 64], scale));
+#pragma unroll
+            for (int r = 0; r < kResRegVecs; ++r)
+                if (kResLdsVecs + r <= g.lastc) store(rq, g, kResLdsVecs + r, cast8_nonfinite_scale(keep[r], scale));
+        }
+    }
+}
+
 enum : int { kPhaseAmax = 1, kPhaseCast = 2 };
+
+// Which tensors of a call a helper below takes: all of them, those that take the resident kernel, or the others.
+enum : int { kTakeAll = 0, kTakeResident = 1, kTakeOthers = 2 };
+static bool resident_fits(const cfp8_tensor_desc& d, int cus);
+static inline bool taken(const cfp8_tensor_desc& d, int take, int cus) {
+    return take == kTakeAll || resident_fits(d, cus) == (take == kTakeResident);
+}
+
+// pass 1 and / or pass 2 as launches of their own over the tensors of the call that `take` selects
+static void two_pass(const cfp8_tensor_desc* descs, int64_t n, u32* slots, int phases, int take, int cus, hipStream_t st) {
+    // Tensors are taken in batches of at most kMaxBatch entries; with both phases requested each
+    // batch runs pass 1 then pass 2 back to back.  Every access streams past the caches (non-temporal
+    // loads in both passes, non-temporal stores).  Measured on MI355X: few large launches with
+    // streaming accesses beat small batches that would let pass 2 hit the 256 MiB memory-side cache,
+    // because every launch pays a ramp-up and a tail.
+    int64_t i = 0;
+    while (i < n) {
+        // the tensors of this batch: at most kMaxBatch, and few enough chunks for one grid
+        int64_t idx[kMaxBatch];
+        uint64_t chunks = 0;
+        int count = 0;
+        while (i < n && count < kMaxBatch) {
+            if (!taken(descs[i], take, cus)) {
+                ++i;
+                continue;
+            }
+            uint64_t nc = (uint64_t)((descs[i].numel / 8 + kChunkVecs - 1) / kChunkVecs);
+            if (nc == 0) nc = 1;  // a tensor with no element still owns one workgroup: it writes the scale
+            if (count > 0 && chunks + nc > 0x7FFFFFFFull) break;
+            chunks += nc;
+            idx[count++] = i++;
+        }
+        if (count == 0) break;
+        // pass 1 gives a workgroup `per` chunks, pass 2 one: two tables that differ in the workgroup prefix
+        for (int phase = kPhaseAmax; phase <= kPhaseCast; phase <<= 1) {
+            if (!(phases & phase)) continue;
+            TensorTable tb;
+            tb.n = count;
+            tb.per = phase == kPhaseAmax ? amax_chunks_per_block(chunks) : 1;
+            unsigned blocks = 0;
+            for (int k = 0; k < count; ++k) {
+                const cfp8_tensor_desc& d = descs[idx[k]];
+                const int64_t nvec = d.numel / 8;
+                uint64_t nc = (uint64_t)((nvec + kChunkVecs - 1) / kChunkVecs);
+                if (nc == 0) nc = 1;
+                tb.x[k] = static_cast<const uint4*>(d.x);
+                tb.q[k] = static_cast<uint2*>(d.q);
+                tb.scale[k] = d.scale;
+                tb.nvec[k] = nvec;
+                tb.amax[k] = slots + idx[k] * kAmaxSlots;
+                tb.first_block[k] = blocks;
+                blocks += (unsigned)((nc + tb.per - 1) / tb.per);
+            }
+            tb.first_block[count] = blocks;
+            if (phase == kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
+            else hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
+        }
+    }
+}
+
+// ---- the resident form: host side ---------------------------------------------------------------
+static int resident_cus() {  // compute units of the current device, 0 if unknown
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int c = cached[dev].load(std::memory_order_relaxed);
+    if (c > 0) return c;
+    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    static std::atomic<bool> raised[kMaxDevices];
+    if (!raised[dev].load(std::memory_order_acquire)) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(tensorwise_resident_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)kResLdsBytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        raised[dev].store(true, std::memory_order_release);
+    }
+    cached[dev].store(c, std::memory_order_relaxed);
+    return c;
+}
+
+// A tensor takes the resident kernel if it is a whole number of 1 KiB chunks, fits the chip, and fills at least three
+// quarters of it: a tensor costs the resident kernel about 12 us plus 0.52 us per million elements (every wave walks
+// all its slots and the workgroups meet in the middle), the two launches 0.82 us per million, level at 50 million.
+static bool resident_fits(const cfp8_tensor_desc& d, int cus) {
+    const uint64_t cap = (uint64_t)cus * kResWaves * kResVecs, nc = (uint64_t)(d.numel / 512);
+    return d.numel % 512 == 0 && nc <= cap && nc * 4 >= cap * 3;
+}
+
+// The tensors of the call that take the resident kernel, kMaxBatch per launch
+static void resident_all(const cfp8_tensor_desc* descs, int64_t n, u32* slots, int cus, hipStream_t st) {
+    int64_t i = 0;
+    while (i < n) {
+        ResidentTable tb;
+        int count = 0;
+        for (; i < n && count < kMaxBatch; ++i) {
+            const cfp8_tensor_desc& d = descs[i];
+            if (!resident_fits(d, cus)) continue;
+            tb.x[count] = static_cast<const uint4*>(d.x);
+            tb.q[count] = static_cast<uint2*>(d.q);
+            tb.scale[count] = d.scale;
+            tb.nchunks[count] = (unsigned)(d.numel / 512);
+            tb.amax[count] = slots + i * kAmaxSlots;
+            ++count;
+        }
+        if (count == 0) break;
+        tb.n = count;
+        tb.wait_ticks = 100u * 1000u * 1000u;  // one second of the 100 MHz clock
+        // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
+        // GPU that no other grid holds they are
+        hipLaunchKernelGGL(tensorwise_resident_kernel, dim3((unsigned)cus), dim3(kResWaves * 64), kResLdsBytes, st, tb);
+    }
+}
 
 static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream, int phases) {
     if (n < 0 || n > (1ll << 24)) return set_error(CFP8_EINVAL, "quant_tensorwise: bad tensor count");
@@ -146,50 +435,17 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
         const int64_t per = 64 * 1024;
         hipLaunchKernelGGL(tensorwise_zero_kernel, dim3((unsigned)((total + per - 1) / per)), dim3(64), 0, st, slots, total);
     }
-    // Tensors are taken in batches of at most kMaxBatch entries; with both phases requested each
-    // batch runs pass 1 then pass 2 back to back.  Every access streams past the caches (non-temporal
-    // loads in both passes, non-temporal stores).  Measured on MI355X: few large launches with
-    // streaming accesses beat small batches that would let pass 2 hit the 256 MiB memory-side cache,
-    // because every launch pays a ramp-up and a tail.
-    int64_t i = 0;
-    while (i < n) {
-        // the tensors of this batch: at most kMaxBatch, and few enough chunks for one grid
-        const int64_t first = i;
-        uint64_t chunks = 0;
-        int count = 0;
-        while (i < n && count < kMaxBatch) {
-            uint64_t nc = (uint64_t)((descs[i].numel / 8 + kChunkVecs - 1) / kChunkVecs);
-            if (nc == 0) nc = 1;  // a tensor with no element still owns one workgroup: it writes the scale
-            if (count > 0 && chunks + nc > 0x7FFFFFFFull) break;
-            chunks += nc;
-            ++count;
-            ++i;
-        }
-        // pass 1 gives a workgroup `per` chunks, pass 2 one: two tables that differ in the workgroup prefix
-        for (int phase = kPhaseAmax; phase <= kPhaseCast; phase <<= 1) {
-            if (!(phases & phase)) continue;
-            TensorTable tb;
-            tb.n = count;
-            tb.per = phase == kPhaseAmax ? amax_chunks_per_block(chunks) : 1;
-            unsigned blocks = 0;
-            for (int k = 0; k < count; ++k) {
-                const cfp8_tensor_desc& d = descs[first + k];
-                const int64_t nvec = d.numel / 8;
-                uint64_t nc = (uint64_t)((nvec + kChunkVecs - 1) / kChunkVecs);
-                if (nc == 0) nc = 1;
-                tb.x[k] = static_cast<const uint4*>(d.x);
-                tb.q[k] = static_cast<uint2*>(d.q);
-                tb.scale[k] = d.scale;
-                tb.nvec[k] = nvec;
-                tb.amax[k] = slots + (first + k) * kAmaxSlots;
-                tb.first_block[k] = blocks;
-                blocks += (unsigned)((nc + tb.per - 1) / tb.per);
-            }
-            tb.first_block[count] = blocks;
-            if (phase == kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
-            else hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
-        }
+    // Both passes requested: tensors that fit the chip (registers + LDS of all CUs) take the resident kernel, which
+    // reads them once; the others take pass 1 and pass 2 as launches of their own.
+    int cus = 0;
+    if (phases == (kPhaseAmax | kPhaseCast) && g_resident_enabled.load(std::memory_order_relaxed)) cus = resident_cus();
+    if (cus <= 0) {
+        two_pass(descs, n, slots, phases, kTakeAll, 0, st);
+        return check_launch("quant_tensorwise");
     }
+    // (the order in which tensors are quantised is free: the large ones first, then the rest in full batches)
+    resident_all(descs, n, slots, cus, st);
+    two_pass(descs, n, slots, phases, kTakeOthers, cus, st);
     return check_launch("quant_tensorwise");
 }
 
@@ -200,7 +456,6 @@ static int run_tensorwise(const cfp8_tensor_desc* descs, int64_t n, float* amax_
 constexpr int kStaticMaxTensors = CFP8_TENSORWISE_STATIC_MAX_TENSORS;
 static __device__ __align__(256) u32 scratch[kStaticMaxTensors * kAmaxSlots];
 
-constexpr int kMaxDevices = 64;
 static u32* g_static_slots[kMaxDevices];  // guarded by g_static_mutex; null until looked up
 static std::mutex g_static_mutex;
 
@@ -244,6 +499,11 @@ extern "C" int cfp8_quant_tensorwise_multi_static(const cfp8_tensor_desc* descs,
     if (int rc = static_slots(&slots)) return rc;
     // the amax phase clears the n * kAmaxSlots slots it uses with a fill kernel before pass 1
     return run_tensorwise(descs, n, reinterpret_cast<float*>(slots), stream, kPhaseAmax | kPhaseCast);
+}
+
+extern "C" int cfp8_tensorwise_resident(int enable) {
+    if (enable < 0) return cfp8::g_resident_enabled.load(std::memory_order_relaxed);
+    return cfp8::g_resident_enabled.exchange(enable ? 1 : 0, std::memory_order_relaxed);
 }
 
 extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {

@@ -100,7 +100,12 @@ int cfp8_quant_rowwise_multi(const cfp8_rowwise_desc* descs, int64_t n, void* st
  * cosmos_rl/utils/fp8/fp8_util.py:121-137 (hp_tensor_to_float8_dynamic).
  * The descriptor array lives in HOST memory; amax_ws is a device array of
  * n * CFP8_TENSORWISE_AMAX_SLOTS floats (scratch, overwritten).
- * numel % 8 == 0 for every tensor. */
+ * numel % 8 == 0 for every tensor.
+ * Tensors that fill three quarters or more of the GPU's registers and LDS and still fit (106-141 MB of
+ * bf16 on a 256-CU MI355X, numel % 512 == 0: the MLP weights of a 7-8 B model) are read once: one
+ * launch of one workgroup per CU keeps them on the chip between the two passes, the workgroups meeting
+ * at a counter in amax_ws in between.  That launch wants the GPU to itself - see cfp8_tensorwise_resident.
+ * The order in which the tensors of a call are quantised is unspecified; the results do not depend on it. */
 #define CFP8_TENSORWISE_AMAX_SLOTS 64
 typedef struct cfp8_tensor_desc {
     const void* x;   /* bf16, contiguous, 16-byte aligned */
@@ -111,6 +116,14 @@ typedef struct cfp8_tensor_desc {
 
 int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
                                 float* amax_ws, void* stream);
+
+/* Switch for the read-once form of cfp8_quant_tensorwise_multi (and _multi_static): enable != 0 allows it
+ * (the default), 0 makes every tensor take the two separate passes, a negative value only queries.  Returns
+ * the previous setting.  The read-once launch needs all its workgroups on the GPU at the same time, one per
+ * CU; two of them issued on different streams of one GPU can each hold part of the CUs and wait for the
+ * rest until a one-second bound expires and the affected tensors come out as NaN.  A process that
+ * quantises from several streams at once switches it off.  No counterpart in the reference. */
+int cfp8_tensorwise_resident(int enable);
 
 /* Split-phase forms of the above.  Pass 1 alone leaves partial maxima of |x| of
  * tensor i in amax_ws[i*SLOTS .. i*SLOTS+SLOTS-1] (non-negative fp32 bit

@@ -85,6 +85,23 @@ def test_graph_batch_quantisers_without_allocation(dev):
         assert torch.equal(q.view(torch.uint8), q1.view(torch.uint8)) and torch.equal(sc, s1)
 
 
+def test_graph_tensorwise_read_once_launch(dev):
+    """A tensor large enough for the launch that keeps it on the chip between the passes (its workgroups meet at a
+    counter in device memory, cleared by the fill kernel in front of it), captured together with a small one."""
+    shapes = [(18944, 3584), (300, 256)]
+    qt = [torch.empty(sh, dtype=torch.float8_e4m3fn, device=dev) for sh in shapes]
+    st = torch.empty(len(shapes), dtype=torch.float32, device=dev)
+
+    def inputs(seed):
+        return [_bf16(dev, seed + 10 * i, *sh, std=0.02 * (i + 1)) for i, sh in enumerate(shapes)]
+
+    def fn(*ws):
+        ops.quant_tensorwise_multi_static(list(ws), qt, st)
+        return (*qt, st)
+
+    _replay_matches_eager(dev, inputs, fn)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 3584), (64, 2048, 3584), (48, 1024, 7168), (1024, 2048, 3584), (2304, 8448, 256)])
 def test_graph_fp8_linear(dev, M, N, K):
     """single-token and 64-token kernels, the split-K pair of launches, 256x256 tiles, and the head + tail pair"""

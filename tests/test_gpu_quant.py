@@ -289,6 +289,62 @@ def test_tensorwise_edges(dev):
     assert_scales(s, so, "per-tensor scale"); assert_bytes(q, qo, "per-tensor bytes")
 
 
+def _two_pass(tensors, dev):
+    """The split-phase entry points in sequence: always the two separate launches."""
+    n = len(tensors)
+    qs = [torch.empty(t.shape, dtype=torch.float8_e4m3fn, device=dev) for t in tensors]
+    sc = torch.empty(n, dtype=torch.float32, device=dev)
+    ws = torch.empty(n * _lib.TENSORWISE_AMAX_SLOTS, dtype=torch.float32, device=dev)
+    d = (_lib.TensorDesc * n)()
+    for i, (t, q) in enumerate(zip(tensors, qs)):
+        d[i].x, d[i].q, d[i].scale, d[i].numel = t.data_ptr(), q.data_ptr(), sc.data_ptr() + 4 * i, t.numel()
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(_lib.load().cfp8_tensorwise_amax_multi(d, n, ws.data_ptr(), st))
+    _lib.check(_lib.load().cfp8_tensorwise_cast_multi(d, n, ws.data_ptr(), st))
+    return qs, sc
+
+
+def test_tensorwise_read_once_launch(dev):
+    """Tensors large enough for the launch that keeps them on the chip between the passes (106-141 MB), mixed
+    with smaller ones in one call: against the oracle, against the two separate passes, twice in a row, with a
+    NaN and an infinity (the scale is then not finite and the bytes take the integer path), through the entry
+    point that allocates nothing, and with the launch switched off."""
+    lib = _lib.load()
+    assert lib.cfp8_tensorwise_resident(-1) == 1
+    g = torch.Generator(device=dev).manual_seed(77)
+    shapes = [(18944, 3584), (512, 3584), (14336, 4096), (3584, 3584), (3584, 18944), (13568, 4096), (17280, 4096)]
+    ws = [(torch.randn(sh, generator=g, device=dev) * (0.01 * (i + 1))).to(torch.bfloat16) for i, sh in enumerate(shapes)]
+    ws[2][7000, 123] = float("inf")          # non-finite scale in a tensor that is kept on the chip
+    ws[4][11, 18000] = float("nan")
+    ws[5].zero_()                             # amax 0: the scale floor
+    ws[6][17279, 4095] = 300.0               # exactly the capacity of 256 CUs; the maximum in the last element of the last chunk
+    qs, scales = ops.quant_tensorwise_multi(ws)
+    q2, s2 = _two_pass(ws, dev)
+    for i in range(len(ws)):
+        assert torch.equal(u8(qs[i]), u8(q2[i])), f"tensor {i}: bytes differ from the two separate passes"
+    assert torch.equal(bits(scales), bits(s2))
+    for i in (0, 2, 4, 5, 6):                 # the oracle on the CPU: a second or two per tensor of this size
+        qo, so = O.quant_tensorwise(ws[i].cpu())
+        assert_scales(scales[i:i + 1], so, f"tensor {i} scale")
+        assert_bytes(qs[i], qo, f"tensor {i} bytes")
+    assert int(bits(scales)[5]) == 0x2720D7C5 and int(u8(qs[5]).max()) == 0
+    # the counters and maxima live in the workspace of the call: a second call starts from zero again
+    qs_b, scales_b = ops.quant_tensorwise_multi(ws)
+    assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, qs_b)) and torch.equal(bits(scales), bits(scales_b))
+    # the library's own slots
+    outs = [torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=dev) for w in ws]
+    sc = torch.empty(len(ws), dtype=torch.float32, device=dev)
+    ops.quant_tensorwise_multi_static(ws, outs, sc)
+    assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, outs)) and torch.equal(bits(scales), bits(sc))
+    # switched off: every tensor takes the two separate passes; same results
+    assert lib.cfp8_tensorwise_resident(0) == 1
+    try:
+        qs_c, scales_c = ops.quant_tensorwise_multi(ws)
+    finally:
+        assert lib.cfp8_tensorwise_resident(1) == 0
+    assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, qs_c)) and torch.equal(bits(scales), bits(scales_c))
+
+
 def test_tensorwise_full_size_properties(dev):
     """lm_head-sized tensor [152064, 3584] on the GPU only: scale equals the closed form of the
     torch amax, the set holds +-448, and the bytes equal a rowwise-kernel-free recomputation on a
