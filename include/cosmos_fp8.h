@@ -122,7 +122,8 @@ int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
  * the previous setting.  The read-once launch needs all its workgroups on the GPU at the same time, one per
  * CU; two of them issued on different streams of one GPU can each hold part of the CUs and wait for the
  * rest until a one-second bound expires and the affected tensors come out as NaN.  A process that
- * quantises from several streams at once switches it off.  No counterpart in the reference. */
+ * quantises from several streams at once, or that runs with part of the CUs masked off, switches it off.
+ * No counterpart in the reference. */
 int cfp8_tensorwise_resident(int enable);
 
 /* Split-phase forms of the above.  Pass 1 alone leaves partial maxima of |x| of
