@@ -18,7 +18,7 @@ LIB_DIR = PKG_DIR / "lib"
 LIB_PATH = LIB_DIR / "libcosmosfp8.so"
 OBJ_DIR = CSRC_DIR / "build"
 
-SOURCES = ["api.hip", "quant_rowwise.hip", "quant_tensorwise.hip", "quant_block.hip", "gemm_fp8.hip", "moe_indices.hip", "quant_mxfp4.hip"]
+SOURCES = ["api.hip", "quant_rowwise.hip", "quant_tensorwise.hip", "quant_block.hip", "gemm_fp8.hip", "moe_indices.hip", "quant_mxfp4.hip", "gemm_mxfp4.hip"]
 
 # -packed-fp32-ops: hipcc must not form v_pk_{add,mul,fma}_f32 (they have returned
 # wrong results on some machines).  -ffp-contract=off: the quantisers rely on

@@ -323,6 +323,56 @@ def quant_mxfp4(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+def gemm_mxfp4(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Tensor, torch.Tensor],
+               out_dtype: torch.dtype = torch.bfloat16, m_indices: Optional[torch.Tensor] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Product of per-token FP8 activations with MXFP4 weights as ``quant_mxfp4`` (``quantize_mx4``,
+    monkey_patch_for_mxfp4.py:18-24) writes them.  lhs = (fp8 [M, K], fp32 [M] or [M, 1]); rhs = (uint8 [N, K/2],
+    uint8 [N, K/32]) or, with ``m_indices`` (int32 [M], groups contiguous and 128-row aligned, negative =
+    padding, rows left untouched), ([E, N, K/2], [E, N, K/32]).  K % 32 == 0, N % 16 == 0."""
+    a, sa = lhs
+    w, ws = rhs
+    _need_gpu(a, sa, w, ws)
+    if a.dim() != 2 or a.dtype != FP8_DTYPE or w.dtype != torch.uint8 or ws.dtype != torch.uint8:
+        raise ValueError("expected fp8 [M, K] activations and uint8 weight codes / scales")
+    M, K = a.shape
+    grouped = m_indices is not None
+    if w.dim() != (3 if grouped else 2):
+        raise ValueError("weights must be [N, K/2] (or [E, N, K/2] with m_indices)")
+    E = w.shape[0] if grouped else 1
+    N = w.shape[-2]
+    if K % 32 or w.shape[-1] != K // 2 or tuple(ws.shape) != (*w.shape[:-1], K // 32) or sa.numel() != M:
+        raise ValueError("shape mismatch in MXFP4 GEMM")
+    if sa.dtype != torch.float32:
+        raise ValueError("activation scales must be fp32")
+    a, sa, w, ws = a.contiguous(), sa.contiguous(), w.contiguous(), ws.contiguous()
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (M, N) or not out.is_contiguous():
+        raise ValueError("out must be a contiguous [M, N] tensor")
+    mi = 0
+    if grouped:
+        _need_gpu(m_indices)
+        if m_indices.numel() != M:
+            raise ValueError("m_indices must have one entry per row")
+        m_indices = m_indices.to(torch.int32).contiguous()
+        mi = m_indices.data_ptr()
+    _lib.check(_lib.load().cfp8_gemm_mxfp4(a.data_ptr(), K, sa.data_ptr(), w.data_ptr(), K // 2, ws.data_ptr(), K // 32,
+                                          mi, E if grouped else 0, out.data_ptr(), N, _out_code(out.dtype), M, N, K, _stream()))
+    return out
+
+
+def linear_mxfp4(x: torch.Tensor, weight: Tuple[torch.Tensor, torch.Tensor],
+                 out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x [..., K] bf16 times MXFP4 weights (codes [N, K/2], scales [N, K/32]): per-token dynamic FP8
+    quantisation of x (as in ``fp8_linear``) followed by ``gemm_mxfp4``."""
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    q, s = quant_rowwise(x2)
+    y = gemm_mxfp4((q, s), weight, out_dtype or x.dtype)
+    return y.reshape(*x.shape[:-1], y.shape[-1])
+
+
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """``per_token_cast_to_fp8`` of the reference's tests/test_deepep.py:75-85, including its
     formula ``x * (448 / amax.clamp(1e-4))`` with scales ``amax / 448``."""

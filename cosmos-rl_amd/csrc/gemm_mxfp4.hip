@@ -1,0 +1,308 @@
+// GEMM of FP8 activations with MXFP4 weights on the gfx950 matrix cores.
+//
+//   out[m, n] = sa[m] * sum_k x[m, k] * (e2m1(w[n, k]) * 2^(ws[n, k / 32] - 127))
+//
+// x is e4m3 [M, K] with one fp32 scale per row (the rowwise activation quantiser), w holds two e2m1 codes per
+// byte (even k in the low nibble) with one e8m0 scale byte per 32 consecutive k, the format cfp8_quant_mxfp4
+// writes.  v_mfma_scale_f32_16x16x128_f8f6f4 takes the two operands in different formats and applies the
+// power-of-two block scales itself: lane l of the "A" operand supplies row l & 15, the 32 k of quarter l >> 4
+// (16 bytes of e2m1) and the scale byte of exactly that row and quarter, so an MXFP4 block is one lane's
+// share of one instruction and no scale arithmetic is left for the vector ALU.  The activation side passes
+// the scale byte 127 (2^0); its fp32 row scale multiplies the accumulator once in the epilogue.
+// The two formats number k differently inside the 128 of one instruction (found with one-hot operands and
+// pinned by the one-hot test): an e2m1 lane's 32 codes are k = 32 q .. 32 q + 31, an e4m3 lane's registers
+// 0-3 are k = 16 q .. 16 q + 15 and its registers 4-7 are k = 64 + 16 q .. 64 + 16 q + 15 (q = l >> 4).
+// As in the FP8 kernels the weight tile is the MFMA "A" operand, so a lane's four accumulators are four
+// consecutive n of one output row.
+//
+// Tiles: BM x BN x 128 per workgroup, two LDS stages filled through registers.  An activation stage is the
+// chunk-major layout of the FP8 kernels (16-row blocks of 2 KiB).  A weight stage holds 64 bytes per row:
+// 16-row blocks of 1 KiB, the 16-byte chunk c (0..3) of row r at c * 256 + ((r ^ (c << 2)) & 15) * 16, so that
+// a fragment read (16 lanes = 16 rows of one chunk) and a staging store (16 lanes = 4 rows x 4 chunks) each
+// cover all 64 banks once.  The scale bytes of a stage are kept as one 32-bit word per (quarter, wave
+// column, row of the MFMA tile) whose byte i belongs to the wave's i-th 16-row tile: one LDS read per lane
+// and K step, the byte is picked by the instruction's op_sel.
+// K need not be a multiple of 128: the chunks of the last step that lie beyond K are loaded as zero with the
+// scale byte 127.
+#include "cfp8_common.h"
+
+namespace cfp8 {
+
+struct Mx4Args {
+    const uint8_t* a;    // activations e4m3 [M, K]
+    const uint8_t* w;    // weights, packed e2m1 [G, N, K / 2]
+    const uint8_t* ws;   // weight scales e8m0 [G, N, K / 32]
+    const float* sa;     // [M]
+    const int32_t* m_indices;  // [M] or null
+    void* out;
+    int64_t ld_a, ld_w, ld_ws, ld_out;
+    int M, N, K;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ int x_chunk_offset(int row, int c) {
+    return ((row >> 4) << 11) + (c << 8) + ((((row & 15) ^ ((c & 1) << 3))) << 4);
+}
+__device__ __forceinline__ int w_chunk_offset(int row, int c) {
+    return ((row >> 4) << 10) + (c << 8) + ((((row & 15) ^ (c << 2)) & 15) << 4);
+}
+
+// workgroup id -> tile: every XCD (workgroup ids are dealt to the 8 XCDs round robin) takes a contiguous
+// range of tiles, walked in bands of GM tile-rows, so that co-resident workgroups share operand rows in L2
+template <int GM>
+__device__ __forceinline__ void mx4_tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    const int lin = xcd * base + (xcd < rem ? xcd : rem) + local;
+    const int band = GM * tiles_n;
+    const int g = lin / band, first = g * GM;
+    const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;
+    const int in = lin - g * band;
+    tm = first + in % gsz;
+    tn = in / gsz;
+}
+
+template <int I>
+__device__ __forceinline__ f32x4 mfma_w4a8(const i32x4& w, const i32x8& x, const f32x4& c, int wscale) {
+    const i32x8 a = {w[0], w[1], w[2], w[3], 0, 0, 0, 0};  // e2m1: the first four registers count
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, x, c, 4 /* A: e2m1 */, 0 /* B: e4m3 */, I, wscale, 0,
+                                                            0x7F7F7F7F);
+}
+
+template <int BM, int BN, int WM, int WN, bool OUT_F32>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args p) {
+    constexpr int NT = WM * WN * 64, NW = WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TJ = WTM / 16, TI = WTN / 16;  // MFMA tiles per wave: TJ along m, TI along n
+    static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TI >= 1 && TI <= 4, "a wave holds 1..4 weight tiles: one scale word");
+    constexpr int XS = BM * 128, WS = BN * 64, SS = WN * 256;  // bytes of one stage (scales: 4 quarters x WN x 16 words)
+    constexpr int STAGE = XS + WS + SS;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    auto Xs = [&](int s) { return smem + s * STAGE; };
+    auto Ws = [&](int s) { return smem + s * STAGE + XS; };
+    auto Ss = [&](int s) { return smem + s * STAGE + XS + WS; };
+
+    int tm, tn;
+    mx4_tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const uint8_t* wptr = p.w;
+    const uint8_t* wsptr = p.ws;
+    int expert = 0;
+    if (p.m_indices) {
+        expert = p.m_indices[m0];  // groups start on multiples of 128 rows, BM divides 128
+        if (expert < 0) return;    // a tile of padding (uniform for the workgroup)
+        wptr += (int64_t)expert * p.N * p.ld_w;
+        wsptr += (int64_t)expert * p.N * p.ld_ws;
+    }
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = (p.K + 127) >> 7;
+
+    // global -> registers -> LDS.  Activations: a wave-wide load covers 8 rows x 128 bytes; weights: 16 rows x
+    // 64 bytes.  Rows past the edge of a matrix read the last valid row (their products are never stored);
+    // chunks past K read the row's first chunk and are replaced by zero.
+    constexpr int X_BLK = BM / 8, W_BLK = BN / 16;
+    constexpr int X_IT = (X_BLK + NW - 1) / NW, W_IT = (W_BLK + NW - 1) / NW;
+    constexpr int S_IT = (BN * 4 + NT - 1) / NT;
+    const int x_row8 = (lane >> 1) & 7, x_c = ((lane >> 4) << 1) | (lane & 1);
+    const int w_row16 = lane >> 2, w_c = lane & 3;
+    uint32_t ox[X_IT], ow[W_IT], os[S_IT];
+    i32x4 rx[X_IT], rw[W_IT];
+    uint32_t rs[S_IT];
+    const uint8_t* const xbase = p.a + (int64_t)m0 * p.ld_a;
+    const uint8_t* const wbase = wptr + (int64_t)n0 * p.ld_w;
+    const uint8_t* const sbase = wsptr + (int64_t)n0 * p.ld_ws;
+#pragma unroll
+    for (int i = 0; i < X_IT; ++i) {
+        const int r = (wave + NW * i) * 8 + x_row8;
+        const int rr = (m0 + r) < p.M ? r : (p.M - 1 - m0);
+        ox[i] = (uint32_t)rr * (uint32_t)p.ld_a;
+    }
+#pragma unroll
+    for (int i = 0; i < W_IT; ++i) {
+        const int r = (wave + NW * i) * 16 + w_row16;
+        const int rr = (n0 + r) < p.N ? r : (p.N - 1 - n0);
+        ow[i] = (uint32_t)rr * (uint32_t)p.ld_w;
+    }
+#pragma unroll
+    for (int i = 0; i < S_IT; ++i) {
+        const int idx = t + NT * i, r = idx >> 2;
+        const int rr = (n0 + r) < p.N ? r : (p.N - 1 - n0);
+        os[i] = (uint32_t)rr * (uint32_t)p.ld_ws;
+    }
+    auto load_tile = [&](int kt_) {
+        const int kt = kt_ < KT ? kt_ : KT - 1;
+        const int k = kt << 7;
+        const bool x_ok = k + x_c * 16 < p.K, w_ok = k + w_c * 32 < p.K;
+        const uint32_t xk = x_ok ? (uint32_t)(k + x_c * 16) : 0u, wk = w_ok ? (uint32_t)((k >> 1) + w_c * 16) : 0u;
+#pragma unroll
+        for (int i = 0; i < X_IT; ++i) {
+            const i32x4 v = *reinterpret_cast<const i32x4*>(xbase + ox[i] + xk);
+            rx[i] = x_ok ? v : i32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < W_IT; ++i) {
+            const i32x4 v = *reinterpret_cast<const i32x4*>(wbase + ow[i] + wk);
+            rw[i] = w_ok ? v : i32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < S_IT; ++i) {
+            const int kb = (kt << 2) + ((t + NT * i) & 3);
+            const bool ok = kb * 32 < p.K;
+            const uint32_t v = sbase[os[i] + (ok ? (uint32_t)kb : 0u)];
+            rs[i] = ok ? v : 127u;
+        }
+    };
+    auto store_tile = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < X_IT; ++i) {
+            const int r = (wave + NW * i) * 8 + x_row8;
+            if (X_BLK % NW == 0 || r < BM) *reinterpret_cast<i32x4*>(Xs(stage) + x_chunk_offset(r, x_c)) = rx[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_IT; ++i) {
+            const int r = (wave + NW * i) * 16 + w_row16;
+            if (W_BLK % NW == 0 || r < BN) *reinterpret_cast<i32x4*>(Ws(stage) + w_chunk_offset(r, w_c)) = rw[i];
+        }
+#pragma unroll
+        for (int i = 0; i < S_IT; ++i) {
+            const int idx = t + NT * i, r = idx >> 2, kb = idx & 3;
+            // word of (quarter kb, wave column r / WTN, tile row r % 16), byte = tile index inside the wave's columns
+            if ((BN * 4) % NT == 0 || r < BN)
+                Ss(stage)[((kb * WN + r / WTN) * 16 + (r & 15)) * 4 + ((r % WTN) >> 4)] = (uint8_t)rs[i];
+        }
+    };
+
+    f32x4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // At the top of step kt, stage kt & 1 holds tile kt and the staging registers hold tile kt + 1.  They are
+    // stored to the other stage (free since the barrier that ended step kt - 1) after the step's fragments have
+    // been read, and the loads of tile kt + 2 follow at once.  The last step stores a tile nobody reads.
+    load_tile(0);
+    store_tile(0);
+    load_tile(1);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        i32x4 fw[TI];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) fw[i] = *reinterpret_cast<const i32x4*>(Ws(cur) + w_chunk_offset(wn * WTN + i * 16 + lrow, quarter));
+        const int sw = *reinterpret_cast<const int*>(Ss(cur) + ((quarter * WN + wn) * 16 + lrow) * 4);
+        i32x8 fx[TJ];
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int row = wm * WTM + j * 16 + lrow;
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(Xs(cur) + x_chunk_offset(row, quarter));
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(Xs(cur) + x_chunk_offset(row, 4 + quarter));
+            fx[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+        store_tile(cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_tile(kt + 2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            acc[0][j] = mfma_w4a8<0>(fw[0], fx[j], acc[0][j], sw);
+            if constexpr (TI > 1) acc[1][j] = mfma_w4a8<1>(fw[1], fx[j], acc[1][j], sw);
+            if constexpr (TI > 2) acc[2][j] = mfma_w4a8<2>(fw[2], fx[j], acc[2][j], sw);
+            if constexpr (TI > 3) acc[3][j] = mfma_w4a8<3>(fw[3], fx[j], acc[3][j], sw);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds out[m][n .. n + 3] for every (i, j); everything read from global memory is read before
+    // the first store (loads and stores share one counter)
+    float sam[TJ];
+    bool keep[TJ];
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int m = m0 + wm * WTM + j * 16 + lrow;
+        keep[j] = m < p.M;
+        sam[j] = keep[j] ? p.sa[m] : 0.f;
+        if (p.m_indices && keep[j]) keep[j] = p.m_indices[m] == expert;
+    }
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const int m = m0 + wm * WTM + j * 16 + lrow;
+        if (!keep[j]) continue;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            const int n = n0 + wn * WTN + i * 16 + quarter * 4;
+            if (n >= p.N) continue;  // N % 16 == 0: a group of four is inside or outside as a whole
+            f32x4 v = acc[i][j];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] *= sam[j];
+            if (OUT_F32) {
+                *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            } else {
+                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_mx4(Mx4Args p, int out_dtype, hipStream_t st) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm_mxfp4: too many tiles");
+    constexpr size_t lds = 2 * (BM * 128 + BN * 64 + WN * 256);
+    static_assert(lds <= 64 * 1024, "two stages must fit the default dynamic LDS limit");
+    if (out_dtype == CFP8_OUT_F32)
+        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, true>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
+    else
+        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, false>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
+    return check_launch("gemm_mxfp4");
+}
+
+}  // namespace cfp8
+
+extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, const void* w, int64_t ld_w, const void* ws,
+                               int64_t ld_ws, const int32_t* m_indices, int64_t num_groups, void* out, int64_t ld_out,
+                               int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+    using namespace cfp8;
+    if (M < 0 || N < 0 || K < 0 || num_groups < 0) return set_error(CFP8_EINVAL, "gemm_mxfp4: negative shape");
+    if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "gemm_mxfp4: out_dtype must be CFP8_OUT_BF16 or CFP8_OUT_F32");
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (!a || !sa || !w || !ws || !out) return set_error(CFP8_EINVAL, "gemm_mxfp4: null pointer");
+    if (K == 0 || K % 32 || N % 16)
+        return set_error(CFP8_EINVAL, "gemm_mxfp4: K=%lld must be a positive multiple of 32 and N=%lld a multiple of 16", (long long)K, (long long)N);
+    if (m_indices ? num_groups < 1 : num_groups > 1)
+        return set_error(CFP8_EINVAL, "gemm_mxfp4: num_groups=%lld needs m_indices (and m_indices at least one group)", (long long)num_groups);
+    if (m_indices && M % 128) return set_error(CFP8_EINVAL, "gemm_mxfp4: grouped rows M=%lld must be a multiple of 128", (long long)M);
+    if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || ld_a >= (1ll << 24) || ld_w >= (1ll << 24) || ld_ws >= (1ll << 24))
+        return set_error(CFP8_EINVAL, "gemm_mxfp4: shape beyond the supported range (M, N, K < 2^31, pitches < 2^24)");
+    if (ld_a < K || ld_a % 16 || ld_w < K / 2 || ld_w % 16 || ld_ws < K / 32 || ld_out < N)
+        return set_error(CFP8_EINVAL, "gemm_mxfp4: pitches: ld_a >= K and ld_w >= K / 2 in bytes, both multiples of 16; ld_ws >= K / 32; ld_out >= N");
+    if (!aligned16(a) || !aligned16(w)) return set_error(CFP8_EINVAL, "gemm_mxfp4: a and w must be 16-byte aligned");
+    const int64_t out_align = out_dtype == CFP8_OUT_F32 ? 16 : 8;
+    if ((reinterpret_cast<uintptr_t>(out) % out_align) || (ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % out_align)
+        return set_error(CFP8_EINVAL, "gemm_mxfp4: out must be aligned to four elements and ld_out a multiple of 4");
+    if (int rc = check_device()) return rc;
+    Mx4Args p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.w = static_cast<const uint8_t*>(w);
+    p.ws = static_cast<const uint8_t*>(ws);
+    p.sa = sa;
+    p.m_indices = m_indices;
+    p.out = out;
+    p.ld_a = ld_a; p.ld_w = ld_w; p.ld_ws = ld_ws; p.ld_out = ld_out;
+    p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (M <= 16) return launch_mx4<16, 64, 1, 4>(p, out_dtype, st);
+    if (M <= 32) return launch_mx4<32, 128, 1, 4>(p, out_dtype, st);
+    if (M <= 64) return launch_mx4<64, 128, 1, 4>(p, out_dtype, st);
+    return launch_mx4<128, 128, 2, 2>(p, out_dtype, st);
+}

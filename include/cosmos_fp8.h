@@ -260,6 +260,26 @@ int cfp8_combine_rows(const void* rows, int64_t ld_rows, int64_t num_rows, const
 int cfp8_quant_mxfp4(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q,
                      void* scales, int64_t ld_scales, void* stream);
 
+/* The consumer of cfp8_quant_mxfp4's output: out[m, n] = sa[m] * sum_k a[m, k] * value(w[g, n, k]), where
+ * value = e2m1 code * 2^(ws[g, n, k / 32] - 127).  a e4m3 [M, K] (pitch ld_a bytes) with one fp32 scale per
+ * row (cfp8_quant_rowwise of the activations), w packed e2m1 [num_groups, N, K / 2] (row pitch ld_w bytes),
+ * ws e8m0 [num_groups, N, K / 32] (row pitch ld_ws bytes); groups lie N rows apart.  The matrix instruction
+ * takes the weight codes and their block scales as they are (v_mfma_scale_f32_16x16x128_f8f6f4, A in e2m1
+ * with hardware-applied e8m0 scales, B in e4m3); accumulation in fp32.  m_indices null: one weight matrix
+ * (num_groups 0 or 1).  m_indices int32 [M] (device): row m uses group m_indices[m], groups start on
+ * multiples of 128 rows, M % 128 == 0, rows with a negative index are padding and their outputs are left
+ * untouched (the layout of cfp8_gemm_grouped_block128).  K % 32 == 0 (not necessarily % 128: GPT-OSS has
+ * K = 2880), N % 16 == 0, ld_a and ld_w multiples of 16, a and w 16-byte aligned, ld_out in elements
+ * (multiple of 4).  out_dtype CFP8_OUT_BF16 or CFP8_OUT_F32.
+ * In the reference the quantised expert weights of mxfp4_quantization
+ * (cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:1000-1045) are handed to the rollout engine's FusedMoE
+ * layers (monkey_patch_for_mxfp4.py:27-47, w13_weight / w2_weight), whose matrix product lives in the
+ * third-party triton_kernels package; this entry is that product for the unswizzled [E, N, K / 2] layout
+ * of vllm_rollout.py:1025-1033, on activations quantised per token as in the FP8 linear. */
+int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, const void* w, int64_t ld_w, const void* ws,
+                    int64_t ld_ws, const int32_t* m_indices, int64_t num_groups, void* out, int64_t ld_out,
+                    int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* cfp8_gather_rows followed by cfp8_quant_group128 (CFP8_GROUP_MODE_DIV) as one pass: row r of the
  * output quantises row src_rows[r] of x (bf16 [*, cols], ld_x in elements), a zero row where src_rows[r] < 0.
  * The gathered bf16 matrix [rows_out, cols] that the reference builds with torch indexing before

@@ -74,3 +74,13 @@ def upcast(packed: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
     vals = E2M1_VALUES[codes & 7] * np.where(codes & 8, np.float32(-1), np.float32(1))
     s = np.ldexp(np.float64(1.0), scales.numpy().astype(np.int64) - 127)
     return torch.from_numpy((vals.astype(np.float64) * np.repeat(s, 32, axis=-1)).astype(np.float32))
+
+
+def gemm(xq: torch.Tensor, sx: torch.Tensor, packed: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """out[m, n] = sx[m] * sum_k xq[m, k] * upcast(packed, scales)[n, k] in float64: the product the rollout engine
+    forms with the weights of ``downcast`` (vllm_rollout.py:1018-1033 hands them to its FusedMoE layers), here on
+    per-token FP8 activations (xq e4m3 [M, K], sx fp32 [M]).  Every product xq * code * 2^e is exact in fp32 and
+    so is this sum in float64 for any K a test uses; the kernel under test may differ by its fp32 accumulation."""
+    w = upcast(packed, scales).double()
+    return (xq.float().double() @ w.t()) * sx.double().reshape(-1, 1)
+

@@ -127,3 +127,152 @@ def test_mxfp4_mirrors_and_pitches(dev):
     assert torch.equal(sp[:, :2].cpu(), ws.reshape(-1, 2)) and bool((sp[:, 2:] == 0xEE).all())
     with pytest.raises(ValueError):
         ops.quant_mxfp4(torch.zeros(4, 48, dtype=torch.bfloat16, device=dev))
+
+
+def test_gemm_oracle_against_loops():
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn(16, 64, generator=g) * 0.1).to(torch.bfloat16)
+    wq, ws = MX.downcast(w)
+    xq = (torch.randn(3, 64, generator=g) * 40).to(torch.float8_e4m3fn)
+    sx = torch.tensor([0.5, 0.013, 3.0])
+    got = MX.gemm(xq, sx, wq, ws)
+    vals = MX.E2M1_VALUES.tolist()
+    for m in range(3):
+        for n in range(16):
+            acc = 0.0
+            for k in range(64):
+                byte = int(wq[n, k // 2])
+                code = (byte >> 4) if k % 2 else (byte & 0xF)
+                v = vals[code & 7] * (-1.0 if code & 8 else 1.0) * 2.0 ** (int(ws[n, k // 32]) - 127)
+                acc += float(xq[m, k].float()) * v
+            assert got[m, n].item() == pytest.approx(acc * float(sx[m]), rel=1e-12, abs=1e-300)
+
+
+def _mx_weights(g, *shape, spread=2.0):
+    w = torch.randn(*shape, generator=g) * 0.05 * torch.exp(torch.randn(*shape[:-1], 1, generator=g) * spread)
+    return MX.downcast(w.to(torch.bfloat16))
+
+
+def _fp8_rows(g, M, K):
+    x = torch.randn(M, K, generator=g) * torch.exp(torch.randn(M, 1, generator=g))
+    amax = x.abs().amax(dim=1, keepdim=True).clamp_min(1e-12)
+    s = (amax / 448.0).float()
+    return (x / s).to(torch.float8_e4m3fn), s.reshape(-1)
+
+
+def _rel(got, want):
+    return float((got.double() - want).norm() / want.norm().clamp_min(1e-300))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1, 16, 32), (5, 48, 96), (16, 64, 128), (17, 80, 160), (33, 128, 2880), (64, 256, 512),
+                                   (100, 272, 896), (128, 128, 128), (129, 144, 64), (300, 512, 2880), (1000, 400, 1056)])
+def test_gemm_mxfp4_against_oracle(dev, M, N, K):
+    """fp32 output within 1e-5 (relative Frobenius) of the exact sum, bf16 output within 1e-3 of the bf16-rounded
+    exact sum; rows and columns beyond M and N of a padded output stay untouched."""
+    from cosmos_rl_amd import ops
+    g = torch.Generator().manual_seed(M * 7919 + N * 31 + K)
+    wq, ws = _mx_weights(g, N, K)
+    xq, sx = _fp8_rows(g, M, K)
+    want = MX.gemm(xq, sx, wq, ws)
+    got = ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), torch.float32)
+    assert _rel(got.cpu(), want) <= 1e-5
+    got16 = ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), torch.bfloat16)
+    assert _rel(got16.cpu().float(), want.float().to(torch.bfloat16).double()) <= 1e-3
+    assert torch.equal(got.to(torch.bfloat16), got16)          # the two epilogues round the same accumulators
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [8, 160])
+def test_gemm_mxfp4_one_hot_is_exact(dev, M):
+    """Row m of the activations is 1.0 at k = m (mod K): the output is the weight value itself, so the nibble
+    order, the lane that owns each block of 32 and the scale byte it is paired with are all pinned bit for bit."""
+    from cosmos_rl_amd import ops
+    K, N = 160, 192
+    g = torch.Generator().manual_seed(6)
+    wq, ws = _mx_weights(g, N, K, spread=6.0)
+    x = torch.zeros(M, K)
+    ks = [(m * 37) % K for m in range(M)]
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    xq = x.to(torch.float8_e4m3fn)
+    sx = torch.ones(M)
+    got = ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), torch.float32).cpu()
+    want = MX.upcast(wq, ws)[:, ks].t().contiguous()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_gemm_mxfp4_grouped(dev):
+    """Groups of 128-aligned rows, one of them empty, padding rows (index -1) left untouched."""
+    from cosmos_rl_amd import ops
+    g = torch.Generator().manual_seed(7)
+    E, N, K = 4, 208, 352
+    counts = [200, 0, 128, 77]
+    wq, ws = _mx_weights(g, E, N, K)
+    idx, rows = [], 0
+    for e, c in enumerate(counts):
+        padded = -(-c // 128) * 128
+        idx += [e] * c + [-1] * (padded - c)
+        rows += padded
+    m_indices = torch.tensor(idx, dtype=torch.int32)
+    xq, sx = _fp8_rows(g, rows, K)
+    out = torch.full((rows, N), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), m_indices=m_indices.to(dev), out=out)
+    out = out.cpu()
+    for e in range(E):
+        sel = m_indices == e
+        if not bool(sel.any()):
+            continue
+        want = MX.gemm(xq[sel], sx[sel], wq[e], ws[e])
+        assert _rel(out[sel].float(), want.float().to(torch.bfloat16).double()) <= 1e-3, e
+    assert bool((out[m_indices < 0] == 7.0).all())
+
+
+@pytest.mark.gpu
+def test_gemm_mxfp4_pitches_and_errors(dev):
+    from cosmos_rl_amd import _lib, ops
+    g = torch.Generator().manual_seed(8)
+    M, N, K = 70, 96, 224
+    wq, ws = _mx_weights(g, N, K)
+    xq, sx = _fp8_rows(g, M, K)
+    want = MX.gemm(xq, sx, wq, ws)
+    # padded pitches of every operand; the output's padding columns keep their bytes
+    xp = torch.zeros(M, 256, dtype=torch.uint8, device=dev); xp[:, :K] = xq.view(torch.uint8).to(dev)
+    wp = torch.full((N, 128), 0x77, dtype=torch.uint8, device=dev); wp[:, :K // 2] = wq.to(dev)
+    sp = torch.full((N, 9), 0xFF, dtype=torch.uint8, device=dev); sp[:, :K // 32] = ws.to(dev)
+    out = torch.full((M, 100), -3.0, dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.cfp8_gemm_mxfp4(xp.data_ptr(), 256, sx.to(dev).data_ptr(), wp.data_ptr(), 128, sp.data_ptr(), 9, None, 0,
+                                   out.data_ptr(), 100, _lib.OUT_F32, M, N, K, st))
+    assert _rel(out[:, :N].cpu(), want) <= 1e-5 and bool((out[:, N:] == -3.0).all())
+    ptr = out.data_ptr()
+    assert lib.cfp8_gemm_mxfp4(ptr, 64, ptr, ptr, 32, ptr, 2, None, 0, ptr, 16, _lib.OUT_F32, 4, 16, 48, st) == _lib.EINVAL    # K % 32
+    assert lib.cfp8_gemm_mxfp4(ptr, 64, ptr, ptr, 32, ptr, 2, None, 0, ptr, 24, _lib.OUT_F32, 4, 24, 64, st) == _lib.EINVAL    # N % 16
+    assert lib.cfp8_gemm_mxfp4(ptr, 64, ptr, ptr, 24, ptr, 2, None, 0, ptr, 16, _lib.OUT_F32, 4, 16, 64, st) == _lib.EINVAL    # ld_w
+    assert lib.cfp8_gemm_mxfp4(ptr, 64, ptr, ptr, 32, ptr, 2, None, 3, ptr, 16, _lib.OUT_F32, 4, 16, 64, st) == _lib.EINVAL    # groups without indices
+    assert lib.cfp8_gemm_mxfp4(ptr, 64, ptr, ptr, 32, ptr, 2, ptr, 2, ptr, 16, _lib.OUT_F32, 100, 16, 64, st) == _lib.EINVAL   # grouped M % 128
+    assert lib.cfp8_gemm_mxfp4(None, 64, None, None, 32, None, 2, None, 0, None, 16, _lib.OUT_F32, 0, 16, 64, st) == 0
+    with pytest.raises(ValueError):
+        ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev)[:, :-1], ws.to(dev)))
+
+
+@pytest.mark.gpu
+def test_linear_mxfp4_end_to_end(dev):
+    """bf16 activations -> per-token FP8 -> MXFP4 product, against the same chain in the oracles."""
+    from cosmos_rl_amd import ops
+    from oracle import fp8_oracle as O
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randn(320, 2880, generator=g) * 0.03).to(torch.bfloat16)
+    x = (torch.randn(2, 45, 2880, generator=g)).to(torch.bfloat16)
+    wq, ws = ops.quant_mxfp4(w.to(dev))
+    y = ops.linear_mxfp4(x.to(dev), (wq, ws))
+    assert y.shape == (2, 45, 320) and y.dtype == torch.bfloat16
+    xq, sx = O.quant_rowwise(x.reshape(-1, 2880))
+    want = MX.gemm(xq.view(torch.float8_e4m3fn), sx.reshape(-1), *MX.downcast(w)).reshape(2, 45, 320)
+    assert _rel(y.cpu().float(), want.float().to(torch.bfloat16).double()) <= 1e-3
+    # and the quantisation error of the whole chain against the unquantised product stays at MXFP4's level
+    exact = x.double() @ w.double().t()
+    assert _rel(y.cpu().float(), exact) < 0.15
+
