@@ -252,6 +252,182 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
     }
 }
 
+// At most 16 tokens (decode): the weight is read once and nothing else matters.  A workgroup owns 16 weight rows,
+// its four waves split K (wave w takes K steps w, w + 4, ...) and each requests the codes and scale bytes of
+// kGemvDepth of its steps - 16 bytes and one byte per lane and step, straight into MFMA operand registers -
+// before the first MFMA.  The few activation rows come from global memory (they stay in L2); rows >= M, and
+// chunks beyond K, are zero.  The four partial sums meet in LDS.
+constexpr int kGemvDepth = 8;
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_mxfp4_gemv_kernel(const Mx4Args p) {
+    __shared__ __attribute__((aligned(16))) float red[3 * 64 * 4];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int KT = (p.K + 127) >> 7;
+    const int wrow = n0 + lrow;
+    const bool wok = wrow < p.N, xok = lrow < p.M;
+    const uint8_t* const wptr = p.w + (int64_t)(wok ? wrow : 0) * p.ld_w + quarter * 16;
+    const uint8_t* const sptr = p.ws + (int64_t)(wok ? wrow : 0) * p.ld_ws + quarter;
+    const uint8_t* const xptr = p.a + (int64_t)(xok ? lrow : 0) * p.ld_a + quarter * 16;
+    const float sam = xok ? p.sa[lrow] : 0.f;  // requested first: nothing at the end waits for memory
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = wave; base < KT; base += 4 * kGemvDepth) {
+        u32x4 wv[kGemvDepth], xl[kGemvDepth], xh[kGemvDepth];
+        uint32_t sc[kGemvDepth];
+#pragma unroll
+        for (int i = 0; i < kGemvDepth; ++i) {
+            const int kt = base + 4 * i;
+            const int k = (kt < KT ? kt : 0) << 7;
+            // a block of 32 lies inside K as a whole or not at all (K % 32 == 0); what lies outside is read from the
+            // start of the row and dropped below
+            const bool in_w = kt < KT && k + quarter * 32 < p.K, in_lo = kt < KT && k + quarter * 16 < p.K,
+                       in_hi = kt < KT && k + 64 + quarter * 16 < p.K;
+            wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + (in_w ? (k >> 1) : 0)));
+            sc[i] = __builtin_nontemporal_load(sptr + (in_w ? (k >> 5) : 0));
+            xl[i] = *reinterpret_cast<const u32x4*>(xptr + (in_lo ? k : 0));
+            xh[i] = *reinterpret_cast<const u32x4*>(xptr + (in_hi ? k + 64 : 0));
+        }
+        __builtin_amdgcn_sched_barrier(0);  // every load of the pass is requested before the first MFMA
+#pragma unroll
+        for (int i = 0; i < kGemvDepth; ++i) {
+            const int kt = base + 4 * i;
+            const int k = (kt < KT ? kt : 0) << 7;
+            const bool in_w = kt < KT && k + quarter * 32 < p.K, in_lo = kt < KT && k + quarter * 16 < p.K,
+                       in_hi = kt < KT && k + 64 + quarter * 16 < p.K;
+            i32x4 fw;
+            i32x8 fx;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                fw[e] = (int)wv[i][e];                             // any e2m1 code is finite: the zero on the other side suffices
+                fx[e] = (in_lo && xok) ? (int)xl[i][e] : 0;
+                fx[4 + e] = (in_hi && xok) ? (int)xh[i][e] : 0;
+            }
+            const int scale = (in_w && wok) ? (int)sc[i] : 127;    // 255 would be NaN
+            acc = mfma_w4a8<0>(fw, fx, acc, scale);
+        }
+    }
+    if (wave > 0) *reinterpret_cast<f32x4*>(red + ((wave - 1) * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + quarter * 4, m = lrow;
+        if (n < p.N && m < p.M) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) {
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + (w * 64 + lane) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += o[e];
+            }
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[e] * sam;
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+    }
+}
+
+// The same for at most kGemvLdsRows tokens with the activations in LDS: a workgroup first requests the weights of its
+// first pass, then copies the M activation rows (K bytes each, zero beyond K) into LDS, and reads its MFMA
+// fragments from there.  Without 64 registers of activations in flight a wave needs half the registers, so that
+// every workgroup of a 18944-row weight is resident at once and the whole weight is requested at the start.
+constexpr int kGemvLdsRows = 8;
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_mxfp4_gemv_lds_kernel(const Mx4Args p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [M][KT * 128 + 16]
+    __shared__ __attribute__((aligned(16))) float red[3 * 64 * 4];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int KT = (p.K + 127) >> 7;
+    const int pitch = KT * 128 + 16;
+    const int wrow = n0 + lrow;
+    const bool wok = wrow < p.N, xok = lrow < p.M;
+    const uint8_t* const wptr = p.w + (int64_t)(wok ? wrow : 0) * p.ld_w + quarter * 16;
+    const uint8_t* const sptr = p.ws + (int64_t)(wok ? wrow : 0) * p.ld_ws + quarter;
+    const uint8_t* const xrow = xs + (xok ? lrow : 0) * pitch + quarter * 16;
+    u32x4 wv[kGemvDepth];
+    uint32_t sc[kGemvDepth];
+    auto load_pass = [&](int base) {
+#pragma unroll
+        for (int i = 0; i < kGemvDepth; ++i) {
+            const int kt = base + 4 * i;
+            const int k = (kt < KT ? kt : 0) << 7;
+            const bool in_w = kt < KT && k + quarter * 32 < p.K;
+            wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + (in_w ? (k >> 1) : 0)));
+            sc[i] = __builtin_nontemporal_load(sptr + (in_w ? (k >> 5) : 0));
+        }
+    };
+    load_pass(wave);
+    const float sam = xok ? p.sa[lrow] : 0.f;  // requested early: nothing at the end waits for memory
+    {
+        const int chunks = KT * 8, total = p.M * chunks;
+        for (int idx = t; idx < total; idx += 256) {
+            const int row = idx / chunks, c = idx - row * chunks;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (c * 16 < p.K) v = *reinterpret_cast<const u32x4*>(p.a + (int64_t)row * p.ld_a + c * 16);
+            *reinterpret_cast<u32x4*>(xs + row * pitch + c * 16) = v;
+        }
+    }
+    __syncthreads();
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = wave; base < KT; base += 4 * kGemvDepth) {
+        if (base != wave) load_pass(base);
+#pragma unroll
+        for (int i = 0; i < kGemvDepth; ++i) {
+            const int kt = base + 4 * i;
+            const int k = (kt < KT ? kt : 0) << 7;
+            const bool in = kt < KT, in_w = in && k + quarter * 32 < p.K;
+            i32x4 fw;
+            i32x8 fx;
+            const u32x4 lo = *reinterpret_cast<const u32x4*>(xrow + k), hi = *reinterpret_cast<const u32x4*>(xrow + k + 64);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                fw[e] = (int)wv[i][e];
+                fx[e] = (in && xok) ? (int)lo[e] : 0;
+                fx[4 + e] = (in && xok) ? (int)hi[e] : 0;
+            }
+            const int scale = (in_w && wok) ? (int)sc[i] : 127;
+            acc = mfma_w4a8<0>(fw, fx, acc, scale);
+        }
+    }
+    if (wave > 0) *reinterpret_cast<f32x4*>(red + ((wave - 1) * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + quarter * 4, m = lrow;
+        if (n < p.N && m < p.M) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) {
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + (w * 64 + lane) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += o[e];
+            }
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[e] * sam;
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+    }
+}
+
+static int launch_mx4_gemv(const Mx4Args& p, int out_dtype, hipStream_t st) {
+    const unsigned blocks = (unsigned)((p.N + 15) / 16);
+    const size_t x_lds = (size_t)p.M * ((size_t)((p.K + 127) / 128) * 128 + 16);
+    if (p.M <= kGemvLdsRows && x_lds <= 32 * 1024) {
+        if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(gemm_mxfp4_gemv_lds_kernel<true>, dim3(blocks), dim3(256), x_lds, st, p);
+        else hipLaunchKernelGGL(gemm_mxfp4_gemv_lds_kernel<false>, dim3(blocks), dim3(256), x_lds, st, p);
+        return check_launch("gemm_mxfp4");
+    }
+    if (out_dtype == CFP8_OUT_F32) hipLaunchKernelGGL(gemm_mxfp4_gemv_kernel<true>, dim3(blocks), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(gemm_mxfp4_gemv_kernel<false>, dim3(blocks), dim3(256), 0, st, p);
+    return check_launch("gemm_mxfp4");
+}
+
 template <int BM, int BN, int WM, int WN>
 static int launch_mx4(Mx4Args p, int out_dtype, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -301,8 +477,9 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     p.ld_a = ld_a; p.ld_w = ld_w; p.ld_ws = ld_ws; p.ld_out = ld_out;
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (M <= 16 && !m_indices) return launch_mx4_gemv(p, out_dtype, st);
     if (M <= 16) return launch_mx4<16, 64, 1, 4>(p, out_dtype, st);
-    if (M <= 32) return launch_mx4<32, 128, 1, 4>(p, out_dtype, st);
-    if (M <= 64) return launch_mx4<64, 128, 1, 4>(p, out_dtype, st);
+    if (M <= 32) return launch_mx4<32, 64, 1, 4>(p, out_dtype, st);
+    if (M <= 64) return launch_mx4<64, 64, 1, 4>(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2>(p, out_dtype, st);
 }
