@@ -15,7 +15,7 @@
 // As in the FP8 kernels the weight tile is the MFMA "A" operand, so a lane's four accumulators are four
 // consecutive n of one output row.
 //
-// Tiles: BM x BN x 128 per workgroup, two LDS stages filled through registers.  An activation stage is the
+// Tiles: BM x BN per workgroup, two LDS stages of KB K steps of 128 each, filled through registers.  An activation stage is the
 // chunk-major layout of the FP8 kernels (16-row blocks of 2 KiB).  A weight stage holds 64 bytes per row:
 // 16-row blocks of 1 KiB, the 16-byte chunk c (0..3) of row r at c * 256 + ((r ^ (c << 2)) & 15) * 16, so that
 // a fragment read (16 lanes = 16 rows of one chunk) and a staging store (16 lanes = 4 rows x 4 chunks) each
@@ -70,19 +70,20 @@ __device__ __forceinline__ f32x4 mfma_w4a8(const i32x4& w, const i32x8& x, const
                                                             0x7F7F7F7F);
 }
 
-template <int BM, int BN, int WM, int WN, bool OUT_F32>
+template <int BM, int BN, int WM, int WN, int KB, bool OUT_F32>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args p) {
     constexpr int NT = WM * WN * 64, NW = WM * WN;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TJ = WTM / 16, TI = WTN / 16;  // MFMA tiles per wave: TJ along m, TI along n
     static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TI >= 1 && TI <= 4, "a wave holds 1..4 weight tiles: one scale word");
     constexpr int XS = BM * 128, WS = BN * 64, SS = WN * 256;  // bytes of one stage (scales: 4 quarters x WN x 16 words)
-    constexpr int STAGE = XS + WS + SS;
+    constexpr int SUB = XS + WS + SS;        // one K step of 128
+    constexpr int STAGE = KB * SUB;          // a stage holds KB consecutive K steps
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    auto Xs = [&](int s) { return smem + s * STAGE; };
-    auto Ws = [&](int s) { return smem + s * STAGE + XS; };
-    auto Ss = [&](int s) { return smem + s * STAGE + XS + WS; };
+    auto Xs = [&](int s, int u) { return smem + s * STAGE + u * SUB; };
+    auto Ws = [&](int s, int u) { return smem + s * STAGE + u * SUB + XS; };
+    auto Ss = [&](int s, int u) { return smem + s * STAGE + u * SUB + XS + WS; };
 
     int tm, tn;
     mx4_tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int lrow = lane & 15, quarter = lane >> 4;
-    const int KT = (p.K + 127) >> 7;
+    const int KT = (p.K + 127) >> 7;        // K steps of 128
+    const int NS = (KT + KB - 1) / KB;      // stages
 
     // global -> registers -> LDS.  Activations: a wave-wide load covers 8 rows x 128 bytes; weights: 16 rows x
     // 64 bytes.  Rows past the edge of a matrix read the last valid row (their products are never stored);
@@ -112,8 +114,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
     const int x_row8 = (lane >> 1) & 7, x_c = ((lane >> 4) << 1) | (lane & 1);
     const int w_row16 = lane >> 2, w_c = lane & 3;
     uint32_t ox[X_IT], ow[W_IT], os[S_IT];
-    i32x4 rx[X_IT], rw[W_IT];
-    uint32_t rs[S_IT];
+    i32x4 rx[KB][X_IT], rw[KB][W_IT];
+    uint32_t rs[KB][S_IT];
     const uint8_t* const xbase = p.a + (int64_t)m0 * p.ld_a;
     const uint8_t* const wbase = wptr + (int64_t)n0 * p.ld_w;
     const uint8_t* const sbase = wsptr + (int64_t)n0 * p.ld_ws;
@@ -135,46 +137,53 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
         const int rr = (n0 + r) < p.N ? r : (p.N - 1 - n0);
         os[i] = (uint32_t)rr * (uint32_t)p.ld_ws;
     }
-    auto load_tile = [&](int kt_) {
-        const int kt = kt_ < KT ? kt_ : KT - 1;
-        const int k = kt << 7;
-        const bool x_ok = k + x_c * 16 < p.K, w_ok = k + w_c * 32 < p.K;
-        const uint32_t xk = x_ok ? (uint32_t)(k + x_c * 16) : 0u, wk = w_ok ? (uint32_t)((k >> 1) + w_c * 16) : 0u;
+    auto load_tile = [&](int s_) {  // stage s_ of the K loop; stages past the end re-read the last one
+        const int s0 = (s_ < NS ? s_ : NS - 1) * KB;
 #pragma unroll
-        for (int i = 0; i < X_IT; ++i) {
-            const i32x4 v = *reinterpret_cast<const i32x4*>(xbase + ox[i] + xk);
-            rx[i] = x_ok ? v : i32x4{0, 0, 0, 0};
-        }
+        for (int u = 0; u < KB; ++u) {
+            const int kt = s0 + u;               // may lie past KT: then every chunk is "beyond K"
+            const int k = kt << 7;
+            const bool x_ok = k + x_c * 16 < p.K, w_ok = k + w_c * 32 < p.K;
+            const uint32_t xk = x_ok ? (uint32_t)(k + x_c * 16) : 0u, wk = w_ok ? (uint32_t)((k >> 1) + w_c * 16) : 0u;
 #pragma unroll
-        for (int i = 0; i < W_IT; ++i) {
-            const i32x4 v = *reinterpret_cast<const i32x4*>(wbase + ow[i] + wk);
-            rw[i] = w_ok ? v : i32x4{0, 0, 0, 0};
-        }
+            for (int i = 0; i < X_IT; ++i) {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(xbase + ox[i] + xk);
+                rx[u][i] = x_ok ? v : i32x4{0, 0, 0, 0};
+            }
 #pragma unroll
-        for (int i = 0; i < S_IT; ++i) {
-            const int kb = (kt << 2) + ((t + NT * i) & 3);
-            const bool ok = kb * 32 < p.K;
-            const uint32_t v = sbase[os[i] + (ok ? (uint32_t)kb : 0u)];
-            rs[i] = ok ? v : 127u;
+            for (int i = 0; i < W_IT; ++i) {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(wbase + ow[i] + wk);
+                rw[u][i] = w_ok ? v : i32x4{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int i = 0; i < S_IT; ++i) {
+                const int kb = (kt << 2) + ((t + NT * i) & 3);
+                const bool ok = kb * 32 < p.K;
+                const uint32_t v = sbase[os[i] + (ok ? (uint32_t)kb : 0u)];
+                rs[u][i] = ok ? v : 127u;
+            }
         }
     };
     auto store_tile = [&](int stage) {
 #pragma unroll
-        for (int i = 0; i < X_IT; ++i) {
-            const int r = (wave + NW * i) * 8 + x_row8;
-            if (X_BLK % NW == 0 || r < BM) *reinterpret_cast<i32x4*>(Xs(stage) + x_chunk_offset(r, x_c)) = rx[i];
-        }
+        for (int u = 0; u < KB; ++u) {
 #pragma unroll
-        for (int i = 0; i < W_IT; ++i) {
-            const int r = (wave + NW * i) * 16 + w_row16;
-            if (W_BLK % NW == 0 || r < BN) *reinterpret_cast<i32x4*>(Ws(stage) + w_chunk_offset(r, w_c)) = rw[i];
-        }
+            for (int i = 0; i < X_IT; ++i) {
+                const int r = (wave + NW * i) * 8 + x_row8;
+                if (X_BLK % NW == 0 || r < BM) *reinterpret_cast<i32x4*>(Xs(stage, u) + x_chunk_offset(r, x_c)) = rx[u][i];
+            }
 #pragma unroll
-        for (int i = 0; i < S_IT; ++i) {
-            const int idx = t + NT * i, r = idx >> 2, kb = idx & 3;
-            // word of (quarter kb, wave column r / WTN, tile row r % 16), byte = tile index inside the wave's columns
-            if ((BN * 4) % NT == 0 || r < BN)
-                Ss(stage)[((kb * WN + r / WTN) * 16 + (r & 15)) * 4 + ((r % WTN) >> 4)] = (uint8_t)rs[i];
+            for (int i = 0; i < W_IT; ++i) {
+                const int r = (wave + NW * i) * 16 + w_row16;
+                if (W_BLK % NW == 0 || r < BN) *reinterpret_cast<i32x4*>(Ws(stage, u) + w_chunk_offset(r, w_c)) = rw[u][i];
+            }
+#pragma unroll
+            for (int i = 0; i < S_IT; ++i) {
+                const int idx = t + NT * i, r = idx >> 2, kb = idx & 3;
+                // word of (quarter kb, wave column r / WTN, tile row r % 16), byte = tile index inside the wave's columns
+                if ((BN * 4) % NT == 0 || r < BN)
+                    Ss(stage, u)[((kb * WN + r / WTN) * 16 + (r & 15)) * 4 + ((r % WTN) >> 4)] = (uint8_t)rs[u][i];
+            }
         }
     };
 
@@ -184,38 +193,45 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
 #pragma unroll
         for (int j = 0; j < TJ; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // At the top of step kt, stage kt & 1 holds tile kt and the staging registers hold tile kt + 1.  They are
-    // stored to the other stage (free since the barrier that ended step kt - 1) after the step's fragments have
-    // been read, and the loads of tile kt + 2 follow at once.  The last step stores a tile nobody reads.
+    // At the top of stage s, LDS stage s & 1 holds the K steps of stage s and the staging registers hold stage s + 1.
+    // They are stored to the other LDS stage (free since the barrier that ended stage s - 1) after the first
+    // step's fragments have been read, and the loads of stage s + 2 follow at once.  The last iteration stores a
+    // stage nobody reads.
     load_tile(0);
     store_tile(0);
     load_tile(1);
     __syncthreads();
 
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        i32x4 fw[TI];
+    for (int s = 0; s < NS; ++s) {
+        const int cur = s & 1;
 #pragma unroll
-        for (int i = 0; i < TI; ++i) fw[i] = *reinterpret_cast<const i32x4*>(Ws(cur) + w_chunk_offset(wn * WTN + i * 16 + lrow, quarter));
-        const int sw = *reinterpret_cast<const int*>(Ss(cur) + ((quarter * WN + wn) * 16 + lrow) * 4);
-        i32x8 fx[TJ];
+        for (int u = 0; u < KB; ++u) {
+            i32x4 fw[TI];
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-            const int row = wm * WTM + j * 16 + lrow;
-            const i32x4 lo = *reinterpret_cast<const i32x4*>(Xs(cur) + x_chunk_offset(row, quarter));
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(Xs(cur) + x_chunk_offset(row, 4 + quarter));
-            fx[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-        store_tile(cur ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        load_tile(kt + 2);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int i = 0; i < TI; ++i)
+                fw[i] = *reinterpret_cast<const i32x4*>(Ws(cur, u) + w_chunk_offset(wn * WTN + i * 16 + lrow, quarter));
+            const int sw = *reinterpret_cast<const int*>(Ss(cur, u) + ((quarter * WN + wn) * 16 + lrow) * 4);
+            i32x8 fx[TJ];
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-            acc[0][j] = mfma_w4a8<0>(fw[0], fx[j], acc[0][j], sw);
-            if constexpr (TI > 1) acc[1][j] = mfma_w4a8<1>(fw[1], fx[j], acc[1][j], sw);
-            if constexpr (TI > 2) acc[2][j] = mfma_w4a8<2>(fw[2], fx[j], acc[2][j], sw);
-            if constexpr (TI > 3) acc[3][j] = mfma_w4a8<3>(fw[3], fx[j], acc[3][j], sw);
+            for (int j = 0; j < TJ; ++j) {
+                const int row = wm * WTM + j * 16 + lrow;
+                const i32x4 lo = *reinterpret_cast<const i32x4*>(Xs(cur, u) + x_chunk_offset(row, quarter));
+                const i32x4 hi = *reinterpret_cast<const i32x4*>(Xs(cur, u) + x_chunk_offset(row, 4 + quarter));
+                fx[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+            if (u == 0) {
+                store_tile(cur ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+                load_tile(s + 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                acc[0][j] = mfma_w4a8<0>(fw[0], fx[j], acc[0][j], sw);
+                if constexpr (TI > 1) acc[1][j] = mfma_w4a8<1>(fw[1], fx[j], acc[1][j], sw);
+                if constexpr (TI > 2) acc[2][j] = mfma_w4a8<2>(fw[2], fx[j], acc[2][j], sw);
+                if constexpr (TI > 3) acc[3][j] = mfma_w4a8<3>(fw[3], fx[j], acc[3][j], sw);
+            }
         }
         __syncthreads();
     }
@@ -428,18 +444,18 @@ static int launch_mx4_gemv(const Mx4Args& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm_mxfp4");
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int KB>
 static int launch_mx4(Mx4Args p, int out_dtype, hipStream_t st) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm_mxfp4: too many tiles");
-    constexpr size_t lds = 2 * (BM * 128 + BN * 64 + WN * 256);
+    constexpr size_t lds = 2 * KB * (BM * 128 + BN * 64 + WN * 256);
     static_assert(lds <= 64 * 1024, "two stages must fit the default dynamic LDS limit");
     if (out_dtype == CFP8_OUT_F32)
-        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, true>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
+        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, KB, true>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
     else
-        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, false>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
+        hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, KB, false>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
     return check_launch("gemm_mxfp4");
 }
 
@@ -478,8 +494,8 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     p.M = (int)M; p.N = (int)N; p.K = (int)K;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M <= 16 && !m_indices) return launch_mx4_gemv(p, out_dtype, st);
-    if (M <= 16) return launch_mx4<16, 64, 1, 4>(p, out_dtype, st);
-    if (M <= 32) return launch_mx4<32, 64, 1, 4>(p, out_dtype, st);
-    if (M <= 64) return launch_mx4<64, 64, 1, 4>(p, out_dtype, st);
-    return launch_mx4<128, 128, 2, 2>(p, out_dtype, st);
+    if (M <= 16) return launch_mx4<16, 64, 1, 4, 2>(p, out_dtype, st);
+    if (M <= 32) return launch_mx4<32, 64, 1, 4, 2>(p, out_dtype, st);
+    if (M <= 64) return launch_mx4<64, 64, 1, 4, 2>(p, out_dtype, st);
+    return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
 }
