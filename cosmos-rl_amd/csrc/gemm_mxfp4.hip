@@ -24,6 +24,8 @@
 // and K step, the byte is picked by the instruction's op_sel.
 // K need not be a multiple of 128: the chunks of the last step that lie beyond K are loaded as zero with the
 // scale byte 127.
+#include <atomic>
+
 #include "cfp8_common.h"
 
 namespace cfp8 {
@@ -75,8 +77,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
     constexpr int NT = WM * WN * 64, NW = WM * WN;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TJ = WTM / 16, TI = WTN / 16;  // MFMA tiles per wave: TJ along m, TI along n
-    static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TI >= 1 && TI <= 4, "a wave holds 1..4 weight tiles: one scale word");
-    constexpr int XS = BM * 128, WS = BN * 64, SS = WN * 256;  // bytes of one stage (scales: 4 quarters x WN x 16 words)
+    static_assert(WTM % 16 == 0 && WTN % 16 == 0 && TI >= 1 && TI <= 8, "a wave holds 1..8 weight tiles: one or two scale words");
+    constexpr int SWN = (TI + 3) / 4;        // scale words per lane and K step
+    constexpr int XS = BM * 128, WS = BN * 64, SS = WN * 256 * SWN;  // bytes of one K step (scales: 4 quarters x WN x 16 lanes x SWN words)
     constexpr int SUB = XS + WS + SS;        // one K step of 128
     constexpr int STAGE = KB * SUB;          // a stage holds KB consecutive K steps
 
@@ -182,7 +185,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
                 const int idx = t + NT * i, r = idx >> 2, kb = idx & 3;
                 // word of (quarter kb, wave column r / WTN, tile row r % 16), byte = tile index inside the wave's columns
                 if ((BN * 4) % NT == 0 || r < BN)
-                    Ss(stage, u)[((kb * WN + r / WTN) * 16 + (r & 15)) * 4 + ((r % WTN) >> 4)] = (uint8_t)rs[u][i];
+                    Ss(stage, u)[((kb * WN + r / WTN) * 16 + (r & 15)) * (4 * SWN) + ((r % WTN) >> 4)] = (uint8_t)rs[u][i];
             }
         }
     };
@@ -210,7 +213,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
 #pragma unroll
             for (int i = 0; i < TI; ++i)
                 fw[i] = *reinterpret_cast<const i32x4*>(Ws(cur, u) + w_chunk_offset(wn * WTN + i * 16 + lrow, quarter));
-            const int sw = *reinterpret_cast<const int*>(Ss(cur, u) + ((quarter * WN + wn) * 16 + lrow) * 4);
+            int sw[SWN];
+#pragma unroll
+            for (int w = 0; w < SWN; ++w)
+                sw[w] = *reinterpret_cast<const int*>(Ss(cur, u) + ((quarter * WN + wn) * 16 + lrow) * (4 * SWN) + 4 * w);
             i32x8 fx[TJ];
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
@@ -227,10 +233,14 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_mxfp4_kernel(const Mx4Args 
             }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                acc[0][j] = mfma_w4a8<0>(fw[0], fx[j], acc[0][j], sw);
-                if constexpr (TI > 1) acc[1][j] = mfma_w4a8<1>(fw[1], fx[j], acc[1][j], sw);
-                if constexpr (TI > 2) acc[2][j] = mfma_w4a8<2>(fw[2], fx[j], acc[2][j], sw);
-                if constexpr (TI > 3) acc[3][j] = mfma_w4a8<3>(fw[3], fx[j], acc[3][j], sw);
+                acc[0][j] = mfma_w4a8<0>(fw[0], fx[j], acc[0][j], sw[0]);
+                if constexpr (TI > 1) acc[1][j] = mfma_w4a8<1>(fw[1], fx[j], acc[1][j], sw[0]);
+                if constexpr (TI > 2) acc[2][j] = mfma_w4a8<2>(fw[2], fx[j], acc[2][j], sw[0]);
+                if constexpr (TI > 3) acc[3][j] = mfma_w4a8<3>(fw[3], fx[j], acc[3][j], sw[0]);
+                if constexpr (TI > 4) acc[4][j] = mfma_w4a8<0>(fw[4], fx[j], acc[4][j], sw[SWN - 1]);
+                if constexpr (TI > 5) acc[5][j] = mfma_w4a8<1>(fw[5], fx[j], acc[5][j], sw[SWN - 1]);
+                if constexpr (TI > 6) acc[6][j] = mfma_w4a8<2>(fw[6], fx[j], acc[6][j], sw[SWN - 1]);
+                if constexpr (TI > 7) acc[7][j] = mfma_w4a8<3>(fw[7], fx[j], acc[7][j], sw[SWN - 1]);
             }
         }
         __syncthreads();
@@ -431,6 +441,188 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_gemv_lds_kernel(const Mx4Args 
     }
 }
 
+// 17..64 tokens: still a weight streamer.  A workgroup of 2 NTL waves owns 16 NTL weight rows; wave (nt, kh) takes the
+// 16 rows of n-tile nt and the kh-th half of every chunk of KS K steps.  K is walked in passes of PC
+// chunks: at the start of a pass a wave requests all of its weight codes and scale bytes of the pass (16 bytes + 1
+// byte per lane and step, straight into MFMA operand registers, 8 steps = 40 registers), then the
+// workgroup stages the activations chunk by chunk through two LDS buffers (the activations of 64 tokens are four
+// times the bytes of the workgroup's weights per chunk, so they must not be fetched per wave).  The two K halves
+// are summed through LDS at the end.
+template <int TM, int NTL, int KS, int PC, bool OUT_F32>
+__global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4Args p) {
+    constexpr int NW = NTL * 2;                   // waves: NTL n-tiles x 2 K halves
+    constexpr int HS = KS / 2;                    // K steps per wave and chunk
+    constexpr int XU = KS * TM * 2;               // wave-wide loads that stage one chunk of activations
+    constexpr int XI = (XU + NW - 1) / NW;
+    constexpr int XSTAGE = KS * TM * 2048;        // bytes of one activation buffer
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int nt = wave % NTL, kh = wave / NTL;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * (NTL * 16);
+    const int KT = (p.K + 127) >> 7;
+    const int chunks = (KT + KS - 1) / KS;
+
+    // activation staging: one wave-wide load = 8 rows x 128 bytes of one K step
+    const int st_row8 = (lane >> 1) & 7, st_c = ((lane >> 4) << 1) | (lane & 1);
+    // through a buffer descriptor that ends with the M-th row: rows beyond M read zero, and the per-lane part of
+    // an address (row, K step inside the chunk, 16-byte piece) is computed once
+    i32x4 xr[XI];
+    uint32_t xoff[XI];
+    const int64_t a_left = (int64_t)p.M * p.ld_a;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.a), 0, a_left < 0xFFFFFFFFll ? (int)a_left : (int)0xFFFFFFFFu, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < XI; ++i) {
+        const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
+        xoff[i] = (unit < XU && row < p.M) ? (uint32_t)row * (uint32_t)p.ld_a + (ks << 7) + st_c * 16 : 0xFFFFFFFFu;
+    }
+    auto xload = [&](int chunk) {
+        const int k0 = (chunk * KS) << 7;
+#pragma unroll
+        for (int i = 0; i < XI; ++i) {
+            const int unit = wave + NW * i, ks = unit % KS;
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[i], k0, 0);
+            const bool ok = k0 + (ks << 7) + st_c * 16 < p.K;     // beyond K the row's pitch or the next row follows
+            xr[i] = ok ? i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]} : i32x4{0, 0, 0, 0};
+        }
+    };
+    auto xstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < XI; ++i) {
+            const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
+            if (XU % NW == 0 || unit < XU)
+                *reinterpret_cast<i32x4*>(smem + buf * XSTAGE + (ks * TM + (row >> 4)) * 2048 + x_chunk_offset(row & 15, st_c)) = xr[i];
+        }
+    };
+    // Weight codes and scale bytes come through buffer descriptors that end with the matrix: a load costs one
+    // scalar offset (the K step is uniform for the wave) on top of a per-lane row offset, rows beyond N read zero,
+    // and a block beyond K reads whatever follows it inside the matrix (any e2m1 code is finite; its scale byte is
+    // replaced and the activations there are zero).
+    const int wrow = n0 + nt * 16 + lrow;
+    const bool wok = wrow < p.N;
+    const int64_t w_left = (int64_t)(p.N - n0) * p.ld_w, s_left = (int64_t)(p.N - n0) * p.ld_ws;
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.w) + (int64_t)n0 * p.ld_w, 0, w_left < 0xFFFFFFFFll ? (int)w_left : (int)0xFFFFFFFFu, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.ws) + (int64_t)n0 * p.ld_ws, 0, s_left < 0xFFFFFFFFll ? (int)s_left : (int)0xFFFFFFFFu, 0x00020000);
+    const uint32_t w_lane = (uint32_t)(nt * 16 + lrow) * (uint32_t)p.ld_w + quarter * 16;
+    const uint32_t s_lane = (uint32_t)(nt * 16 + lrow) * (uint32_t)p.ld_ws + quarter;
+
+    f32x4 acc[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    xload(0);
+    for (int c0 = 0; c0 < chunks; c0 += PC) {
+        // this wave's weights of the pass: chunk c0 + cc, steps kh * HS + h
+        u32x4 wv[PC][HS];
+        uint32_t sc[PC][HS];
+#pragma unroll
+        for (int cc = 0; cc < PC; ++cc)
+#pragma unroll
+            for (int h = 0; h < HS; ++h) {
+                const int k = ((c0 + cc) * KS + kh * HS + h) << 7;
+                wv[cc][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_lane, k >> 1, 2);
+                sc[cc][h] = __builtin_amdgcn_raw_buffer_load_b8(rs, s_lane, k >> 5, 2);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int cc = 0; cc < PC; ++cc) {
+            const int c = c0 + cc;
+            // the buffer of chunk c was last read during chunk c - 2, two barriers ago
+            xstore(c & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            xload(c + 1);           // chunks past the end load zeros
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+#pragma unroll
+            for (int h = 0; h < HS; ++h) {
+                const int ks = kh * HS + h;
+                const int k = (c * KS + ks) << 7;
+                const bool in_w = k + quarter * 32 < p.K;
+                const int scale = (in_w && wok) ? (int)sc[cc][h] : 127;  // 255 would be NaN; beyond K the activations are zero
+                i32x4 fw;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) fw[e] = (int)wv[cc][h][e];
+#pragma unroll
+                for (int j = 0; j < TM; ++j) {
+                    const uint8_t* const xt = smem + (c & 1) * XSTAGE + (ks * TM + j) * 2048;
+                    const i32x4 lo = *reinterpret_cast<const i32x4*>(xt + x_chunk_offset(lrow, quarter));
+                    const i32x4 hi = *reinterpret_cast<const i32x4*>(xt + x_chunk_offset(lrow, 4 + quarter));
+                    const i32x8 fx = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    acc[j] = mfma_w4a8<0>(fw, fx, acc[j], scale);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // fragments of one K step at a time; nothing of the next chunk moves up
+            }
+            // the MFMAs are pure functions of registers: without a use here the compiler sinks all of a pass behind its
+            // last barrier and keeps every fragment of the pass alive until then
+#pragma unroll
+            for (int j = 0; j < TM; ++j) asm volatile("" : "+v"(acc[j]));
+        }
+    }
+
+    // sum the two K halves through LDS (both buffers may still be read by a slower wave: barrier first)
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(smem);
+    if (kh == 1) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) *reinterpret_cast<f32x4*>(red + ((nt * TM + j) * 64 + lane) * 4) = acc[j];
+    }
+    __syncthreads();
+    if (kh == 0) {
+        const int n = n0 + nt * 16 + quarter * 4;
+        if (n < p.N) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int m = j * 16 + lrow;
+                if (m >= p.M) continue;
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + ((nt * TM + j) * 64 + lane) * 4);
+                const float sam = p.sa[m];
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = (acc[j][e] + o[e]) * sam;
+                if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+                else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                        make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+    }
+}
+
+// more dynamic LDS than the default 64 KiB: the limit is raised once per device and kernel
+static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64]) {
+    if (lds <= 64 * 1024) return CFP8_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm_mxfp4: no current device");
+    const bool cached = dev >= 0 && dev < 64;
+    if (cached && raised[dev].load(std::memory_order_acquire)) return CFP8_OK;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+        (void)hipGetLastError();
+        return set_error(CFP8_ELAUNCH, "gemm_mxfp4: cannot raise the dynamic LDS limit to %zu bytes", lds);
+    }
+    if (cached) raised[dev].store(true, std::memory_order_release);
+    return CFP8_OK;
+}
+
+template <int TM, int NTL>
+static int launch_mx4_skinny(const Mx4Args& p, int out_dtype, hipStream_t st) {
+    // 64 KiB of activation buffers either way, eight K steps of weights per wave in flight
+    constexpr int KS = TM > 2 ? 4 : 8, PC = TM > 2 ? 4 : 2;
+    constexpr size_t lds = (size_t)2 * KS * TM * 2048;  // >= the NTL * TM * 1 KiB of the final reduction
+    static_assert(lds >= (size_t)NTL * TM * 1024 && lds <= 160 * 1024, "skinny kernel LDS");
+    const unsigned blocks = (unsigned)((p.N + NTL * 16 - 1) / (NTL * 16));
+    const bool f32 = out_dtype == CFP8_OUT_F32;
+    const void* fn = f32 ? reinterpret_cast<const void*>(gemm_mxfp4_skinny_kernel<TM, NTL, KS, PC, true>)
+                         : reinterpret_cast<const void*>(gemm_mxfp4_skinny_kernel<TM, NTL, KS, PC, false>);
+    static std::atomic<bool> raised[2][64];
+    if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
+    if (f32) hipLaunchKernelGGL((gemm_mxfp4_skinny_kernel<TM, NTL, KS, PC, true>), dim3(blocks), dim3(NTL * 128), lds, st, p);
+    else hipLaunchKernelGGL((gemm_mxfp4_skinny_kernel<TM, NTL, KS, PC, false>), dim3(blocks), dim3(NTL * 128), lds, st, p);
+    return check_launch("gemm_mxfp4");
+}
+
 static int launch_mx4_gemv(const Mx4Args& p, int out_dtype, hipStream_t st) {
     const unsigned blocks = (unsigned)((p.N + 15) / 16);
     const size_t x_lds = (size_t)p.M * ((size_t)((p.K + 127) / 128) * 128 + 16);
@@ -450,8 +642,13 @@ static int launch_mx4(Mx4Args p, int out_dtype, hipStream_t st) {
     p.tiles_n = (p.N + BN - 1) / BN;
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm_mxfp4: too many tiles");
-    constexpr size_t lds = 2 * KB * (BM * 128 + BN * 64 + WN * 256);
-    static_assert(lds <= 64 * 1024, "two stages must fit the default dynamic LDS limit");
+    constexpr size_t lds = 2 * KB * (BM * 128 + BN * 64 + WN * 256 * ((BN / WN / 16 + 3) / 4));
+    static_assert(lds <= 160 * 1024, "two stages must fit LDS");
+    const bool f32 = out_dtype == CFP8_OUT_F32;
+    static std::atomic<bool> raised[2][64];
+    const void* fn = f32 ? reinterpret_cast<const void*>(gemm_mxfp4_kernel<BM, BN, WM, WN, KB, true>)
+                         : reinterpret_cast<const void*>(gemm_mxfp4_kernel<BM, BN, WM, WN, KB, false>);
+    if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
     if (out_dtype == CFP8_OUT_F32)
         hipLaunchKernelGGL((gemm_mxfp4_kernel<BM, BN, WM, WN, KB, true>), dim3((unsigned)tiles), dim3(WM * WN * 64), lds, st, p);
     else
@@ -495,7 +692,15 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M <= 16 && !m_indices) return launch_mx4_gemv(p, out_dtype, st);
     if (M <= 16) return launch_mx4<16, 64, 1, 4, 2>(p, out_dtype, st);
+    if (M <= 64 && !m_indices) {
+        // few weight rows: narrow workgroups, so that there are enough of them
+        const bool narrow = (N + 15) / 16 <= 512;
+        if (M <= 32) return narrow ? launch_mx4_skinny<2, 3>(p, out_dtype, st) : launch_mx4_skinny<2, 5>(p, out_dtype, st);
+        return narrow ? launch_mx4_skinny<4, 3>(p, out_dtype, st) : launch_mx4_skinny<4, 5>(p, out_dtype, st);
+    }
     if (M <= 32) return launch_mx4<32, 64, 1, 4, 2>(p, out_dtype, st);
     if (M <= 64) return launch_mx4<64, 64, 1, 4, 2>(p, out_dtype, st);
+    // 256 x 256 tiles (one wave per SIMD, 128 x 128 per wave) once they fill the GPU at least twice
+    if (!m_indices && (M + 255) / 256 * ((N + 255) / 256) >= 512) return launch_mx4<256, 256, 2, 2, 1>(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
 }
