@@ -591,6 +591,244 @@ __global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4A
     }
 }
 
+// ---------------------------------------------------------------------------
+// Large full tiles: 256 x 256 x 128 per workgroup, four wavefronts (one per SIMD, 2 x 2), each owning a 128 x 128
+// block = 64 accumulators of 16 x 16.  Operands go from global memory straight into LDS (buffer_load ... lds: no
+// staging registers, no LDS store instructions; the LDS layout is dictated by which bytes each lane asks for):
+//   activations  two stages of 32 KiB, row-major, the 16-byte chunk c of row r at position c ^ ((r >> 1) & 7);
+//   weights      three stages of 16 KiB, row r at r * 64, chunk c (0..3) at position c ^ ((r >> 2) & 3): a fragment
+//                read (16 rows, one chunk) covers all 64 banks once;
+//   scale bytes  three stages of 1 KiB: the four scale bytes of a row and K step are one 32-bit word, stored so
+//                that a lane finds the words of its eight 16-row tiles next to each other (word index
+//                wn * 128 + lrow * 8 + tile) and picks its quarter's byte with a shift.
+// The K step is a software pipeline of 32 groups of two MFMAs, each preceded by at most one direct-to-LDS load
+// and one fragment read; step kt computes from activation stage kt % 2 and weight / scale stage kt % 3:
+//   S0 (w0,x0): LDS reads x1            S1 (w0,x1): LDS reads w1
+//   -- wait for all but the five newest loads and for own LDS reads, barrier --
+//   S2 (w1,x0): LDS reads next w0 and its scales + loads of activation tile kt + 2
+//   S3 (w1,x1): LDS reads next x0 + loads of weight and scale tile kt + 3 (the five newest at the next barrier)
+// Requires M % 256 == 0, N % 256 == 0, K % 128 == 0 and 4-byte aligned scale rows.
+// ---------------------------------------------------------------------------
+#define MX4_PHASE_END() __builtin_amdgcn_sched_barrier(0)
+// written out as instructions: in front of a barrier it knows of, the compiler waits for every load it has issued,
+// including the direct-to-LDS loads that are meant to stay in flight across the barrier
+#define MX4_WAIT_BARRIER(vm) asm volatile("s_waitcnt vmcnt(" #vm ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#define MX4_MMA2(wh, xb, xh, g)                                                                              \
+    {                                                                                                        \
+        _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                      \
+            const int j = (g) >> 1, i = ((g)&1) * 2 + e;                                                     \
+            acc[(wh)*4 + i][(xh)*4 + j] =                                                                    \
+                mfma_w4a8<0>(W[wh][i], X[xb][j], acc[(wh)*4 + i][(xh)*4 + j], (int)S[(wh)*4 + i]);          \
+        }                                                                                                    \
+    }
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_mxfp4_256_kernel(const Mx4Args p) {
+    constexpr int BM = 256, BN = 256;
+    constexpr int XS = BM * 128, WS = BN * 64, SS = BN * 4;
+    constexpr int WBASE = 2 * XS, SBASE = WBASE + 3 * WS, ABASE = SBASE + 3 * SS;  // + 1 KiB of activation scales
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    mx4_tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+
+    // Wave-uniform bases pass through an empty asm so that they stay in SGPRs for the whole K loop (a scalar load
+    // inside the loop would have to be waited for with lgkmcnt(0), which drains the fragment reads in flight).
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t w_wave = reinterpret_cast<uint64_t>(p.w) + ((uint64_t)n0 + (uint64_t)wave * 16) * (uint64_t)p.ld_w;
+    uint64_t s_tile = reinterpret_cast<uint64_t>(p.ws) + (uint64_t)n0 * (uint64_t)p.ld_ws;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, w_step = 64u * (uint32_t)p.ld_w;  // pitches are < 2^24
+    asm volatile("" : "+s"(a_wave), "+s"(w_wave), "+s"(s_tile), "+s"(a_step), "+s"(w_step));
+    // activations: load i covers rows (wave + 4 i) * 8 .. + 7; (r >> 1) & 7 of row r = (wave + 4 i) * 8 + (lane >> 3)
+    // is (wave & 1) * 4 + (lane >> 4)
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    // weights: load i covers rows (wave + 4 i) * 16 .. + 15; lane (row16, position) fetches chunk position ^ (row16 >> 2)
+    const uint32_t vw_lane = (uint32_t)(lane >> 2) * (uint32_t)p.ld_w + (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+    // scale words: word wave * 64 + lane = wn' * 128 + lrow' * 8 + tile' belongs to row wn' * 128 + tile' * 16 + lrow'
+    const int sword = wave * 64 + lane;
+    const uint32_t vs_lane = (uint32_t)((sword >> 7) * 128 + (sword & 7) * 16 + ((sword >> 3) & 15)) * (uint32_t)p.ld_ws;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, 0xFFFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(w_wave), 0, 0xFFFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(s_tile), 0, 0xFFFFFFFF, 0x00020000);
+    auto dma_x = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    auto dma_w = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, vw_lane,
+                                                 (uint32_t)i * w_step + ((uint32_t)kt << 6), 0, 0);
+    };
+    auto dma_s = [&](int kt, int stage) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + SBASE + stage * SS + wave * 256), 4, vs_lane,
+                                                 (uint32_t)kt << 2, 0, 0);
+    };
+
+    f32x4 acc[8][8];  // [n tile][m tile]
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // activation fragment: the e4m3 operand's registers 0-3 are k = 16 q .. + 15, registers 4-7 k = 64 + 16 q .. + 15
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 128 + lrow) * 128 + ((quarter ^ fsw) << 4);
+    const int x_off2 = (wm * 128 + lrow) * 128 + (((4 + quarter) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 128 + lrow) * 64 + ((quarter ^ ((lrow >> 2) & 3)) << 4);
+    const int s_off = SBASE + (wn * 128 + lrow * 8) * 4;
+    const unsigned sshift = 8u * (unsigned)quarter;
+    auto xfrag = [&](int stage_bytes, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + x_off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + x_off2);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    auto wfrag = [&](int stage, int tile16) { return *reinterpret_cast<const i32x4*>(smem + stage * WS + tile16 * 1024 + w_off); };
+    auto sfrag = [&](int stage, int half) { return *reinterpret_cast<const u32x4*>(smem + stage * SS + s_off + half * 16); };
+    i32x4 W[2][4];
+    i32x8 X[2][4];
+    uint32_t S[8];  // this lane's scale byte of the wave's eight weight tiles, in the low byte
+    u32x4 sraw, sraw_hi;  // scale words of tiles 0-3 / 4-7 of the next K step
+
+    // prologue: the tile's 256 activation scales for the epilogue (64 per wave, 4 bytes per lane, a region of their
+    // own), then activation tiles 0, 1 and weight + scale tiles 0, 1, 2 into their stages
+    __builtin_amdgcn_global_load_lds((gbl_void*)(p.sa + m0 + wave * 64 + lane), (lds_void*)(smem + ABASE + wave * 256), 4, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(0, 0, i);
+    dma_s(0, 0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_x(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(1 < last ? 1 : last, 1, i);
+    dma_s(1 < last ? 1 : last, 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(2 < last ? 2 : last, 2, i);
+    dma_s(2 < last ? 2 : last, 2);
+    MX4_WAIT_BARRIER(18);  // the scales and tile 0 (14 loads) have landed; the other 18 stay in flight
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        W[0][g] = wfrag(0, g);
+        X[0][g] = xfrag(0, g);
+    }
+    sraw = sfrag(0, 0);
+    sraw_hi = sfrag(0, 1);
+    asm volatile("" : "+v"(sraw), "+v"(sraw_hi));  // two 16-byte reads, not eight of four bytes
+#pragma unroll
+    for (int g = 0; g < 4; ++g) S[g] = sraw[g] >> sshift;
+    MX4_PHASE_END();
+
+    int ws_cur = 0;  // kt % 3
+    for (int kt = 0; kt < KT; ++kt) {
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ws_cur == 2 ? 0 : ws_cur + 1;
+        // past the end: the last tile again, into a stage nobody reads any more (no branch in the K loop)
+        const int kw = kt + 3 < last ? kt + 3 : last, kx = kt + 2 < last ? kt + 2 : last;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) X[1][g] = xfrag(xs_cur, 4 + g);
+            MX4_MMA2(0, 0, 0, g);
+            MX4_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) W[1][g] = wfrag(ws_cur, 4 + g);
+            if (g >= 4) S[g] = sraw_hi[g - 4] >> sshift;
+            MX4_MMA2(0, 1, 1, g);
+            MX4_PHASE_END();
+        }
+        MX4_WAIT_BARRIER(5);
+        MX4_PHASE_END();
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) W[0][g] = wfrag(ws_nxt, g);  // after the last step: stale data, unused
+            if (g == 4) {
+                sraw = sfrag(ws_nxt, 0);
+                asm volatile("" : "+v"(sraw));
+            }
+            if (g == 5) {
+                sraw_hi = sfrag(ws_nxt, 1);  // S[4..7] are still in use: shifted into place in S1 of the next step
+                asm volatile("" : "+v"(sraw_hi));
+            }
+            dma_x(kx, kt & 1, g);
+            MX4_MMA2(1, 0, 0, g);
+            MX4_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g < 4) X[0][g] = xfrag(xs_nxt, g);
+            if (g < 4) dma_w(kw, ws_cur, g);
+            if (g == 4) dma_s(kw, ws_cur);
+            if (g >= 4) S[g - 4] = sraw[g - 4] >> sshift;
+            MX4_MMA2(1, 1, 1, g);
+            MX4_PHASE_END();
+        }
+        ws_cur = ws_nxt;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the scales have landed, and nothing may still land in the stages
+    __syncthreads();
+    const float* const sa_lds = reinterpret_cast<const float*>(smem + ABASE);
+
+    float sam[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sam[j] = sa_lds[wm * 128 + j * 16 + lrow];
+    if (OUT_F32) {
+        // a lane already owns 16 contiguous bytes: store directly
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int n = n0 + wn * 128 + i * 16 + quarter * 4;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int m = m0 + wm * 128 + j * 16 + lrow;
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j];
+                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: scale, convert, turn the wave's 128 x 128 block through LDS in two halves of 64 rows
+    // (row stride 272 B keeps the 8-byte stores of 16 rows on different banks)
+    __syncthreads();  // all waves are done reading the operand stages
+    constexpr int EST = 272;
+    static_assert(4 * 64 * EST <= ABASE, "the epilogue buffers must not reach the activation scales");
+    uint8_t* const ebuf = smem + wave * (64 * EST);
+    const int rd_row = lane >> 4, rd_chunk = lane & 15;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = h * 4 + jj;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j];
+                *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = r * 4 + rd_row;  // 0..63 within the half
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            const int m = m0 + wm * 128 + h * 64 + row;
+            __builtin_nontemporal_store(
+                d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 128 + rd_chunk * 8));
+        }
+    }
+}
+
 // more dynamic LDS than the default 64 KiB: the limit is raised once per device and kernel
 static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64]) {
     if (lds <= 64 * 1024) return CFP8_OK;
@@ -604,6 +842,20 @@ static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64
     }
     if (cached) raised[dev].store(true, std::memory_order_release);
     return CFP8_OK;
+}
+
+static int launch_mx4_256(Mx4Args p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 256;
+    constexpr size_t lds = 2 * 256 * 128 + 3 * 256 * 64 + 3 * 256 * 4 + 1024;
+    const bool f32 = out_dtype == CFP8_OUT_F32;
+    static std::atomic<bool> raised[2][64];
+    const void* fn = f32 ? reinterpret_cast<const void*>(gemm_mxfp4_256_kernel<true>) : reinterpret_cast<const void*>(gemm_mxfp4_256_kernel<false>);
+    if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
+    const unsigned blocks = (unsigned)(p.tiles_m * p.tiles_n);
+    if (f32) hipLaunchKernelGGL(gemm_mxfp4_256_kernel<true>, dim3(blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL(gemm_mxfp4_256_kernel<false>, dim3(blocks), dim3(256), lds, st, p);
+    return check_launch("gemm_mxfp4");
 }
 
 template <int TM, int NTL>
@@ -700,7 +952,10 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     }
     if (M <= 32) return launch_mx4<32, 64, 1, 4, 2>(p, out_dtype, st);
     if (M <= 64) return launch_mx4<64, 64, 1, 4, 2>(p, out_dtype, st);
-    // 256 x 256 tiles (one wave per SIMD, 128 x 128 per wave) once they fill the GPU at least twice
-    if (!m_indices && (M + 255) / 256 * ((N + 255) / 256) >= 512) return launch_mx4<256, 256, 2, 2, 1>(p, out_dtype, st);
+    // 256 x 256 tiles of the direct-to-LDS pipeline once they fill at least half of the GPU
+    const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0;
+    if (!m_indices && M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && ld_ws % 4 == 0 && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0 &&
+        out16 && (M / 256) * (N / 256) >= 128 && (M / 256) * (N / 256) <= 0x7FFFFFFFll)
+        return launch_mx4_256(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
 }

@@ -168,7 +168,8 @@ def _rel(got, want):
 @pytest.mark.parametrize("M,N,K", [(1, 16, 32), (5, 48, 96), (16, 64, 128), (17, 80, 160), (33, 128, 2880), (64, 256, 512),
                                    (100, 272, 896), (128, 128, 128), (129, 144, 64), (300, 512, 2880), (1000, 400, 1056),
                                    (16, 80, 2880), (2, 528, 4256), (9, 2064, 3584),
-                                   (17, 96, 128), (24, 8400, 2880), (31, 176, 6304), (50, 8272, 896), (64, 320, 4096), (64, 18944, 3584), (4096, 8192, 288), (4000, 8208, 160)])
+                                   (17, 96, 128), (24, 8400, 2880), (31, 176, 6304), (50, 8272, 896), (64, 320, 4096), (64, 18944, 3584), (4096, 8192, 288), (4000, 8208, 160),
+                                   (2048, 4096, 384), (4096, 8192, 128), (2048, 4096, 256), (2560, 3328, 1152)])
 def test_gemm_mxfp4_against_oracle(dev, M, N, K):
     """fp32 output within 1e-5 (relative Frobenius) of the exact sum, bf16 output within 1e-3 of the bf16-rounded
     exact sum; rows and columns beyond M and N of a padded output stay untouched."""
