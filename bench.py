@@ -519,6 +519,24 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         lambda: check(lib.cfp8_quant_mxfp4(wx.data_ptr(), RX, KX, KX, qx.data_ptr(), KX // 2, sx.data_ptr(), KX // 32, stream)))
     del wx, qx, sx
 
+    # the consumer of those weights: FP8 activations (per-token scales) x MXFP4 weights on the scaled matrix
+    # instruction.  Config 3's shape, so that the lines sit beside linear_rowwise_cfg3_M* (FP8 weights: twice the
+    # weight bytes), and the GPT-OSS-20B gate_up shape of one expert's worth of columns at 8192 tokens.
+    for (nm, M, N, K) in [("cfg3", 1, 18944, 3584), ("cfg3", 16, 18944, 3584), ("cfg3", 64, 18944, 3584),
+                          ("cfg3", 8192, 18944, 3584), ("gptoss_5632x2816", 8192, 5632, 2816)]:
+        name = f"gemm_mxfp4_{nm}_M{M}"
+        if only and only not in name:
+            continue
+        w4 = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev, generator=gen)
+        s4 = torch.randint(118, 126, (N, K // 32), dtype=torch.uint8, device=dev, generator=gen)
+        xq = torch.randn(M, K, generator=gen, device=dev).mul_(60).to(torch.float8_e4m3fn)
+        sxq = torch.rand(M, generator=gen, device=dev) + 0.5
+        o = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        mfma(name, 2.0 * M * N * K, N * K // 2 + N * K // 32 + M * K + 4 * M + M * N * 2,
+             lambda: check(lib.cfp8_gemm_mxfp4(xq.data_ptr(), K, sxq.data_ptr(), w4.data_ptr(), K // 2, s4.data_ptr(), K // 32,
+                                               None, 0, o.data_ptr(), N, 0, M, N, K, stream)), iters=50)
+        del w4, s4, xq, sxq, o
+
     # config 5: Qwen3-30B-A3B experts, 8192 tokens routed top-8 over 128 experts
     E, H, I, T, TOPK = 128, 2048, 768, 8192, 8
     wgu = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)

@@ -1,6 +1,7 @@
-"""Instruction census of the walking GEMM kernels, from hipcc's own assembly listing of csrc/gemm_fp8.hip.
+"""Instruction census of the GEMM kernels with hand-counted waits, from hipcc's own assembly listing of
+csrc/gemm_fp8.hip and csrc/gemm_mxfp4.hip.
 
-gemm_rowwise_256p_kernel and gemm_block_w8p_kernel order their LDS traffic with hand-written
+gemm_rowwise_256p_kernel, gemm_block_w8p_kernel and gemm_mxfp4_256_kernel order their LDS traffic with hand-written
 ``s_waitcnt vmcnt(N)`` + ``s_barrier`` pairs: N is the number of vector-memory operations the author
 counted between the loads a barrier needs and the barrier.  That is right only while the compiler
 emits exactly those operations, so the census (vector-memory instructions by kind, barriers, the N of
@@ -22,26 +23,30 @@ ROOT = Path(__file__).resolve().parent.parent
 sys.path.insert(0, str(ROOT / "cosmos-rl_amd"))
 from cosmos_rl_amd import _build  # noqa: E402
 
-WALKING = ("gemm_rowwise_256p_kernel", "gemm_block_w8p_kernel")
+WALKING = ("gemm_rowwise_256p_kernel", "gemm_block_w8p_kernel", "gemm_mxfp4_256_kernel")
+SOURCES = ("gemm_fp8.hip", "gemm_mxfp4.hip")
 _VMEM = re.compile(r"^\s+((?:buffer|global|flat|scratch)_(?:load|store|atomic)\w*)\b(.*)")
 _PAIR = re.compile(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)")
 
 
 def assembly() -> list[str]:
-    """hipcc -S of gemm_fp8.hip for gfx950 with the library's own flags (about 15 s)."""
+    """hipcc -S of the GEMM sources for gfx950 with the library's own flags (about 20 s)."""
+    lines: list[str] = []
     with tempfile.TemporaryDirectory() as tmp:
-        out = Path(tmp) / "gemm_fp8.s"
-        cmd = [_build.hipcc(), *_build.HIPCC_FLAGS, f"-I{_build.INCLUDE_DIR}", f"-I{_build.CSRC_DIR}", "--cuda-device-only", "-S",
-               str(_build.CSRC_DIR / "gemm_fp8.hip"), "-o", str(out)]
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError(f"hipcc -S failed:\n{res.stderr}")
-        return out.read_text().splitlines()
+        for src in SOURCES:
+            out = Path(tmp) / (src + ".s")
+            cmd = [_build.hipcc(), *_build.HIPCC_FLAGS, f"-I{_build.INCLUDE_DIR}", f"-I{_build.CSRC_DIR}", "--cuda-device-only", "-S",
+                   str(_build.CSRC_DIR / src), "-o", str(out)]
+            res = subprocess.run(cmd, capture_output=True, text=True)
+            if res.returncode != 0:
+                raise RuntimeError(f"hipcc -S failed:\n{res.stderr}")
+            lines += out.read_text().splitlines()
+    return lines
 
 
 def demangled_key(symbol: str) -> str:
     """_ZN4cfp821gemm_block_w8p_kernelILi128ELi256ELi2ELb0ELb1EEEvNS_8GemmArgsE -> gemm_block_w8p_kernel<128,256,2,0,1>"""
-    m = re.match(r"_ZN4cfp8\d+([a-z0-9_]+?)I(.*)EEvNS_8GemmArgsE$", symbol)
+    m = re.match(r"_ZN4cfp8\d+([a-z0-9_]+?)I(.*)EEvNS_\d+\w+ArgsE$", symbol)
     if not m:
         return symbol
     args = re.findall(r"L[ib](\d+)E", m.group(2))
@@ -63,16 +68,21 @@ def census(lines: list[str]) -> dict[str, dict]:
         ops: Counter[str] = Counter()
         pairs: list[int] = []
         barriers = 0
+        mfmas = [k for k, line in enumerate(body) if re.match(r"^\s+v_mfma", line)]
+        spills_between_mfmas = 0  # scratch accesses inside the K loop (anything between the first and the last MFMA)
         for k, line in enumerate(body):
             v = _VMEM.match(line)
             if v:
                 ops[v.group(1) + (" lds" if re.search(r"\blds\b", v.group(2)) else "")] += 1
+                if v.group(1).startswith("scratch_") and mfmas and mfmas[0] < k < mfmas[-1]:
+                    spills_between_mfmas += 1
             if "s_barrier" in line:
                 barriers += 1
                 p = _PAIR.search(body[k - 1])
                 if p:
                     pairs.append(int(p.group(1)))
         out[demangled_key(m.group(1))] = {"vector_memory": dict(sorted(ops.items())), "barriers": barriers,
-                                         "hand_written_vmcnt_before_barrier": sorted(pairs)}
+                                         "hand_written_vmcnt_before_barrier": sorted(pairs), "mfma": len(mfmas),
+                                         "scratch_between_mfmas": spills_between_mfmas}
         i = j
     return out
