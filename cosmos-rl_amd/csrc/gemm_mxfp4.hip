@@ -448,6 +448,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_gemv_lds_kernel(const Mx4Args 
 // workgroup stages the activations chunk by chunk through two LDS buffers (the activations of 64 tokens are four
 // times the bytes of the workgroup's weights per chunk, so they must not be fetched per wave).  The two K halves
 // are summed through LDS at the end.
+constexpr uint32_t kBeyond = 0xF0000000u;  // a per-lane buffer offset no descriptor of this kernel covers
 template <int TM, int NTL, int KS, int PC, bool OUT_F32>
 __global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4Args p) {
     constexpr int NW = NTL * 2;                   // waves: NTL n-tiles x 2 K halves
@@ -472,20 +473,20 @@ __global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4A
     uint32_t xoff[XI];
     const int64_t a_left = (int64_t)p.M * p.ld_a;
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.a), 0, a_left < 0xFFFFFFFFll ? (int)a_left : (int)0xFFFFFFFFu, 0x00020000);
+        const_cast<uint8_t*>(p.a), 0, a_left < (int64_t)kBeyond ? (int)a_left : (int)kBeyond, 0x00020000);
 #pragma unroll
     for (int i = 0; i < XI; ++i) {
         const int unit = wave + NW * i, ks = unit % KS, row = (unit / KS) * 8 + st_row8;
-        xoff[i] = (unit < XU && row < p.M) ? (uint32_t)row * (uint32_t)p.ld_a + (ks << 7) + st_c * 16 : 0xFFFFFFFFu;
+        xoff[i] = (unit < XU && row < p.M) ? (uint32_t)row * (uint32_t)p.ld_a + (ks << 7) + st_c * 16 : kBeyond;
     }
     auto xload = [&](int chunk) {
         const int k0 = (chunk * KS) << 7;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             const int unit = wave + NW * i, ks = unit % KS;
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, xoff[i], k0, 0);
-            const bool ok = k0 + (ks << 7) + st_c * 16 < p.K;     // beyond K the row's pitch or the next row follows
-            xr[i] = ok ? i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]} : i32x4{0, 0, 0, 0};
+            const bool ok = k0 + (ks << 7) + st_c * 16 < p.K;     // beyond K: not fetched, zero
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? xoff[i] : kBeyond, k0, 0);
+            xr[i] = i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
         }
     };
     auto xstore = [&](int buf) {
@@ -497,16 +498,17 @@ __global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4A
         }
     };
     // Weight codes and scale bytes come through buffer descriptors that end with the matrix: a load costs one
-    // scalar offset (the K step is uniform for the wave) on top of a per-lane row offset, rows beyond N read zero,
-    // and a block beyond K reads whatever follows it inside the matrix (any e2m1 code is finite; its scale byte is
-    // replaced and the activations there are zero).
+    // scalar offset (the K step is uniform for the wave) on top of a per-lane row offset.  Rows beyond N and blocks
+    // beyond K are not fetched at all: their lane offset is kBeyond, past the end of any descriptor here (a
+    // workgroup's rows span less than 2^31 bytes and a scalar offset is below 2^24, so the sum neither wraps nor
+    // comes back into range), and such a load returns zero.
     const int wrow = n0 + nt * 16 + lrow;
-    const bool wok = wrow < p.N;
+    const bool wok = wrow < p.N;  // rows beyond N lie past the descriptors' end by themselves
     const int64_t w_left = (int64_t)(p.N - n0) * p.ld_w, s_left = (int64_t)(p.N - n0) * p.ld_ws;
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.w) + (int64_t)n0 * p.ld_w, 0, w_left < 0xFFFFFFFFll ? (int)w_left : (int)0xFFFFFFFFu, 0x00020000);
+        const_cast<uint8_t*>(p.w) + (int64_t)n0 * p.ld_w, 0, w_left < (int64_t)kBeyond ? (int)w_left : (int)kBeyond, 0x00020000);
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.ws) + (int64_t)n0 * p.ld_ws, 0, s_left < 0xFFFFFFFFll ? (int)s_left : (int)0xFFFFFFFFu, 0x00020000);
+        const_cast<uint8_t*>(p.ws) + (int64_t)n0 * p.ld_ws, 0, s_left < (int64_t)kBeyond ? (int)s_left : (int)kBeyond, 0x00020000);
     const uint32_t w_lane = (uint32_t)(nt * 16 + lrow) * (uint32_t)p.ld_w + quarter * 16;
     const uint32_t s_lane = (uint32_t)(nt * 16 + lrow) * (uint32_t)p.ld_ws + quarter;
 
@@ -524,8 +526,9 @@ __global__ __launch_bounds__(NTL * 128) void gemm_mxfp4_skinny_kernel(const Mx4A
 #pragma unroll
             for (int h = 0; h < HS; ++h) {
                 const int k = ((c0 + cc) * KS + kh * HS + h) << 7;
-                wv[cc][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, w_lane, k >> 1, 2);
-                sc[cc][h] = __builtin_amdgcn_raw_buffer_load_b8(rs, s_lane, k >> 5, 2);
+                const bool in_w = k + quarter * 32 < p.K;
+                wv[cc][h] = __builtin_amdgcn_raw_buffer_load_b128(rw, in_w ? w_lane : kBeyond, k >> 1, 2);
+                sc[cc][h] = __builtin_amdgcn_raw_buffer_load_b8(rs, in_w ? s_lane : kBeyond, k >> 5, 2);
             }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
