@@ -525,7 +525,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     for (nm, M, N, K) in [("cfg3", 1, 18944, 3584), ("cfg3", 16, 18944, 3584), ("cfg3", 64, 18944, 3584),
                           ("cfg3", 8192, 18944, 3584), ("gptoss_5632x2816", 8192, 5632, 2816)]:
         name = f"gemm_mxfp4_{nm}_M{M}"
-        if only and only not in name:
+        if only and only not in name and only not in f"linear_mxfp4_{nm}_M{M}":
             continue
         w4 = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device=dev, generator=gen)
         s4 = torch.randint(118, 126, (N, K // 32), dtype=torch.uint8, device=dev, generator=gen)
@@ -535,6 +535,14 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         mfma(name, 2.0 * M * N * K, N * K // 2 + N * K // 32 + M * K + 4 * M + M * N * 2,
              lambda: check(lib.cfp8_gemm_mxfp4(xq.data_ptr(), K, sxq.data_ptr(), w4.data_ptr(), K // 2, s4.data_ptr(), K // 32,
                                                None, 0, o.data_ptr(), N, 0, M, N, K, stream)), iters=50)
+        if M == 1:
+            # the same layer from bf16 activations: quantisation inside the weight-streaming kernel, one launch
+            # (beside roofline_decode's M1_ms, the FP8 form of the same layer)
+            xb = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
+            mfma(f"linear_mxfp4_{nm}_M{M}", 2.0 * M * N * K, N * K // 2 + N * K // 32 + M * K * 2 + M * N * 2,
+                 lambda: check(lib.cfp8_linear_mxfp4(xb.data_ptr(), K, w4.data_ptr(), K // 2, s4.data_ptr(), K // 32, o.data_ptr(), N, 0,
+                                                     M, N, K, None, 0, stream)), iters=50)
+            del xb
         del w4, s4, xq, sxq, o
 
     # config 5: Qwen3-30B-A3B experts, 8192 tokens routed top-8 over 128 experts

@@ -57,6 +57,8 @@ SIGNATURES = {
     "cfp8_quant_mxfp4": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "cfp8_gemm_mxfp4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                 c_int, c_int64, c_int64, c_int64, c_void_p]),
+    "cfp8_linear_mxfp4": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int, c_int64, c_int64, c_int64,
+                                  c_void_p, c_size_t, c_void_p]),
     "cfp8_gather_quant_group128": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
     "cfp8_scatter_quant_group128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                             c_void_p, c_void_p]),

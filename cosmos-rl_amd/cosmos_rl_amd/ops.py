@@ -365,12 +365,28 @@ def gemm_mxfp4(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Tensor, 
 def linear_mxfp4(x: torch.Tensor, weight: Tuple[torch.Tensor, torch.Tensor],
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """x [..., K] bf16 times MXFP4 weights (codes [N, K/2], scales [N, K/32]): per-token dynamic FP8
-    quantisation of x (as in ``fp8_linear``) followed by ``gemm_mxfp4``."""
+    quantisation of x (as in ``fp8_linear``) and ``gemm_mxfp4``, one launch for up to 4 tokens."""
+    w, ws = weight
+    _need_gpu(x, w, ws)
     K = x.shape[-1]
+    if x.dtype != torch.bfloat16 or w.dtype != torch.uint8 or ws.dtype != torch.uint8 or w.dim() != 2:
+        raise ValueError("expected bf16 activations and uint8 [N, K/2] codes / [N, K/32] scales")
+    N = w.shape[0]
+    if K % 32 or w.shape[1] != K // 2 or tuple(ws.shape) != (N, K // 32):
+        raise ValueError("shape mismatch in MXFP4 linear")
     x2 = x.reshape(-1, K)
-    q, s = quant_rowwise(x2)
-    y = gemm_mxfp4((q, s), weight, out_dtype or x.dtype)
-    return y.reshape(*x.shape[:-1], y.shape[-1])
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    M = x2.shape[0]
+    w, ws = w.contiguous(), ws.contiguous()
+    out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
+    lib = _lib.load()
+    wsb = lib.cfp8_linear_workspace_bytes(M, K)
+    work = torch.empty(max(wsb, 1), dtype=torch.uint8, device=x.device)
+    ld_x = x2.stride(0) if M > 1 else K
+    _lib.check(lib.cfp8_linear_mxfp4(x2.data_ptr(), ld_x, w.data_ptr(), K // 2, ws.data_ptr(), K // 32, out.data_ptr(), N,
+                                     _out_code(out.dtype), M, N, K, work.data_ptr(), wsb, _stream()))
+    return out.reshape(*x.shape[:-1], N)
 
 
 def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -878,6 +878,122 @@ static int launch_mx4_skinny(const Mx4Args& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm_mxfp4");
 }
 
+// The linear layer for at most 4 tokens and K <= 4096 in ONE launch: gemm_mxfp4_gemv_lds_kernel with the per-token FP8
+// quantisation of the bf16 activations folded in.  A workgroup first requests its weights (all of a wave's K steps
+// are in flight before anything else happens), then its 256 threads quantise the tokens together - a thread holds at
+// most two 16-byte vectors of a token between the amax and the cast, the arithmetic of the rowwise quantiser -
+// into LDS, from where the MFMA fragments are read.  Bit-identical to quantising first and calling the kernel above.
+template <int MR, bool OUT_F32>
+__global__ __launch_bounds__(256) void linear_mxfp4_gemv_fused_kernel(const uint4* __restrict__ x, int64_t ldx, const Mx4Args p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // [M][KT * 128 + 16] fp8
+    __shared__ __attribute__((aligned(16))) float red[3 * 64 * 4];
+    __shared__ u32 amax_red[4][MR];
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int KT = (p.K + 127) >> 7;  // <= 32: one pass of kGemvDepth K steps per wave
+    const int pitch = KT * 128 + 16;
+    const int wrow = n0 + lrow;
+    const bool wok = wrow < p.N, xok = lrow < p.M;
+    const uint8_t* const wptr = p.w + (int64_t)(wok ? wrow : 0) * p.ld_w + quarter * 16;
+    const uint8_t* const sptr = p.ws + (int64_t)(wok ? wrow : 0) * p.ld_ws + quarter;
+    u32x4 wv[kGemvDepth];
+    uint32_t sc[kGemvDepth];
+#pragma unroll
+    for (int i = 0; i < kGemvDepth; ++i) {
+        const int kt = wave + 4 * i;
+        const int k = (kt < KT ? kt : 0) << 7;
+        const bool in_w = kt < KT && k + quarter * 32 < p.K;
+        wv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wptr + (in_w ? (k >> 1) : 0)));
+        sc[i] = __builtin_nontemporal_load(sptr + (in_w ? (k >> 5) : 0));
+    }
+    // the tokens (MR >= M of them): amax, scale, cast - rows >= M read row 0 and are never used
+    const int nvec = p.K >> 3, nvec_pad = KT * 16;
+    uint4 v[MR][2];
+    float scale[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        const uint4* xr = x + (int64_t)(r < p.M ? r : 0) * ldx;
+        u32 m = 0;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int idx = t + 256 * j;
+            v[r][j] = idx < nvec ? xr[idx] : make_uint4(0, 0, 0, 0);
+            m = absmax8(m, v[r][j]);
+        }
+        m = wave_max(pk_fold(m));
+        if (lane == 0) amax_red[wave][r] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < MR; ++r) {
+        const u32 m = umax(umax(amax_red[0][r], amax_red[1][r]), umax(amax_red[2][r], amax_red[3][r]));
+        scale[r] = scale_from_amax(amax_from_bits(m));
+        const Divider d(scale[r]);
+        if (r < p.M) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int idx = t + 256 * j;  // vectors between K and the end of the last K step are zero
+                if (idx < nvec_pad) *reinterpret_cast<uint2*>(xs + r * pitch + idx * 8) = idx < nvec ? cast8(v[r][j], d) : make_uint2(0u, 0u);
+            }
+        }
+    }
+    __syncthreads();
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const uint8_t* const xrow = xs + (xok ? lrow : 0) * pitch + quarter * 16;
+#pragma unroll
+    for (int i = 0; i < kGemvDepth; ++i) {
+        const int kt = wave + 4 * i;
+        const int k = (kt < KT ? kt : 0) << 7;
+        const bool in = kt < KT, in_w = in && k + quarter * 32 < p.K;
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(xrow + k), hi = *reinterpret_cast<const u32x4*>(xrow + k + 64);
+        i32x4 fw;
+        i32x8 fx;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            fw[e] = (int)wv[i][e];
+            fx[e] = (in && xok) ? (int)lo[e] : 0;
+            fx[4 + e] = (in && xok) ? (int)hi[e] : 0;
+        }
+        const int scale_w = (in_w && wok) ? (int)sc[i] : 127;
+        acc = mfma_w4a8<0>(fw, fx, acc, scale_w);
+    }
+    if (wave > 0) *reinterpret_cast<f32x4*>(red + ((wave - 1) * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + quarter * 4, m = lrow;
+        if (n < p.N && m < p.M) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) {
+                const f32x4 o = *reinterpret_cast<const f32x4*>(red + (w * 64 + lane) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += o[e];
+            }
+            float sam = scale[0];
+#pragma unroll
+            for (int r = 1; r < MR; ++r) sam = m == r ? scale[r] : sam;
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = acc[e] * sam;
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = o;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+        }
+    }
+}
+
+template <int MR>
+static int launch_linear_mx4_fused_mr(const void* x, int64_t ld_x, const Mx4Args& p, int out_dtype, hipStream_t st) {
+    const unsigned blocks = (unsigned)((p.N + 15) / 16);
+    const size_t lds = (size_t)p.M * ((size_t)((p.K + 127) / 128) * 128 + 16);  // <= 4 x 4112 bytes
+    if (out_dtype == CFP8_OUT_F32)
+        hipLaunchKernelGGL((linear_mxfp4_gemv_fused_kernel<MR, true>), dim3(blocks), dim3(256), lds, st, static_cast<const uint4*>(x), ld_x / 8, p);
+    else
+        hipLaunchKernelGGL((linear_mxfp4_gemv_fused_kernel<MR, false>), dim3(blocks), dim3(256), lds, st, static_cast<const uint4*>(x), ld_x / 8, p);
+    return check_launch("linear_mxfp4");
+}
+
 static int launch_mx4_gemv(const Mx4Args& p, int out_dtype, hipStream_t st) {
     const unsigned blocks = (unsigned)((p.N + 15) / 16);
     const size_t x_lds = (size_t)p.M * ((size_t)((p.K + 127) / 128) * 128 + 16);
@@ -961,4 +1077,50 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
         out16 && (M / 256) * (N / 256) >= 128 && (M / 256) * (N / 256) <= 0x7FFFFFFFll)
         return launch_mx4_256(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
+}
+
+
+namespace cfp8 {
+// quant_rowwise.hip
+int launch_quant_rowwise(const void* x, int64_t rows, int64_t cols, int64_t ld_x, void* q, int64_t ld_q, float* scales,
+                         bool streaming_out, hipStream_t st);
+}  // namespace cfp8
+
+extern "C" int cfp8_linear_mxfp4(const void* x, int64_t ld_x, const void* w, int64_t ld_w, const void* ws, int64_t ld_ws,
+                                 void* out, int64_t ld_out, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+    using namespace cfp8;
+    if (M < 0 || N < 0 || K <= 0) return set_error(CFP8_EINVAL, "linear_mxfp4: bad shape");
+    if (M == 0 || N == 0) return CFP8_OK;
+    if (!x || !aligned16(x) || ld_x % 8 || ld_x < K) return set_error(CFP8_EINVAL, "linear_mxfp4: bad activation pointer or leading dimension");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (M <= 4 && K <= 4096) {
+        // one launch; the checks of cfp8_gemm_mxfp4 that apply to it
+        if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "linear_mxfp4: out_dtype must be CFP8_OUT_BF16 or CFP8_OUT_F32");
+        if (!w || !ws || !out) return set_error(CFP8_EINVAL, "linear_mxfp4: null pointer");
+        if (K % 32 || N % 16) return set_error(CFP8_EINVAL, "linear_mxfp4: K=%lld must be a multiple of 32 and N=%lld a multiple of 16", (long long)K, (long long)N);
+        if (N > 0x7FFFFFFFll || ld_w >= (1ll << 24) || ld_ws >= (1ll << 24) || ld_w < K / 2 || ld_w % 16 || ld_ws < K / 32 || ld_out < N || !aligned16(w))
+            return set_error(CFP8_EINVAL, "linear_mxfp4: pitches: ld_w >= K / 2 bytes and a multiple of 16, ld_ws >= K / 32, ld_out >= N; w 16-byte aligned");
+        const int64_t out_align = out_dtype == CFP8_OUT_F32 ? 16 : 8;
+        if ((reinterpret_cast<uintptr_t>(out) % out_align) || (ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % out_align)
+            return set_error(CFP8_EINVAL, "linear_mxfp4: out must be aligned to four elements and ld_out a multiple of 4");
+        if (int rc = check_device()) return rc;
+        Mx4Args p{};
+        p.w = static_cast<const uint8_t*>(w);
+        p.ws = static_cast<const uint8_t*>(ws);
+        p.out = out;
+        p.ld_w = ld_w; p.ld_ws = ld_ws; p.ld_out = ld_out;
+        p.M = (int)M; p.N = (int)N; p.K = (int)K;
+        if (M == 1) return launch_linear_mx4_fused_mr<1>(x, ld_x, p, out_dtype, st);
+        if (M == 2) return launch_linear_mx4_fused_mr<2>(x, ld_x, p, out_dtype, st);
+        return launch_linear_mx4_fused_mr<4>(x, ld_x, p, out_dtype, st);
+    }
+    if (!workspace || workspace_bytes < cfp8_linear_workspace_bytes(M, K))
+        return set_error(CFP8_EWORKSPACE, "linear_mxfp4: workspace of %zu bytes needed, %zu given", cfp8_linear_workspace_bytes(M, K), workspace_bytes);
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u) return set_error(CFP8_EINVAL, "linear_mxfp4: workspace must be 256-byte aligned");
+    uint8_t* qx = static_cast<uint8_t*>(workspace);
+    float* sx = reinterpret_cast<float*>(qx + (((size_t)M * (size_t)K + 255) & ~(size_t)255));
+    if (int rc = check_device()) return rc;
+    if (int rc = launch_quant_rowwise(x, M, K, ld_x, qx, K, sx, false, st)) return rc;
+    return cfp8_gemm_mxfp4(qx, K, sx, w, ld_w, ws, ld_ws, nullptr, 0, out, ld_out, out_dtype, M, N, K, stream);
 }

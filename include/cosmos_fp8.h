@@ -280,6 +280,17 @@ int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, const void* w,
                     int64_t ld_ws, const int32_t* m_indices, int64_t num_groups, void* out, int64_t ld_out,
                     int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The linear layer on MXFP4 weights from bf16 activations: per-token dynamic FP8 quantisation of x (bf16 [M, K], ld_x in
+ * elements, multiple of 8, x 16-byte aligned; the arithmetic of cfp8_quant_rowwise) followed by cfp8_gemm_mxfp4 on one
+ * weight matrix.  Up to 4 tokens with K <= 4096 run as one launch (the quantisation inside the weight-streaming
+ * kernel, bit-identical to the two steps) and need no workspace; otherwise the quantised activations and their scales
+ * go to `workspace` (device memory, 256-byte aligned, at least cfp8_linear_workspace_bytes(M, K) bytes).  The other
+ * arguments are those of cfp8_gemm_mxfp4.  The counterpart of cfp8_linear_rowwise for the weights of
+ * cosmos_rl/rollout/vllm_rollout/vllm_rollout.py:1000-1045. */
+int cfp8_linear_mxfp4(const void* x, int64_t ld_x, const void* w, int64_t ld_w, const void* ws, int64_t ld_ws,
+                      void* out, int64_t ld_out, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* cfp8_gather_rows followed by cfp8_quant_group128 (CFP8_GROUP_MODE_DIV) as one pass: row r of the
  * output quantises row src_rows[r] of x (bf16 [*, cols], ld_x in elements), a zero row where src_rows[r] < 0.
  * The gathered bf16 matrix [rows_out, cols] that the reference builds with torch indexing before
