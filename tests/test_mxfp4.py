@@ -169,7 +169,8 @@ def _rel(got, want):
                                    (100, 272, 896), (128, 128, 128), (129, 144, 64), (300, 512, 2880), (1000, 400, 1056),
                                    (16, 80, 2880), (2, 528, 4256), (9, 2064, 3584),
                                    (17, 96, 128), (24, 8400, 2880), (31, 176, 6304), (50, 8272, 896), (64, 320, 4096), (64, 18944, 3584), (4096, 8192, 288), (4000, 8208, 160),
-                                   (2048, 4096, 384), (4096, 8192, 128), (2048, 4096, 256), (2560, 3328, 1152)])
+                                   (2048, 4096, 384), (4096, 8192, 128), (2048, 4096, 256), (2560, 3328, 1152),
+                                   (2000, 2064, 2880), (1025, 4112, 160), (8192, 272, 128), (130, 16400, 416), (1024, 4096, 3552)])
 def test_gemm_mxfp4_against_oracle(dev, M, N, K):
     """fp32 output within 1e-4 (relative Frobenius; the fp32 accumulation of the matrix pipe) of the exact sum, bf16 output within 1e-3 of the bf16-rounded
     exact sum; rows and columns beyond M and N of a padded output stay untouched."""
@@ -230,6 +231,36 @@ def test_gemm_mxfp4_grouped(dev):
         want = MX.gemm(xq[sel], sx[sel], wq[e], ws[e])
         assert _rel(out[sel].float(), want.float().to(torch.bfloat16).double()) <= 1e-3, e
     assert bool((out[m_indices < 0] == 7.0).all())
+
+
+@pytest.mark.gpu
+def test_gemm_mxfp4_grouped_large(dev):
+    """Enough tiles for the direct-to-LDS grouped kernel: K = 2880 (a last K step of 64), N with a ragged last tile,
+    an empty expert, experts whose last 128 rows are partly padding; the padding keeps its bytes, bf16 and fp32."""
+    from cosmos_rl_amd import ops
+    g = torch.Generator().manual_seed(10)
+    E, N, K = 6, 1040, 2880
+    counts = [300, 0, 128, 77, 1000, 513]
+    wq, ws = _mx_weights(g, E, N, K)
+    idx, rows = [], 0
+    for e, c in enumerate(counts):
+        padded = -(-c // 128) * 128
+        idx += [e] * c + [-1] * (padded - c)
+        rows += padded
+    m_indices = torch.tensor(idx, dtype=torch.int32)
+    xq, sx = _fp8_rows(g, rows, K)
+    for dt, tol in ((torch.bfloat16, 1e-3), (torch.float32, 1e-4)):
+        out = torch.full((rows, N), 7.0, dtype=dt, device=dev)
+        ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), m_indices=m_indices.to(dev), out=out)
+        out = out.cpu()
+        for e in range(E):
+            sel = m_indices == e
+            if not bool(sel.any()):
+                continue
+            want = MX.gemm(xq[sel], sx[sel], wq[e], ws[e])
+            ref = want.float().to(torch.bfloat16).double() if dt == torch.bfloat16 else want
+            assert _rel(out[sel].float(), ref) <= tol, (e, dt)
+        assert bool((out[m_indices < 0] == 7.0).all())
 
 
 @pytest.mark.gpu
