@@ -1102,6 +1102,267 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_128_kernel(const Mx4Args p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// The kernel above with twice the weight rows: 128 x 512 tiles, four waves, 2 x 2, each a 64 x 256 block = 64
+// accumulators (all 256 AGPRs), i.e. the operand traffic per MFMA of the 256 x 256 kernel on tiles that are only
+// 128 rows high - what the grouped layout allows.  Two activation stages of 16 KiB, three weight stages of 32 KiB,
+// three scale stages of 2 KiB; a K step is four phases of eight groups of two MFMAs (one weight tile against the
+// two activation tiles of a half).  Per wave and step 4 activation + 8 weight + 2 scale loads; the barrier lets the
+// ten newest pass.  Edges and the last K step as above.
+// ---------------------------------------------------------------------------
+#define MX4_MMA2W(wh, xb, xh, g)                                                                             \
+    {                                                                                                        \
+        _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                      \
+            acc[(wh)*8 + (g)][(xh)*2 + e] =                                                                  \
+                mfma_w4a8<0>(W[wh][g], X[xb][e], acc[(wh)*8 + (g)][(xh)*2 + e], (int)S[(wh)*8 + (g)]);      \
+        }                                                                                                    \
+    }
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_mxfp4_128x512_kernel(const Mx4Args p) {
+    constexpr int BM = 128, BN = 512;
+    constexpr int XS = BM * 128, WS = BN * 64, SS = BN * 4;
+    constexpr int WBASE = 2 * XS, SBASE = WBASE + 3 * WS, ABASE = SBASE + 3 * SS;  // + 512 bytes of activation scales
+    constexpr uint32_t kEnd = 0xEFFFFFFFu;  // the longest descriptor: kBeyond stays beyond it
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    if (p.m_indices) mx4_tile_of_block<4>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    else mx4_tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const uint8_t* wmat = p.w;
+    const uint8_t* smat = p.ws;
+    int expert = 0;
+    if (p.m_indices) {
+        expert = p.m_indices[m0];  // groups start on multiples of 128 rows
+        if (expert < 0) return;    // a tile of padding (uniform for the workgroup)
+        wmat += (int64_t)expert * p.N * p.ld_w;
+        smat += (int64_t)expert * p.N * p.ld_ws;
+    }
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = (p.K + 127) >> 7;
+    const int last = KT - 1;
+    const int k_tail = p.K - (last << 7);            // 32 .. 128 elements in the last step
+    const int vq = k_tail >> 5;                      // its valid quarters, 1 .. 4
+
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t w_wave = reinterpret_cast<uint64_t>(wmat) + ((uint64_t)n0 + (uint64_t)wave * 16) * (uint64_t)p.ld_w;
+    uint64_t s_tile = reinterpret_cast<uint64_t>(smat) + (uint64_t)n0 * (uint64_t)p.ld_ws;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, w_step = 64u * (uint32_t)p.ld_w;  // pitches are < 2^24
+    const int64_t a_rows = (int64_t)p.M - m0 - wave * 8, w_rows = (int64_t)p.N - n0 - wave * 16, s_rows = (int64_t)p.N - n0;
+    const int64_t a_left = a_rows > 0 ? a_rows * p.ld_a : 0, w_left = w_rows > 0 ? w_rows * p.ld_w : 0, s_left = s_rows > 0 ? s_rows * p.ld_ws : 0;
+    uint32_t a_end = a_left < (int64_t)kEnd ? (uint32_t)a_left : kEnd, w_end = w_left < (int64_t)kEnd ? (uint32_t)w_left : kEnd,
+             s_end = s_left < (int64_t)kEnd ? (uint32_t)s_left : kEnd;
+    asm volatile("" : "+s"(a_wave), "+s"(w_wave), "+s"(s_tile), "+s"(a_step), "+s"(w_step), "+s"(a_end), "+s"(w_end), "+s"(s_end));
+    const int xc = (lane & 7) ^ ((wave & 1) * 4 + (lane >> 4));
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + (uint32_t)(xc << 4);
+    const uint32_t va_tail = xc * 16 < k_tail ? va_lane : kBeyond;
+    const int wc = (lane & 3) ^ ((lane >> 4) & 3);
+    const uint32_t vw_lane = (uint32_t)(lane >> 2) * (uint32_t)p.ld_w + (uint32_t)(wc << 4);
+    const uint32_t vw_tail = wc * 32 < k_tail ? vw_lane : kBeyond;
+    // scale words: word (2 wave + u) * 64 + lane = wn' * 256 + lrow' * 16 + tile' belongs to row wn' * 256 + tile' * 16 + lrow'
+    uint32_t vs_lane[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int sword = (wave * 2 + u) * 64 + lane;
+        vs_lane[u] = (uint32_t)((sword >> 8) * 256 + (sword & 15) * 16 + ((sword >> 4) & 15)) * (uint32_t)p.ld_ws;
+    }
+    const uint32_t s_last = (uint32_t)(last * 4 - (4 - vq));  // the last step's word ends with the row (K >= 128)
+    const unsigned sshift = 8u * (unsigned)quarter, sshift_tail = 8u * (unsigned)(quarter + 4 - vq);
+    const bool q_in_tail = quarter < vq;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    typedef __attribute__((address_space(3))) void lds_void;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, (int)a_end, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(w_wave), 0, (int)w_end, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(s_tile), 0, (int)s_end, 0x00020000);
+    auto dma_x = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, kt == last ? va_tail : va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    auto dma_w = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16, kt == last ? vw_tail : vw_lane,
+                                                 (uint32_t)i * w_step + ((uint32_t)kt << 6), 0, 0);
+    };
+    auto dma_s = [&](int kt, int stage, int u) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + SBASE + stage * SS + (wave * 2 + u) * 256), 4, vs_lane[u],
+                                                 kt == last ? s_last : (uint32_t)kt << 2, 0, 0);
+    };
+
+    f32x4 acc[16][4];  // [n tile][m tile]
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 64 + lrow) * 128 + ((quarter ^ fsw) << 4);
+    const int x_off2 = (wm * 64 + lrow) * 128 + (((4 + quarter) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 256 + lrow) * 64 + ((quarter ^ ((lrow >> 2) & 3)) << 4);
+    const int s_off = SBASE + (wn * 256 + lrow * 16) * 4;
+    auto xfrag = [&](int stage_bytes, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + x_off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + x_off2);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    auto wfrag = [&](int stage, int tile16) { return *reinterpret_cast<const i32x4*>(smem + stage * WS + tile16 * 1024 + w_off); };
+    auto sfrag = [&](int stage, int part) { return *reinterpret_cast<const u32x4*>(smem + stage * SS + s_off + part * 16); };
+    auto sbyte = [&](uint32_t word, int kt) -> uint32_t {
+        const bool tail = kt == last;
+        const uint32_t b = word >> (tail ? sshift_tail : sshift);
+        return (tail && !q_in_tail) ? 127u : b;
+    };
+    i32x4 W[2][8];
+    i32x8 X[2][2];
+    uint32_t S[16];
+    u32x4 sraw[4];  // scale words of tiles 0-3, 4-7 (the next step's first weight half) and 8-11, 12-15 (its second)
+
+    {
+        const int m = m0 + (wave & 1) * 64 + lane;
+        __builtin_amdgcn_global_load_lds((gbl_void*)(p.sa + (m < p.M ? m : p.M - 1)), (lds_void*)(smem + ABASE + (wave & 1) * 256), 4, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(0, 0, i);
+    dma_s(0, 0, 0);
+    dma_s(0, 0, 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_x(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(1 < last ? 1 : last, 1, i);
+    dma_s(1 < last ? 1 : last, 1, 0);
+    dma_s(1 < last ? 1 : last, 1, 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_w(2 < last ? 2 : last, 2, i);
+    dma_s(2 < last ? 2 : last, 2, 0);
+    dma_s(2 < last ? 2 : last, 2, 1);
+    MX4_WAIT_BARRIER(24);  // the scales and tile 0 (15 loads) have landed; the other 24 stay in flight
+#pragma unroll
+    for (int g = 0; g < 8; ++g) W[0][g] = wfrag(0, g);
+#pragma unroll
+    for (int g = 0; g < 2; ++g) X[0][g] = xfrag(0, g);
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) sraw[q4] = sfrag(0, q4);
+    asm volatile("" : "+v"(sraw[0]), "+v"(sraw[1]), "+v"(sraw[2]), "+v"(sraw[3]));  // four 16-byte reads, not sixteen of four bytes
+#pragma unroll
+    for (int g = 0; g < 8; ++g) S[g] = sbyte(sraw[g >> 2][g & 3], 0);
+    MX4_PHASE_END();
+
+    int ws_cur = 0;  // kt % 3
+    for (int kt = 0; kt < KT; ++kt) {
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ws_cur == 2 ? 0 : ws_cur + 1;
+        const int kw = kt + 3 < last ? kt + 3 : last, kx = kt + 2 < last ? kt + 2 : last;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {  // S0 (w0, x0): reads x1
+            if (g < 2) X[1][g] = xfrag(xs_cur, 2 + g);
+            MX4_MMA2W(0, 0, 0, g);
+            MX4_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {  // S1 (w0, x1): reads w1, scale bytes of w1
+            W[1][g] = wfrag(ws_cur, 8 + g);
+            S[8 + g] = sbyte(sraw[2 + (g >> 2)][g & 3], kt);
+            MX4_MMA2W(0, 1, 1, g);
+            MX4_PHASE_END();
+        }
+        MX4_WAIT_BARRIER(10);
+        MX4_PHASE_END();
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {  // S2 (w1, x0): reads next w0 and the next scale words; loads of activation tile kt + 2
+            W[0][g] = wfrag(ws_nxt, g);  // after the last step: stale data, unused
+            if (g >= 4) {
+                // words 8-15 are shifted into place in S1 of the next step (S[8..15] are still in use)
+                sraw[g - 4] = sfrag(ws_nxt, g - 4);
+                asm volatile("" : "+v"(sraw[g - 4]));
+            }
+            if (g < 4) dma_x(kx, kt & 1, g);
+            MX4_MMA2W(1, 0, 0, g);
+            MX4_PHASE_END();
+        }
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {  // S3 (w1, x1): reads next x0; loads of weight and scale tile kt + 3
+            if (g < 2) X[0][g] = xfrag(xs_nxt, g);
+            dma_w(kw, ws_cur, g);
+            if (g >= 6) dma_s(kw, ws_cur, g - 6);
+            S[g] = sbyte(sraw[g >> 2][g & 3], kt + 1);
+            MX4_MMA2W(1, 1, 1, g);
+            MX4_PHASE_END();
+        }
+        ws_cur = ws_nxt;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the scales have landed, and nothing may still land in the stages
+    __syncthreads();
+    const float* const sa_lds = reinterpret_cast<const float*>(smem + ABASE);
+
+    float sam[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sam[j] = sa_lds[wm * 64 + j * 16 + lrow];
+    if (OUT_F32) {
+        bool keep[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int m = m0 + wm * 64 + j * 16 + lrow;
+            keep[j] = m < p.M;
+            if (p.m_indices && keep[j]) keep[j] = p.m_indices[m] == expert;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int n = n0 + wn * 256 + i * 16 + quarter * 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int m = m0 + wm * 64 + j * 16 + lrow;
+                f32x4 v = acc[i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j];
+                if (keep[j] && n < p.N)
+                    __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: the wave's 64 x 256 block goes through LDS in two halves of 128 columns
+    constexpr int EST = 272;
+    static_assert(4 * 64 * EST <= ABASE, "the epilogue buffers must not reach the activation scales");
+    const int rd_row = lane >> 4, rd_chunk = lane & 15;
+    bool keep[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + r * 4 + rd_row;
+        keep[r] = m < p.M;
+        if (p.m_indices && keep[r]) keep[r] = p.m_indices[m] == expert;
+    }
+    __syncthreads();  // all waves are done reading the operand stages
+    uint8_t* const ebuf = smem + wave * (64 * EST);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                f32x4 v = acc[h * 8 + i][j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * sam[j];
+                *reinterpret_cast<uint2*>(ebuf + (j * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+        const int n = n0 + wn * 256 + h * 128 + rd_chunk * 8;  // N % 16 == 0: a chunk of 8 is inside or outside as a whole
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = r * 4 + rd_row;
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            const int m = m0 + wm * 64 + row;
+            if (keep[r] && n < p.N)
+                __builtin_nontemporal_store(d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n));
+        }
+    }
+}
+
 // more dynamic LDS than the default 64 KiB: the limit is raised once per device and kernel
 static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64]) {
     if (lds <= 64 * 1024) return CFP8_OK;
@@ -1143,6 +1404,21 @@ static int launch_mx4_128(Mx4Args p, int out_dtype, hipStream_t st) {
     if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
     if (f32) hipLaunchKernelGGL(gemm_mxfp4_128_kernel<true>, dim3((unsigned)tiles), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_mxfp4_128_kernel<false>, dim3((unsigned)tiles), dim3(256), lds, st, p);
+    return check_launch("gemm_mxfp4");
+}
+
+static int launch_mx4_128x512(Mx4Args p, int out_dtype, hipStream_t st) {
+    p.tiles_m = (p.M + 127) / 128;
+    p.tiles_n = (p.N + 511) / 512;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    if (tiles > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm_mxfp4: too many tiles");
+    constexpr size_t lds = 2 * 128 * 128 + 3 * 512 * 64 + 3 * 512 * 4 + 512;
+    const bool f32 = out_dtype == CFP8_OUT_F32;
+    static std::atomic<bool> raised[2][64];
+    const void* fn = f32 ? reinterpret_cast<const void*>(gemm_mxfp4_128x512_kernel<true>) : reinterpret_cast<const void*>(gemm_mxfp4_128x512_kernel<false>);
+    if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
+    if (f32) hipLaunchKernelGGL(gemm_mxfp4_128x512_kernel<true>, dim3((unsigned)tiles), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL(gemm_mxfp4_128x512_kernel<false>, dim3((unsigned)tiles), dim3(256), lds, st, p);
     return check_launch("gemm_mxfp4");
 }
 
@@ -1362,6 +1638,9 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
         out16 && (M / 256) * (N / 256) >= 128 && (M / 256) * (N / 256) <= 0x7FFFFFFFll)
         return launch_mx4_256(p, out_dtype, st);
     // every other shape with enough 128 x 256 tiles, and the grouped layout: the same pipeline with edges
+    // (128 x 512 tiles when that still gives every CU a tile and wastes under an eighth of the last tile-column)
+    if (out16 && K >= 128 && (M + 127) / 128 * ((N + 511) / 512) >= 256 && (N + 511) / 512 * 512 - N <= N / 8)
+        return launch_mx4_128x512(p, out_dtype, st);
     if (out16 && K >= 128 && (M + 127) / 128 * ((N + 255) / 256) >= 64) return launch_mx4_128(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
 }

@@ -170,7 +170,8 @@ def _rel(got, want):
                                    (16, 80, 2880), (2, 528, 4256), (9, 2064, 3584),
                                    (17, 96, 128), (24, 8400, 2880), (31, 176, 6304), (50, 8272, 896), (64, 320, 4096), (64, 18944, 3584), (4096, 8192, 288), (4000, 8208, 160),
                                    (2048, 4096, 384), (4096, 8192, 128), (2048, 4096, 256), (2560, 3328, 1152),
-                                   (2000, 2064, 2880), (1025, 4112, 160), (8192, 272, 128), (130, 16400, 416), (1024, 4096, 3552)])
+                                   (2000, 2064, 2880), (1025, 4112, 160), (8192, 272, 128), (130, 16400, 416), (1024, 4096, 3552),
+                                   (4000, 4112, 160), (8192, 2544, 416), (4100, 4096, 2880)])
 def test_gemm_mxfp4_against_oracle(dev, M, N, K):
     """fp32 output within 1e-4 (relative Frobenius; the fp32 accumulation of the matrix pipe) of the exact sum, bf16 output within 1e-3 of the bf16-rounded
     exact sum; rows and columns beyond M and N of a padded output stay untouched."""
@@ -234,13 +235,14 @@ def test_gemm_mxfp4_grouped(dev):
 
 
 @pytest.mark.gpu
-def test_gemm_mxfp4_grouped_large(dev):
-    """Enough tiles for the direct-to-LDS grouped kernel: K = 2880 (a last K step of 64), N with a ragged last tile,
+@pytest.mark.parametrize("N,K,counts", [(1040, 2880, [300, 0, 128, 77, 1000, 513]),          # 128 x 256 tiles
+                                        (1520, 1120, [3000, 0, 128, 77, 5000, 2600])])       # 128 x 512 tiles
+def test_gemm_mxfp4_grouped_large(dev, N, K, counts):
+    """Enough tiles for the direct-to-LDS grouped kernels: a last K step of 64 or 96, N with a ragged last tile,
     an empty expert, experts whose last 128 rows are partly padding; the padding keeps its bytes, bf16 and fp32."""
     from cosmos_rl_amd import ops
     g = torch.Generator().manual_seed(10)
-    E, N, K = 6, 1040, 2880
-    counts = [300, 0, 128, 77, 1000, 513]
+    E = len(counts)
     wq, ws = _mx_weights(g, E, N, K)
     idx, rows = [], 0
     for e, c in enumerate(counts):
