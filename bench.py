@@ -545,6 +545,34 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
             del xb
         del w4, s4, xq, sxq, o
 
+    # the grouped form on the expert shapes of GPT-OSS-20B: 32 experts, 8192 tokens routed top-4, gate_up [5760, 2880]
+    # (K = 2880 is not a multiple of 128, N = 5760 not one of 512: the last K step and the last tile-column are ragged)
+    name = "gemm_mxfp4_grouped_gptoss20b_gate_up"
+    if not only or only in name:
+        EX, NX, KX2, TX, TOPX = 32, 5760, 2880, 8192, 4
+        logits = torch.rand(TX, EX, generator=gen, device=dev)
+        topi = torch.topk(logits, TOPX, dim=1).indices.reshape(-1)
+        counts = torch.bincount(topi, minlength=EX)
+        padded = torch.clamp_min(((counts + 127) // 128) * 128, 128)
+        offs = torch.cumsum(padded, 0)
+        total = int(offs[-1])
+        rows = torch.arange(total, device=dev)
+        e_of_row = torch.searchsorted(offs, rows, right=True)
+        start = offs - padded
+        m_idx = torch.where(rows - start[e_of_row] < counts[e_of_row], e_of_row, torch.full_like(e_of_row, -1)).to(torch.int32)
+        routed = int(counts.sum())
+        w4 = torch.randint(0, 256, (EX, NX, KX2 // 2), dtype=torch.uint8, device=dev, generator=gen)
+        s4 = torch.randint(118, 126, (EX, NX, KX2 // 32), dtype=torch.uint8, device=dev, generator=gen)
+        xq = torch.randn(total, KX2, generator=gen, device=dev).mul_(60).to(torch.float8_e4m3fn)
+        sxq = torch.rand(total, generator=gen, device=dev) + 0.5
+        o = torch.zeros(total, NX, dtype=torch.bfloat16, device=dev)
+        mfma(name, 2.0 * routed * NX * KX2, EX * NX * (KX2 // 2 + KX2 // 32) + routed * (KX2 + 4 + NX * 2),
+             lambda: check(lib.cfp8_gemm_mxfp4(xq.data_ptr(), KX2, sxq.data_ptr(), w4.data_ptr(), KX2 // 2, s4.data_ptr(), KX2 // 32,
+                                               m_idx.data_ptr(), EX, o.data_ptr(), NX, 0, total, NX, KX2, stream)), iters=30)
+        out[name]["routed_rows"] = routed
+        out[name]["padded_rows"] = total
+        del w4, s4, xq, sxq, o, m_idx, logits, topi
+
     # config 5: Qwen3-30B-A3B experts, 8192 tokens routed top-8 over 128 experts
     E, H, I, T, TOPK = 128, 2048, 768, 8192, 8
     wgu = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).normal_(0, 0.02, generator=gen)
