@@ -188,6 +188,27 @@ def test_gemm_mxfp4_against_oracle(dev, M, N, K):
 
 
 @pytest.mark.gpu
+def test_gemm_mxfp4_random_shapes_every_kernel_form(dev):
+    """Seeded random shapes across the dispatch boundaries (1..16 tokens, 17..64, small register-staged tiles, ragged
+    and aligned direct-to-LDS tiles, K with and without a partial last step), fp32 output against the exact sum."""
+    from cosmos_rl_amd import ops
+    rng = np.random.default_rng(11)
+    shapes = []
+    for _ in range(8):
+        shapes.append((int(rng.integers(1, 17)), 16 * int(rng.integers(1, 600)), 32 * int(rng.integers(1, 140))))
+        shapes.append((int(rng.integers(17, 65)), 16 * int(rng.integers(1, 600)), 32 * int(rng.integers(1, 140))))
+        shapes.append((int(rng.integers(65, 700)), 16 * int(rng.integers(1, 80)), 32 * int(rng.integers(1, 100))))
+        shapes.append((int(rng.integers(700, 5000)), 16 * int(rng.integers(100, 400)), 32 * int(rng.integers(4, 40))))
+    shapes += [(256 * int(rng.integers(8, 20)), 256 * int(rng.integers(16, 30)), 128 * int(rng.integers(1, 8))) for _ in range(3)]
+    g = torch.Generator().manual_seed(12)
+    for M, N, K in shapes:
+        wq, ws = _mx_weights(g, N, K)
+        xq, sx = _fp8_rows(g, M, K)
+        got = ops.gemm_mxfp4((xq.to(dev), sx.to(dev)), (wq.to(dev), ws.to(dev)), torch.float32)
+        assert _rel(got.cpu(), MX.gemm(xq, sx, wq, ws)) <= 1e-4, (M, N, K)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("M", [8, 160])
 def test_gemm_mxfp4_one_hot_is_exact(dev, M):
     """Row m of the activations is 1.0 at k = m (mod K): the output is the weight value itself, so the nibble
