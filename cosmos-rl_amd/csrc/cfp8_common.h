@@ -75,11 +75,11 @@ __device__ __forceinline__ float scale_from_amax(float amax) {
 }
 
 // Per reduction set divider.  x / s is needed correctly rounded (the bytes must
-// equal those of an IEEE fp32 division followed by an RNE cast).  With r = 1/s
-// correctly rounded, q0 = x*r, e = fma(-q0, s, x), q1 = fma(e, r, q0) is the
-// correctly rounded quotient wherever it is a normal number (Markstein); below
-// 2^-11 every quotient rounds to a zero byte and only the sign matters, which
-// copysign restores.  Non-finite scales (amax Inf or NaN) take the slow path.
+// equal those of an IEEE fp32 division followed by a clamp to +-448 and an RNE cast).
+// With r = 1/s correctly rounded, q0 = x*r, e = fma(q0, s, -x), q1 = fma(-e, r, q0) is
+// the correctly rounded quotient wherever it is a normal number (Markstein); below
+// 2^-11 every quotient rounds to a zero byte and only the sign matters, which this
+// form of the residual keeps.  Non-finite scales (amax Inf or NaN) take the slow path.
 struct Divider {
     float s, r;
     bool finite;
@@ -88,13 +88,17 @@ struct Divider {
         finite = (__float_as_uint(scale) & 0x7F800000u) != 0x7F800000u;
         r = 1.0f / scale;
     }
-    // quotient clamped to +-448; valid for finite x when `finite`
+    // The correctly rounded quotient x / s for finite x when `finite`, for the callers of this library: s is the
+    // amax / 448 (amax floored at 1e-12) of a set that x belongs to, so |x / s| <= 448 * (1 + 2^-22) - the quotient
+    // of the largest element is 448 or the fp32 value next to it - which is below 464 and which the conversion to
+    // e4m3 rounds to at most 448 by itself: no clamp.  Reciprocal, product, residual, correction; the residual is
+    // formed with the opposite sign, e = q0 * s - x, and subtracted, so that a zero keeps the sign of x without a
+    // copysign (x = -0: q0 = -0, e = +0, (-e) * r + q0 = -0 + -0 = -0; x = +0: e = +0, -0 + +0 = +0; a q0 that
+    // underflowed to a signed zero is met by (-e) * r = x * r of the same sign).
     __device__ __forceinline__ float fast(float x) const {
         float q0 = x * r;
-        float e = __builtin_fmaf(-q0, s, x);
-        float q1 = __builtin_fmaf(e, r, q0);
-        q1 = __builtin_copysignf(q1, x);
-        return __builtin_amdgcn_fmed3f(q1, -kE4M3Max, kE4M3Max);
+        float e = __builtin_fmaf(q0, s, -x);
+        return __builtin_fmaf(-e, r, q0);
     }
 };
 

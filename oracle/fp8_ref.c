@@ -263,14 +263,14 @@ void fp8ref_combine_rows(const uint16_t* rows, int64_t H, const int32_t* row_map
         }
 }
 
-/* Division shortcut used by the kernels: r = 1/s (IEEE), q0 = x*r,
- * e = fma(-q0, s, x), q1 = copysign(fma(e, r, q0), x).  Returns the number of (x, s) pairs,
- * x over all 65536 bf16 patterns with |x| <= amax(s) := 448*s-ish bound lifted
- * (all finite x with |x/s| <= 1024 are checked), for which q1 != x / s bitwise
- * AND the e4m3 byte of the clamped value differs.  *fp32_mismatch receives the
- * count of fp32-level mismatches with |x/s| >= 2^-11, i.e. everywhere the
- * quotient can still round to a non-zero byte (below that only the sign
- * survives, which copysign restores). */
+/* Division shortcut used by the kernels: r = 1/s (IEEE), q0 = x*r, e = fma(q0, s, -x),
+ * q1 = fma(-e, r, q0), the byte is the e4m3 conversion of q1 WITHOUT a clamp.  The kernels only
+ * divide by the scale of a set that x belongs to, so |x/s| <= 448 * (1 + 2^-22) there; every
+ * finite bf16 x with an IEEE quotient in that range is checked.  Returns the number of (x, s)
+ * pairs whose byte differs from the byte of the clamped IEEE quotient (signed zeros included:
+ * the byte carries the sign).  *fp32_mismatch receives the count of pairs with
+ * |x/s| >= 2^-11 - everywhere the quotient can still round to a non-zero byte - whose q1 is not
+ * the IEEE quotient bit for bit. */
 int64_t fp8ref_check_fast_div(const float* scales, int64_t n, int64_t* fp32_mismatch) {
     int64_t bad = 0, soft = 0;
     for (int64_t i = 0; i < n; ++i) {
@@ -280,16 +280,13 @@ int64_t fp8ref_check_fast_div(const float* scales, int64_t n, int64_t* fp32_mism
             float x = bf16_to_f32((uint16_t)h);
             if (x != x || isinf(x)) continue;
             float want = x / s;
-            if (!(fabsf(want) <= 1024.0f)) continue;
+            if (!(fabsf(want) <= 448.0f * (1.0f + 0x1p-22f))) continue;
             float q0 = x * r;
-            float e = fmaf(-q0, s, x);
-            float q1 = copysignf(fmaf(e, r, q0), x);
-            if (f32_bits(q1) != f32_bits(want)) {
-                if (fabsf(want) >= 0x1p-11f) ++soft;
-                float a = want > 448.f ? 448.f : (want < -448.f ? -448.f : want);
-                float b = q1 > 448.f ? 448.f : (q1 < -448.f ? -448.f : q1);
-                if (fp8ref_e4m3_from_f32(a) != fp8ref_e4m3_from_f32(b)) ++bad;
-            }
+            float e = fmaf(q0, s, -x);
+            float q1 = fmaf(-e, r, q0);
+            if (f32_bits(q1) != f32_bits(want) && fabsf(want) >= 0x1p-11f) ++soft;
+            float a = want > 448.f ? 448.f : (want < -448.f ? -448.f : want);
+            if (fp8ref_e4m3_from_f32(a) != fp8ref_e4m3_from_f32(q1)) ++bad;
         }
     }
     if (fp32_mismatch) *fp32_mismatch = soft;

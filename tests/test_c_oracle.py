@@ -118,14 +118,15 @@ def test_block_and_group_agree():
 
 
 def test_division_shortcut_is_exact():
-    """r = 1/s; q0 = x*r; e = fma(-q0, s, x); q1 = copysign(fma(e, r, q0), x) equals the IEEE
-    quotient x/s bit for bit wherever |x/s| >= 2^-11, and gives the same e4m3 byte everywhere,
-    for all 65536 bf16 x and 1500 scales spanning the fp32 range."""
+    """r = 1/s; q0 = x*r; e = fma(q0, s, -x); q1 = fma(-e, r, q0) equals the IEEE quotient x/s bit for bit wherever
+    |x/s| >= 2^-11, and its e4m3 byte - converted without a clamp - is the byte of the clamped IEEE quotient, signed
+    zeros included, for all bf16 x with |x/s| <= 448 (1 + 2^-22) (a scale is the amax / 448 of a set x belongs to) and
+    1500 scales spanning the fp32 range; among them amax values whose own quotient is the fp32 value above 448."""
     g = torch.Generator().manual_seed(0)
     pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
     pos = pats[(pats > 0) & torch.isfinite(pats)]
     amax = torch.cat([torch.rand(500, generator=g) * 2, torch.exp(torch.rand(500, generator=g) * 170 - 85).clamp(max=3e38),
-                      pos[::66], torch.tensor([0.0, 1e-12, 1e-13, 3.3895e38, 448.0])])
+                      pos[::66], torch.tensor([0.0, 1e-12, 1e-13, 3.3895e38, 448.0, 0.00799560546875, 0.0084228515625])])
     scales = O.scale_from_amax(amax).numpy()
     bad, soft = C.check_fast_div(scales)
     assert bad == 0 and soft == 0

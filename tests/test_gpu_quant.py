@@ -314,6 +314,11 @@ def test_tensorwise_read_once_launch(dev):
     g = torch.Generator(device=dev).manual_seed(77)
     shapes = [(18944, 3584), (512, 3584), (14336, 4096), (3584, 3584), (3584, 18944), (13568, 4096), (17280, 4096)]
     ws = [(torch.randn(sh, generator=g, device=dev) * (0.01 * (i + 1))).to(torch.bfloat16) for i, sh in enumerate(shapes)]
+    # amax = 0.00799560546875: fp32(amax / fp32(amax / 448)) is 448.0000305, the value next to 448 - the resident
+    # kernel's cast has no clamp and relies on the conversion to round that to 448
+    ws[0].clamp_(-0.0079, 0.0079)
+    ws[0][0, 0], ws[0][18943, 3583], ws[0][9000, 77] = 0.00799560546875, -0.00799560546875, 0.00799560546875
+    ws[0][5, 5], ws[0][5, 6] = -0.0, 0.0     # signed zeros keep their sign (bytes 0x80 and 0x00)
     ws[2][7000, 123] = float("inf")          # non-finite scale in a tensor that is kept on the chip
     ws[4][11, 18000] = float("nan")
     ws[5].zero_()                             # amax 0: the scale floor
@@ -328,6 +333,9 @@ def test_tensorwise_read_once_launch(dev):
         assert_scales(scales[i:i + 1], so, f"tensor {i} scale")
         assert_bytes(qs[i], qo, f"tensor {i} bytes")
     assert int(bits(scales)[5]) == 0x2720D7C5 and int(u8(qs[5]).max()) == 0
+    assert [int(u8(qs[0])[i, j]) for i, j in ((0, 0), (18943, 3583), (9000, 77))] == [0x7E, 0xFE, 0x7E]
+    assert float(ws[0][0, 0].float().cpu() / scales[0].cpu()) > 448.0
+    assert int(u8(qs[0])[5, 5]) == 0x80 and int(u8(qs[0])[5, 6]) == 0x00
     # the counters and maxima live in the workspace of the call: a second call starts from zero again
     qs_b, scales_b = ops.quant_tensorwise_multi(ws)
     assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, qs_b)) and torch.equal(bits(scales), bits(scales_b))
