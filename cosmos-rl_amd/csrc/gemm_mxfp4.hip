@@ -1639,7 +1639,8 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
         return launch_mx4_256(p, out_dtype, st);
     // every other shape with enough 128 x 256 tiles, and the grouped layout: the same pipeline with edges
     // (128 x 512 tiles when that still gives every CU a tile and wastes under an eighth of the last tile-column)
-    if (out16 && K >= 128 && (M + 127) / 128 * ((N + 511) / 512) >= 256 && (N + 511) / 512 * 512 - N <= N / 8)
+    // (its byte offsets inside a tile reach 463 weight rows: the pitch must stay below 2^23 for 32 bits)
+    if (out16 && K >= 128 && ld_w < (1ll << 23) && (M + 127) / 128 * ((N + 511) / 512) >= 256 && (N + 511) / 512 * 512 - N <= N / 8)
         return launch_mx4_128x512(p, out_dtype, st);
     if (out16 && K >= 128 && (M + 127) / 128 * ((N + 255) / 256) >= 64) return launch_mx4_128(p, out_dtype, st);
     return launch_mx4<128, 128, 2, 2, 1>(p, out_dtype, st);
