@@ -1918,6 +1918,175 @@ static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// ---------------------------------------------------------------------------
+// Rowwise GEMM for 17..128 tokens (batched decode): a strip kernel.  A workgroup of four waves owns all BM (64 or
+// 128) token rows and BN = 16 TN weight rows (80, or 32 for a narrow weight) over the whole of K, so the weight is
+// read once by ~N / 80 workgroups - one per CU for an 18944-row weight.  Both operand tiles of a K step go from
+// global memory straight into LDS (buffer_load ... lds, the row-major XOR-swizzled layout of the 256 x 256 kernel) in
+// a ring of S stages; step kt waits for tile kt, requests tile kt + S - 1 into the stage that step kt - 1 used, and
+// computes: one barrier per step, kStripLoads = BM / 32 + ceil(BN / 32) loads per wave and step, the barrier lets the
+// loads of the S - 2 tiles in between pass.  What is in flight is therefore S - 1 steps of both operands: the ring
+// is as deep as the LDS allows (BM = 64: 8 stages, 70 KB of weights in flight per CU; BM = 128: 5 stages).
+// Rows beyond M and N are not fetched: the descriptors end with the matrix and a direct-to-LDS load writes zero for a
+// lane beyond its descriptor.  Wave w computes token rows w BM / 4 ... against all TN weight tiles.
+// ---------------------------------------------------------------------------
+template <int BM, int TN, bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs p) {
+    constexpr int BN = TN * 16;
+    constexpr int WROWS = (BN + 31) / 32 * 32;          // weight rows requested per step: 8 per wave and load
+    constexpr int LX = BM / 32, LW = WROWS / 32;        // loads per wave and step
+    constexpr int XS = BM * 128, WS = WROWS * 128;
+    constexpr int S = BM == 64 ? 8 : 5;                 // ring depth: what the LDS holds (160 / 140 KiB)
+    constexpr int XT = BM / 64;                         // token tiles per wave
+    constexpr uint32_t kEnd = 0xEFFFFFFFu;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // S activation stages, then S weight stages
+    constexpr int WBASE = S * XS;
+    // token blocks of one weight strip are neighbours in the grid: they run at the same time and the second reads the
+    // strip from the caches
+    const int m0 = (int)(blockIdx.x % (unsigned)p.tiles_m) * BM, n0 = (int)(blockIdx.x / (unsigned)p.tiles_m) * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, b_step = 32u * (uint32_t)p.ld_b;  // leading dimensions are < 2^24
+    const int64_t a_rows = (int64_t)p.M - m0 - wave * 8, b_rows = (int64_t)p.N - n0 - wave * 8;
+    const int64_t a_left = a_rows > 0 ? a_rows * p.ld_a : 0, b_left = b_rows > 0 ? b_rows * p.ld_b : 0;
+    uint32_t a_end = a_left < (int64_t)kEnd ? (uint32_t)a_left : kEnd, b_end = b_left < (int64_t)kEnd ? (uint32_t)b_left : kEnd;
+    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step), "+s"(a_end), "+s"(b_end));
+    // load i covers rows (wave + 4 i) * 8 .. + 7; (r >> 1) & 7 of row r = (wave + 4 i) * 8 + (lane >> 3) is (wave & 1) * 4 + (lane >> 4)
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(3))) void lds_void;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, (int)a_end, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(b_wave), 0, (int)b_end, 0x00020000);
+    auto dma = [&](int kt, int stage) {
+#pragma unroll
+        for (int i = 0; i < LX; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, va_lane,
+                                                     (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+#pragma unroll
+        for (int i = 0; i < LW; ++i)  // the rows of the last load that lie beyond BN are not fetched (zeros nobody reads)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16,
+                                                     (wave + 4 * i) * 8 < BN ? vb_lane : 0xF0000000u,
+                                                     (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 2);
+    };
+
+    // the scales of the epilogue first: they are the oldest loads, every later wait covers them
+    float sam[XT];
+    f32x4 sbn[TN];
+#pragma unroll
+    for (int j = 0; j < XT; ++j) {
+        const int m = m0 + wave * (BM / 4) + j * 16 + lrow;
+        sam[j] = p.sa[m < p.M ? m : p.M - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        const int n = n0 + i * 16 + quarter * 4;
+        sbn[i] = *reinterpret_cast<const f32x4*>(p.sb + (n < p.N ? n : 0));
+    }
+
+    f32x4 acc[TN][XT];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < XT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wave * (BM / 4) + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wave * (BM / 4) + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + lrow * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + lrow * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+#pragma unroll
+    for (int d = 0; d < S - 1; ++d) dma(d < last ? d : last, d);
+    int cur = 0;  // kt % S
+    for (int kt = 0; kt < KT; ++kt) {
+        // tile kt has landed when at most the loads of the S - 2 tiles behind it are outstanding; after the barrier
+        // nobody reads the stage of step kt - 1 any more
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * (LX + LW)) : "memory");
+        const int nxt = cur == 0 ? S - 1 : cur - 1;  // (kt + S - 1) % S
+        dma(kt + S - 1 < last ? kt + S - 1 : last, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        i32x8 wf[TN];
+#pragma unroll
+        for (int i = 0; i < TN; ++i) wf[i] = frag(cur * WS, w_off, w_off2, i);
+#pragma unroll
+        for (int j = 0; j < XT; ++j) {
+            const i32x8 xf = frag(cur * XS, x_off, x_off2, j);
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[i], xf, acc[i][j], 0, 0, 0, 0, 0, 0);
+        }
+        // the MFMAs are pure functions of registers: pinned here, or the compiler may move them past the next barrier
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < XT; ++j) asm volatile("" : "+v"(acc[i][j]));
+        cur = cur == S - 1 ? 0 : cur + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS once the workgroup has gone
+
+#pragma unroll
+    for (int j = 0; j < XT; ++j) {
+        const int m = m0 + wave * (BM / 4) + j * 16 + lrow;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int n = n0 + i * 16 + quarter * 4;
+            if (n >= p.N) continue;  // N % 16 == 0: a group of four is inside or outside as a whole
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e] * sam[j] * sbn[i][e];
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+    }
+}
+
+template <int BM, int TN>
+static int launch_rowwise_strip_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
+    constexpr int BN = TN * 16, WROWS = (BN + 31) / 32 * 32, S = BM == 64 ? 8 : 5;
+    constexpr size_t lds = (size_t)S * (BM + WROWS) * 128;
+    static_assert(lds <= 160 * 1024, "strip kernel LDS");
+    p.tiles_m = (p.M + BM - 1) / BM;
+    const int64_t blocks = (p.N + BN - 1) / BN * p.tiles_m;
+    static std::atomic<bool> raised[65][2];
+    const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
+    const void* fn = v ? reinterpret_cast<const void*>(gemm_rowwise_strip_kernel<BM, TN, true>)
+                       : reinterpret_cast<const void*>(gemm_rowwise_strip_kernel<BM, TN, false>);
+    const int slot = device_slot();
+    if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
+    {
+        char name[64];
+        snprintf(name, sizeof(name), "gemm_rowwise_strip<%d,%d>", BM, TN);
+        if (!note_launch(name, (unsigned)blocks, 256, lds)) return CFP8_OK;
+    }
+    if (v) hipLaunchKernelGGL((gemm_rowwise_strip_kernel<BM, TN, true>), dim3((unsigned)blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL((gemm_rowwise_strip_kernel<BM, TN, false>), dim3((unsigned)blocks), dim3(256), lds, st, p);
+    return check_launch("gemm");
+}
+// 17..128 tokens; 80 weight rows per workgroup unless that leaves most CUs without one.  (129..256 tokens as two token
+// blocks on strips of 160 rows, still one workgroup per CU for an 18944-row weight, measured 41 against 48 us for the
+// 256 x 128 tiles at 256 tokens: four ring stages and as many LDS cycles as MFMA cycles per step; not kept.)
+static int launch_rowwise_strip(GemmArgs& p, int out_dtype, hipStream_t st) {
+    const bool narrow = (p.N + 79) / 80 < 128;
+    if (p.M <= 64) return narrow ? launch_rowwise_strip_cfg<64, 2>(p, out_dtype, st) : launch_rowwise_strip_cfg<64, 5>(p, out_dtype, st);
+    return narrow ? launch_rowwise_strip_cfg<128, 2>(p, out_dtype, st) : launch_rowwise_strip_cfg<128, 5>(p, out_dtype, st);
+}
+
 // Sum of the K slices in slice order, scales, conversion: out[m, n] = (sum_s partial[s, m, n]) * sa[m] * sb[n]
 template <bool OUT_F32>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int slices, int M, int N,
@@ -2551,10 +2720,12 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
             return launch_cfg<128, 256, 2, 4, kGrouped>(p, out_dtype, st);
         return launch_cfg<128, 128, 2, 2, kGrouped>(p, out_dtype, st);
     }
-    if (MODE == kRowwise && p.M <= 64) {
-        if (p.M <= 16) return launch_rowwise_gemv(p, out_dtype, st);
-        if (p.M <= 32) return launch_rowwise_skinny<2>(p, out_dtype, st);
-        return launch_rowwise_skinny<4>(p, out_dtype, st);
+    if (MODE == kRowwise && p.M <= 16) return launch_rowwise_gemv(p, out_dtype, st);
+    if (MODE == kRowwise && p.M <= 128) {
+        // a narrow weight with a long K is cut into K slices (the skinny kernels, at most 64 tokens); everything else
+        // of 17..128 tokens takes the strip kernel
+        if (p.M <= 64 && pick_k_slices(p, 4) > 1) return p.M <= 32 ? launch_rowwise_skinny<2>(p, out_dtype, st) : launch_rowwise_skinny<4>(p, out_dtype, st);
+        return launch_rowwise_strip(p, out_dtype, st);
     }
     if (p.M <= 16) return launch_cfg<16, 64, 1, 4, MODE>(p, out_dtype, st);
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);

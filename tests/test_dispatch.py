@@ -30,7 +30,10 @@ CASES = [
      "gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
     ("cfg3 M=1024", (ROW, 1024, 18944, 3584),
      f"gemm_rowwise_256 grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=160 block=256 lds=65536"),
-    ("cfg3 M=64", (LIN, 64, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_skinny<4,5> k_slices=1 grid=237 block=640 lds=131072"),
+    ("cfg3 M=64", (LIN, 64, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),
+    ("cfg3 M=17", (LIN, 17, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),
+    ("cfg3 M=128", (LIN, 128, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<128,5> grid=237 block=256 lds=143360"),
+    ("qkv M=100: a narrow weight takes 32-row strips", (LIN, 100, 4608, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<128,2> grid=144 block=256 lds=102400"),
     ("cfg3 M=1", (LIN, 1, 18944, 3584), "linear_gemv_fused grid=1184 block=256 lds=3584"),
     ("cfg3 M=16", (LIN, 16, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_gemv grid=1184 block=256 lds=0"),
     ("down projection M=64, split-K workspace", (LIN, 64, 3584, 18944, L.OUT_BF16, 256, True),

@@ -55,10 +55,13 @@ def rowwise_operands(M, N, K, seed, dev):
                                    (2048, 8448, 256),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
                                    (1000, 512, 384), (520, 256, 256),
-                                   # 17..64 tokens: the weight streamer with 32, 48, 64, 80, 96 and 128 weight rows per
-                                   # workgroup (chosen from N), ragged last workgroup, K of 1, 3, 8 and 9 steps
+                                   # 17..64 tokens: the strip kernel with 32 or 80 weight rows per workgroup (chosen from
+                                   # N), ragged last workgroup, K of 1, 3, 8 and 9 steps (fewer and more than the ring holds)
                                    (40, 528, 1152), (20, 8208, 128), (64, 12272, 384), (33, 16400, 1024), (64, 20016, 128),
-                                   (18, 24592, 256), (50, 28688, 128), (32, 40976, 128)])
+                                   (18, 24592, 256), (50, 28688, 128), (32, 40976, 128),
+                                   # 65..128 tokens: its 128-row form, ring of five stages, K of 1, 3, 5, 9 and 28 steps
+                                   (65, 12272, 384), (128, 16400, 1152), (100, 20016, 128), (127, 10480, 640), (96, 18944, 3584),
+                                   (128, 4608, 896)])
 def test_scaled_mm_rowwise(dev, M, N, K):
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
     ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
