@@ -1363,6 +1363,150 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_128x512_kernel(const Mx4Args p
     }
 }
 
+// ---------------------------------------------------------------------------
+// 17..128 tokens (batched decode) on one weight matrix: a strip kernel.  A workgroup of four waves owns all BM (64 or
+// 128) token rows and 80 weight rows over the whole of K, so the weight is read once by N / 80 workgroups - one per CU
+// for an 18944-row weight.  Activation tile, weight codes and scale words of a K step go straight into LDS in a ring
+// of S stages (9 for 64 rows, 6 for 128: all the LDS holds); step kt waits for tile kt, requests tile kt + S - 1 into
+// the stage that step kt - 1 used, and computes: one barrier per step, BM / 32 activation + 2 weight + 1 scale loads
+// per wave and step, the barrier lets the loads of the S - 2 tiles in between pass.  Wave w computes token rows
+// w BM / 4 ... against the five weight tiles.  Edges and the last K step as in the 128 x 256 kernel.
+// ---------------------------------------------------------------------------
+template <int BM, bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_mxfp4_strip_kernel(const Mx4Args p) {
+    constexpr int TN = 5, BN = TN * 16;
+    constexpr int LX = BM / 32, L = LX + 3;             // loads per wave and step
+    constexpr int XS = BM * 128, WS = 8 * 1024, SS = 1024;  // a weight stage holds 8 groups of 16 rows x 64 bytes, 5 are used
+    constexpr int S = BM == 64 ? 9 : 6;
+    constexpr int XT = BM / 64;
+    constexpr int WBASE = S * XS, SBASE = WBASE + S * WS;
+    constexpr uint32_t kEnd = 0xEFFFFFFFu;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int m0 = (int)(blockIdx.x % (unsigned)p.tiles_m) * BM, n0 = (int)(blockIdx.x / (unsigned)p.tiles_m) * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = (p.K + 127) >> 7;
+    const int last = KT - 1;
+    const int k_tail = p.K - (last << 7);
+    const int vq = k_tail >> 5;
+
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t w_wave = reinterpret_cast<uint64_t>(p.w) + ((uint64_t)n0 + (uint64_t)wave * 16) * (uint64_t)p.ld_w;
+    uint64_t s_tile = reinterpret_cast<uint64_t>(p.ws) + (uint64_t)n0 * (uint64_t)p.ld_ws;
+    uint32_t a_step = 32u * (uint32_t)p.ld_a, w_step = 64u * (uint32_t)p.ld_w;
+    const int64_t a_rows = (int64_t)p.M - m0 - wave * 8, w_rows = (int64_t)p.N - n0 - wave * 16, s_rows = (int64_t)p.N - n0;
+    const int64_t a_left = a_rows > 0 ? a_rows * p.ld_a : 0, w_left = w_rows > 0 ? w_rows * p.ld_w : 0, s_left = s_rows > 0 ? s_rows * p.ld_ws : 0;
+    uint32_t a_end = a_left < (int64_t)kEnd ? (uint32_t)a_left : kEnd, w_end = w_left < (int64_t)kEnd ? (uint32_t)w_left : kEnd,
+             s_end = s_left < (int64_t)kEnd ? (uint32_t)s_left : kEnd;
+    asm volatile("" : "+s"(a_wave), "+s"(w_wave), "+s"(s_tile), "+s"(a_step), "+s"(w_step), "+s"(a_end), "+s"(w_end), "+s"(s_end));
+    const int xc = (lane & 7) ^ ((wave & 1) * 4 + (lane >> 4));
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + (uint32_t)(xc << 4);
+    const uint32_t va_tail = xc * 16 < k_tail ? va_lane : kBeyond;
+    const int wc = (lane & 3) ^ ((lane >> 4) & 3);
+    const uint32_t vw_lane = (uint32_t)(lane >> 2) * (uint32_t)p.ld_w + (uint32_t)(wc << 4);
+    const uint32_t vw_tail = wc * 32 < k_tail ? vw_lane : kBeyond;
+    // scale words: word wave * 64 + lane = lrow' * 8 + tile' belongs to row tile' * 16 + lrow'; tiles 5..7 and the words of
+    // waves 2 and 3 do not exist
+    const int sword = wave * 64 + lane;
+    const uint32_t vs_lane = (sword < 128 && (sword & 7) < TN) ? (uint32_t)((sword & 7) * 16 + (sword >> 3)) * (uint32_t)p.ld_ws : kBeyond;
+    const uint32_t s_last = (uint32_t)(last * 4 - (4 - vq));
+    const unsigned sshift = 8u * (unsigned)quarter, sshift_tail = 8u * (unsigned)(quarter + 4 - vq);
+    const bool q_in_tail = quarter < vq;
+    typedef __attribute__((address_space(3))) void lds_void;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, (int)a_end, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(w_wave), 0, (int)w_end, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(s_tile), 0, (int)s_end, 0x00020000);
+    auto dma = [&](int kt, int stage) {
+        const bool tail = kt == last;
+#pragma unroll
+        for (int i = 0; i < LX; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 4 * i) * 1024), 16, tail ? va_tail : va_lane,
+                                                     (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)  // groups of 16 weight rows wave and wave + 4: only group 4 of the second set exists
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void*)(smem + WBASE + stage * WS + (wave + 4 * i) * 1024), 16,
+                                                     (wave + 4 * i) < TN ? (tail ? vw_tail : vw_lane) : kBeyond,
+                                                     (uint32_t)i * w_step + ((uint32_t)kt << 6), 0, 2);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + SBASE + stage * SS + wave * 256), 4, vs_lane,
+                                                 tail ? s_last : (uint32_t)kt << 2, 0, 0);
+    };
+
+    float sam[XT];
+#pragma unroll
+    for (int j = 0; j < XT; ++j) {
+        const int m = m0 + wave * (BM / 4) + j * 16 + lrow;
+        sam[j] = p.sa[m < p.M ? m : p.M - 1];  // the oldest load: every later wait covers it
+    }
+    f32x4 acc[TN][XT];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < XT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wave * (BM / 4) + lrow) * 128 + ((quarter ^ fsw) << 4);
+    const int x_off2 = (wave * (BM / 4) + lrow) * 128 + (((4 + quarter) ^ fsw) << 4);
+    const int w_off = WBASE + lrow * 64 + ((quarter ^ ((lrow >> 2) & 3)) << 4);
+    const int s_off = SBASE + lrow * 32;
+
+#pragma unroll
+    for (int d = 0; d < S - 1; ++d) dma(d < last ? d : last, d);
+    int cur = 0;  // kt % S
+    for (int kt = 0; kt < KT; ++kt) {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * L) : "memory");
+        const int nxt = cur == 0 ? S - 1 : cur - 1;  // (kt + S - 1) % S
+        dma(kt + S - 1 < last ? kt + S - 1 : last, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        const bool tail = kt == last;
+        u32x4 s03 = *reinterpret_cast<const u32x4*>(smem + cur * SS + s_off);
+        uint32_t s4 = *reinterpret_cast<const uint32_t*>(smem + cur * SS + s_off + 16);
+        asm volatile("" : "+v"(s03));
+        i32x4 fw[TN];
+        uint32_t sb_[TN];
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            fw[i] = *reinterpret_cast<const i32x4*>(smem + cur * WS + i * 1024 + w_off);
+            const uint32_t word = i < 4 ? s03[i] : s4;
+            const uint32_t b = word >> (tail ? sshift_tail : sshift);
+            sb_[i] = (tail && !q_in_tail) ? 127u : b;
+        }
+#pragma unroll
+        for (int j = 0; j < XT; ++j) {
+            const uint8_t* base = smem + cur * XS + j * 2048;
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(base + x_off);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(base + x_off2);
+            const i32x8 xf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+            for (int i = 0; i < TN; ++i) acc[i][j] = mfma_w4a8<0>(fw[i], xf, acc[i][j], (int)sb_[i]);
+        }
+        // pinned, or the compiler may move the MFMAs (pure functions of registers) past the next barrier
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < XT; ++j) asm volatile("" : "+v"(acc[i][j]));
+        cur = cur == S - 1 ? 0 : cur + 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in LDS once the workgroup has gone
+
+#pragma unroll
+    for (int j = 0; j < XT; ++j) {
+        const int m = m0 + wave * (BM / 4) + j * 16 + lrow;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int n = n0 + i * 16 + quarter * 4;
+            if (n >= p.N) continue;  // N % 16 == 0: a group of four is inside or outside as a whole
+            f32x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e] * sam[j];
+            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
+            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+    }
+}
+
 // more dynamic LDS than the default 64 KiB: the limit is raised once per device and kernel
 static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64]) {
     if (lds <= 64 * 1024) return CFP8_OK;
@@ -1419,6 +1563,22 @@ static int launch_mx4_128x512(Mx4Args p, int out_dtype, hipStream_t st) {
     if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
     if (f32) hipLaunchKernelGGL(gemm_mxfp4_128x512_kernel<true>, dim3((unsigned)tiles), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_mxfp4_128x512_kernel<false>, dim3((unsigned)tiles), dim3(256), lds, st, p);
+    return check_launch("gemm_mxfp4");
+}
+
+template <int BM>
+static int launch_mx4_strip(Mx4Args p, int out_dtype, hipStream_t st) {
+    constexpr int S = BM == 64 ? 9 : 6;
+    constexpr size_t lds = (size_t)S * (BM * 128 + 8 * 1024 + 1024);
+    static_assert(lds <= 160 * 1024, "strip kernel LDS");
+    p.tiles_m = (p.M + BM - 1) / BM;
+    const int64_t blocks = (p.N + 79) / 80 * p.tiles_m;
+    const bool f32 = out_dtype == CFP8_OUT_F32;
+    static std::atomic<bool> raised[2][64];
+    const void* fn = f32 ? reinterpret_cast<const void*>(gemm_mxfp4_strip_kernel<BM, true>) : reinterpret_cast<const void*>(gemm_mxfp4_strip_kernel<BM, false>);
+    if (int rc = ensure_lds(fn, lds, raised[f32])) return rc;
+    if (f32) hipLaunchKernelGGL((gemm_mxfp4_strip_kernel<BM, true>), dim3((unsigned)blocks), dim3(256), lds, st, p);
+    else hipLaunchKernelGGL((gemm_mxfp4_strip_kernel<BM, false>), dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm_mxfp4");
 }
 
@@ -1624,6 +1784,8 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (M <= 16 && !m_indices) return launch_mx4_gemv(p, out_dtype, st);
     if (M <= 16) return launch_mx4<16, 64, 1, 4, 2>(p, out_dtype, st);
+    // 17..128 tokens on a wide weight: the strip kernel (a narrow weight leaves most CUs without a strip)
+    if (M <= 128 && !m_indices && K >= 128 && (N + 79) / 80 >= 128) return M <= 64 ? launch_mx4_strip<64>(p, out_dtype, st) : launch_mx4_strip<128>(p, out_dtype, st);
     if (M <= 64 && !m_indices) {
         // few weight rows: narrow workgroups, so that there are enough of them
         const bool narrow = (N + 15) / 16 <= 512;
