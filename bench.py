@@ -265,7 +265,7 @@ def summarise_top_level(extra):
          "configs[4]: 128 experts, 8192 tokens top-8: 1x128 quant, gate_up GEMM + SwiGLU + requant, down GEMM",
          {"swiglu_separate": "grouped_cfg5_mlp_swiglu_as_separate_launch"})
     dec = {}
-    for M in (1, 64):
+    for M in (1, 64, 128):
         e = extra.get(f"linear_rowwise_cfg3_M{M}")
         if e and "ms" in e:
             dec[f"M{M}_ms"], dec[f"M{M}_GBps"], dec[f"M{M}_frac_hbm"] = e["ms"], e["GB/s"], e["frac_hbm"]
@@ -274,7 +274,7 @@ def summarise_top_level(extra):
         dec["copy_same_bytes_ms"], dec["copy_GBps"], dec["copy_frac_hbm"] = c["ms"], c["GB/s"], c["frac_hbm"]
     if dec:
         dec.update({"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "workload": "configs[2] M=1 and M=64: the 68 MB fp8 weight streamed once; beside them a plain device copy moving the same 68 MB"})
+                    "workload": "configs[2] at 1, 64 and 128 tokens: the 68 MB fp8 weight streamed once; beside them a plain device copy moving the same 68 MB"})
         top["roofline_decode"] = dec
     r = extra.get("rowwise_multi_qwen25_7b_sync_112_weights")
     if r:
@@ -452,7 +452,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     cdst = torch.empty_like(csrc)
     hbm("plain_copy_same_bytes_as_cfg3_weight", N3 * K3, lambda: cdst.copy_(csrc))
     del csrc, cdst
-    for M in (1, 64, 1024, 8192):
+    for M in (1, 64, 128, 1024, 8192):
         x = torch.randn(M, K3, generator=gen, device=dev)
         chan = torch.rand(K3, generator=gen, device=dev) < 0.005
         x = torch.where(chan[None, :], x * 30, x).to(torch.bfloat16)
@@ -462,7 +462,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
         mfma(f"linear_rowwise_cfg3_M{M}", 2.0 * M * N3 * K3, N3 * K3 + 4 * N3 + M * K3 * 2 + M * N3 * 2,
              lambda: check(lib.cfp8_linear_rowwise(x.data_ptr(), K3, qw3.data_ptr(), K3, sw3.data_ptr(), o.data_ptr(), N3, 0,
                                                    M, N3, K3, ws.data_ptr(), wsb, stream)), iters=50)
-        if M >= 64:
+        if M >= 64 and M != 128:
             # the GEMM alone on the quantised operands, and the vendor library's rowwise scaled GEMM
             # (torch._scaled_mm) on the same bytes beside it - a comparison figure, nothing here calls it otherwise
             qx, sx = ops.quant_rowwise(x)
@@ -522,7 +522,7 @@ def run_extra(torch, lib, _lib, ops, dev, stream, gen, tensors, only=""):
     # the consumer of those weights: FP8 activations (per-token scales) x MXFP4 weights on the scaled matrix
     # instruction.  Config 3's shape, so that the lines sit beside linear_rowwise_cfg3_M* (FP8 weights: twice the
     # weight bytes), and the GPT-OSS-20B gate_up shape of one expert's worth of columns at 8192 tokens.
-    for (nm, M, N, K) in [("cfg3", 1, 18944, 3584), ("cfg3", 16, 18944, 3584), ("cfg3", 64, 18944, 3584),
+    for (nm, M, N, K) in [("cfg3", 1, 18944, 3584), ("cfg3", 16, 18944, 3584), ("cfg3", 64, 18944, 3584), ("cfg3", 128, 18944, 3584),
                           ("cfg3", 8192, 18944, 3584), ("gptoss_5632x2816", 8192, 5632, 2816)]:
         name = f"gemm_mxfp4_{nm}_M{M}"
         if only and only not in name and only not in f"linear_mxfp4_{nm}_M{M}":
