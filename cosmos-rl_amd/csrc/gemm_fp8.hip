@@ -2014,7 +2014,7 @@ __global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs 
     for (int kt = 0; kt < KT; ++kt) {
         // tile kt has landed when at most the loads of the S - 2 tiles behind it are outstanding; after the barrier
         // nobody reads the stage of step kt - 1 any more
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * (LX + LW)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((S - 2) * (LX + LW)) : "memory");
         const int nxt = cur == 0 ? S - 1 : cur - 1;  // (kt + S - 1) % S
         dma(kt + S - 1 < last ? kt + S - 1 : last, nxt);
         __builtin_amdgcn_sched_barrier(0);

@@ -1454,7 +1454,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_strip_kernel(const Mx4Args p) 
     for (int d = 0; d < S - 1; ++d) dma(d < last ? d : last, d);
     int cur = 0;  // kt % S
     for (int kt = 0; kt < KT; ++kt) {
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((S - 2) * L) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((S - 2) * L) : "memory");
         const int nxt = cur == 0 ? S - 1 : cur - 1;  // (kt + S - 1) % S
         dma(kt + S - 1 < last ? kt + S - 1 : last, nxt);
         __builtin_amdgcn_sched_barrier(0);

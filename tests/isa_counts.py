@@ -1,7 +1,8 @@
 """Instruction census of the GEMM kernels with hand-counted waits, from hipcc's own assembly listing of
 csrc/gemm_fp8.hip and csrc/gemm_mxfp4.hip.
 
-gemm_rowwise_256p_kernel, gemm_block_w8p_kernel and the three direct-to-LDS kernels of gemm_mxfp4.hip order their LDS traffic with hand-written
+gemm_rowwise_256p_kernel, gemm_block_w8p_kernel, the strip kernels and the direct-to-LDS kernels of gemm_mxfp4.hip order their
+LDS traffic with hand-written
 ``s_waitcnt vmcnt(N)`` + ``s_barrier`` pairs: N is the number of vector-memory operations the author
 counted between the loads a barrier needs and the barrier.  That is right only while the compiler
 emits exactly those operations, so the census (vector-memory instructions by kind, barriers, the N of
@@ -24,7 +25,7 @@ sys.path.insert(0, str(ROOT / "cosmos-rl_amd"))
 from cosmos_rl_amd import _build  # noqa: E402
 
 WALKING = ("gemm_rowwise_256p_kernel", "gemm_block_w8p_kernel", "gemm_mxfp4_256_kernel", "gemm_mxfp4_128_kernel",
-           "gemm_mxfp4_128x512_kernel")
+           "gemm_mxfp4_128x512_kernel", "gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel")
 SOURCES = ("gemm_fp8.hip", "gemm_mxfp4.hip")
 _VMEM = re.compile(r"^\s+((?:buffer|global|flat|scratch)_(?:load|store|atomic)\w*)\b(.*)")
 _PAIR = re.compile(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)")

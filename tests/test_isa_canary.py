@@ -35,6 +35,7 @@ def test_no_scratch_and_counts_add_up(census):
         assert rec["scratch_between_mfmas"] == 0, f"{name} spills inside its K loop: {ops}"
         assert not any(k.startswith("flat_") for k in ops), f"{name} uses flat addressing: {ops}"
         m = re.match(r"(\w+)<(.*)>", name)
+        args = [int(a) for a in m.group(2).split(",")]
         mx4 = {"gemm_mxfp4_256_kernel": (8, 4, 1, 64), "gemm_mxfp4_128_kernel": (4, 4, 1, 32), "gemm_mxfp4_128x512_kernel": (4, 8, 2, 64)}
         if m.group(1) in mx4:
             # per wave and K step x activation + w weight loads of 16 bytes and s scale loads of 4 bytes (and so many
@@ -49,6 +50,21 @@ def test_no_scratch_and_counts_add_up(census):
             assert ops["buffer_load_dwordx4 lds"] == (2 * x + 3 * w) + copies * (x + w), (name, ops)
             assert ops["buffer_load_dword lds"] == 3 * sc + copies * sc and ops["global_load_lds_dword"] == 1, (name, ops)
             assert rec["mfma"] == copies * mfma_per_step, (name, rec)
+            continue
+        if m.group(1) in ("gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel"):
+            # a ring of S stages: the prologue requests S - 1 tiles, every step one more; the barrier of a step lets the
+            # loads of the S - 2 tiles behind the one it needs pass
+            bm = args[0]
+            if m.group(1) == "gemm_rowwise_strip_kernel":
+                x4, w4, s1, stages = bm // 32, (args[1] * 16 + 31) // 32, 0, 8 if bm == 64 else 5
+            else:
+                x4, w4, s1, stages = bm // 32, 2, 1, 9 if bm == 64 else 6
+            per_step = x4 + w4 + s1
+            pairs = [n for n in rec["hand_written_vmcnt_before_barrier"] if n]
+            assert pairs and set(pairs) == {(stages - 2) * per_step}, (name, rec)
+            assert ops["buffer_load_dwordx4 lds"] == (stages - 1 + len(pairs)) * (x4 + w4), (name, ops)
+            assert ops.get("buffer_load_dword lds", 0) == (stages - 1 + len(pairs)) * s1, (name, ops)
+            assert not any(k.startswith("scratch_") for k in ops), f"{name} spills: {ops}"
             continue
         assert not any(k.startswith("scratch_") for k in ops), f"{name} spills: {ops}"
         stores = sum(n for k, n in ops.items() if "_store_" in k)
