@@ -133,8 +133,9 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
 // c mod waves, so that at any moment the GPU reads one compact window that moves through the tensor),
 // reduces |x|, the workgroup publishes its maximum with one atomic max, the workgroups meet at a counter in
 // device memory, and every wave casts what it holds with the tensor's scale and stores it: 2 B read and 1 B
-// written per element instead of 2 + 2 + 1.  A workgroup that is done storing goes on to load the next tensor
-// while others still store.  Every kept vector has its own registers, hence its own instructions: the code a
+// written per element instead of 2 + 2 + 1.  A slot that has been cast and stored is requested anew at once with
+// the next tensor's chunk (register slots by loads into the same registers, LDS slots by direct-to-LDS loads), so
+// one tensor's stores and the next one's loads are in flight together.  Every kept vector has its own registers, hence its own instructions: the code a
 // wave runs per tensor is 30 KB of straight line, shared by the CU's twelve waves and small enough to stay in
 // the instruction cache from one tensor to the next (with one wave per SIMD and all 512 registers it was 350 KB
 // and the kernel spent its time fetching it).
@@ -215,30 +216,42 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
     };
     // Chunks 0 .. kResLdsVecs - 1 of the wave live in LDS and pass through the first register slots; chunk
     // kResLdsVecs + r lives in register slot r.
+    // Direct-to-LDS loads of the next tensor and the reads of this one's LDS slots: the reads are written as
+    // instructions of their own, which the compiler does not take for LDS accesses - behind a direct-to-LDS load it
+    // would otherwise wait for every load in flight before each of them.
+    typedef __attribute__((address_space(3))) void lds_void;
+    uint8_t* const wave_lds = reinterpret_cast<uint8_t*>(res_lds + wave * (kResLdsVecs * 64));
+    const u32 lds_lane = (u32) reinterpret_cast<uintptr_t>((lds_void*)my_lds);
+    auto load_lds = [&](__amdgpu_buffer_rsrc_t rx, const Geo& g, int l) {  // the wave's chunk l, 16 bytes per lane, to its LDS slot l
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(wave_lds + l * 1024), 16, g.lane_vec * 16u, slot_vec(g, l) * 16u, 0, 2);
+    };
     uint4 keep[kResRegVecs];
+    Geo g = geo(0);
+    u32 m = 0;
+    // ---- the first tensor's loads: kResDepth in flight per wave, issued in chunk order, straight into the registers
+    // that keep them
+    {
+        constexpr int kResDepth = 8;
+        const __amdgpu_buffer_rsrc_t rx = rsrc(tb.x[0]);
+#pragma unroll
+        for (int l = 0; l < kResDepth; ++l) keep[l] = load(rx, g, l);
+#pragma unroll
+        for (int l = 0; l < kResLdsVecs; ++l) {
+            m = absmax8(m, keep[l]);
+            my_lds[l * 64] = keep[l];
+            if (l + kResDepth < kResLdsVecs) keep[l + kResDepth] = load(rx, g, l + kResDepth);
+        }
+#pragma unroll
+        for (int r = 0; r < kResDepth; ++r) keep[r] = load(rx, g, kResLdsVecs + r);
+#pragma unroll
+        for (int r = 0; r < kResRegVecs; ++r) {
+            m = absmax8(m, keep[r]);
+            if (r + kResDepth < kResRegVecs) keep[r + kResDepth] = load(rx, g, kResLdsVecs + r + kResDepth);
+        }
+    }
     for (int t = 0; t < tb.n; ++t) {
-        const Geo g = geo(t);
-        // ---- pass 1: kResDepth loads in flight per wave, issued in chunk order, straight into the registers that
-        // keep them
+        // here the wave holds tensor t and m is the lane's maximum of it
         {
-            constexpr int kResDepth = 8;
-            const __amdgpu_buffer_rsrc_t rx = rsrc(tb.x[t]);
-            u32 m = 0;
-#pragma unroll
-            for (int l = 0; l < kResDepth; ++l) keep[l] = load(rx, g, l);
-#pragma unroll
-            for (int l = 0; l < kResLdsVecs; ++l) {
-                m = absmax8(m, keep[l]);
-                my_lds[l * 64] = keep[l];
-                if (l + kResDepth < kResLdsVecs) keep[l + kResDepth] = load(rx, g, l + kResDepth);
-            }
-#pragma unroll
-            for (int r = 0; r < kResDepth; ++r) keep[r] = load(rx, g, kResLdsVecs + r);
-#pragma unroll
-            for (int r = 0; r < kResRegVecs; ++r) {
-                m = absmax8(m, keep[r]);
-                if (r + kResDepth < kResRegVecs) keep[r + kResDepth] = load(rx, g, kResLdsVecs + r + kResDepth);
-            }
             const u32 w = wave_max(pk_fold(m));
             if (lane == 0) red[wave] = w;
         }
@@ -266,30 +279,65 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             }
         }
         __syncthreads();
-        // ---- pass 2: cast what is held and store it
+        // ---- cast what is held and store it; every slot that has been stored is requested anew at once with the next
+        // tensor's chunk, so the stores of this tensor and the loads of the next share the memory system.  Behind the
+        // last tensor the loads go through a descriptor of no bytes: they fetch nothing.
         static_assert(kAmaxSlots == 64, "one slot per lane");
         const float amax = __uint_as_float(wave_max(lane ? __hip_atomic_load(tb.amax[t] + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u));
         const float scale = *gave_up != 0u ? __uint_as_float(kCanonNaN) : scale_from_amax(amax);
         if (gw == 0 && lane == 0) *tb.scale[t] = scale;
         const Divider d(scale);
         const __amdgpu_buffer_rsrc_t rq = rsrc(tb.q[t]);
-        // (slots past the wave's last chunk hold copies of it: skipped here, where a branch costs nothing - a wave with
-        // no chunk of its own stores the one it copied once more, the same bytes)
-        if (d.finite) {  // (one branch per tensor: the code of the other case is never fetched)
-#pragma unroll
-            for (int l = 0; l < kResLdsVecs; ++l)
-                if (l <= g.lastc) store(rq, g, l, cast8_finite(my_lds[l * 64], d));
-#pragma unroll
-            for (int r = 0; r < kResRegVecs; ++r)
-                if (kResLdsVecs + r <= g.lastc) store(rq, g, kResLdsVecs + r, cast8_finite(keep[r], d));
-        } else {
+        const bool more = t + 1 < tb.n;
+        const Geo gn = more ? geo(t + 1) : g;
+        const __amdgpu_buffer_rsrc_t rx =
+            more ? rsrc(tb.x[t + 1]) : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(tb.x[t]), 0, 0, 0x00020000);
+        auto lds_slot = [&](int l) {  // this tensor's LDS slot l, read before the slot is requested anew
+            u32x4 v;
+            asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_lane), "n"(l * 1024) : "memory");
+            return make_uint4(v[0], v[1], v[2], v[3]);
+        };
+        // (slots past the wave's last chunk hold copies of it: not stored - a wave with no chunk of its own stores the
+        // one it copied once more, the same bytes)
+        int last_store = g.lastc;
+        if (!d.finite) {
+            // a scale that is infinite or NaN: the bytes are stored here, and the code below, which every other tensor
+            // takes, only requests the next tensor (one definition of the kept registers: with a second one in this
+            // branch the compiler spills most of them)
 #pragma unroll
             for (int l = 0; l < kResLdsVecs; ++l)
                 if (l <= g.lastc) store(rq, g, l, cast8_nonfinite_scale(my_lds[l * 64], scale));
 #pragma unroll
             for (int r = 0; r < kResRegVecs; ++r)
                 if (kResLdsVecs + r <= g.lastc) store(rq, g, kResLdsVecs + r, cast8_nonfinite_scale(keep[r], scale));
+            last_store = -1;
         }
+#pragma unroll
+        for (int l = 0; l < kResLdsVecs; ++l) {
+            const uint4 v = lds_slot(l);
+            if (l <= last_store) store(rq, g, l, cast8_finite(v, d));
+            load_lds(rx, gn, l);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < kResRegVecs; ++r) {
+            if (kResLdsVecs + r <= last_store) store(rq, g, kResLdsVecs + r, cast8_finite(keep[r], d));
+            keep[r] = load(rx, gn, kResLdsVecs + r);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        g = gn;
+        if (!more) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the empty loads still write LDS: none is in flight when the wave ends)
+            break;
+        }
+        // ---- the next tensor's maximum, slot by slot as the loads land (they return in order); the LDS slots were
+        // requested first, so they are complete once the last register slot is
+        m = 0;
+#pragma unroll
+        for (int r = 0; r < kResRegVecs; ++r) m = absmax8(m, keep[r]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int l = 0; l < kResLdsVecs; ++l) m = absmax8(m, my_lds[l * 64]);
     }
 }
 
