@@ -81,3 +81,38 @@ def test_no_scratch_and_counts_add_up(census):
             assert ops["buffer_load_dwordx4 lds"] == 2 * a_it + 3 * b_it + 2 * (a_it + b_it), (name, ops)
         else:
             assert pairs, name
+
+
+def test_resident_tensorwise_kernel_merged_phase():
+    """The resident tensorwise kernel stores a slot and requests it anew with the next tensor's chunk.  That only
+    overlaps stores and loads while (a) no kept vector is spilled, (b) nothing waits for a vector-memory operation
+    between the first direct-to-LDS load and the last load of the phase, and (c) every LDS slot is read (by an
+    instruction the source writes out) before the direct-to-LDS load that overwrites it is issued."""
+    import subprocess
+    import tempfile
+
+    from cosmos_rl_amd import _build
+
+    with tempfile.TemporaryDirectory() as tmp:
+        out = Path(tmp) / "quant_tensorwise.s"
+        cmd = [_build.hipcc(), *_build.HIPCC_FLAGS, f"-I{_build.INCLUDE_DIR}", f"-I{_build.CSRC_DIR}", "--cuda-device-only", "-S",
+               str(_build.CSRC_DIR / "quant_tensorwise.hip"), "-o", str(out)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr
+        lines = out.read_text().splitlines()
+    start = next(i for i, line in enumerate(lines) if re.match(r"^_ZN4cfp8\d+tensorwise_resident_kernel\w*:", line))
+    end = next(i for i in range(start, len(lines)) if lines[i].startswith(".Lfunc_end"))
+    body = lines[start:end]
+    assert not any(re.match(r"^\s+scratch_", line) for line in body), "the resident kernel spills"
+    dma = [i for i, line in enumerate(body) if re.match(r"^\s+buffer_load_dwordx4 .*\blds\b", line)]
+    assert len(dma) == 13, f"{len(dma)} direct-to-LDS loads, one per LDS slot expected"
+    # the register slots' loads follow the last direct-to-LDS load: the next 32 plain 16-byte buffer loads
+    plain = [i for i, line in enumerate(body) if i > dma[-1] and re.match(r"^\s+buffer_load_dwordx4 (?!.*\blds\b)", line)][:32]
+    assert len(plain) == 32
+    phase = body[dma[0]:plain[-1] + 1]
+    assert not any("s_waitcnt vmcnt" in line for line in phase), "a wait for vector memory inside the merged phase"
+    # one written-out LDS read in front of every direct-to-LDS load (slot l is read, then requested anew)
+    reads = [i for i, line in enumerate(body) if re.match(r"^\s+ds_read_b128 ", line) and i < dma[-1]]
+    for k, d in enumerate(dma):
+        lo = dma[k - 1] if k else 0
+        assert any(lo < r < d for r in reads), f"no LDS read between direct-to-LDS loads {k - 1} and {k}"
