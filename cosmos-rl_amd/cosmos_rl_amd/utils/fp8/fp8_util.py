@@ -54,23 +54,14 @@ class FP8Config:
 
 def module_filter_fn(mod: nn.Module, fqn: str, filter_fqns: List[str]) -> bool:
     """fp8_util.py:62-87: convert only ``nn.Linear`` whose two dimensions are multiples of 16
-    and whose fully qualified name contains none of ``filter_fqns``.
-
-    One condition is stricter here than in the reference: the FP8 MFMA GEMM consumes K in steps of
-    128, so ``in_features`` must be a multiple of 128 (the reference's torchao path takes any multiple
-    of 16).  A layer that fails it stays an ``nn.Linear`` and computes in its own dtype instead of
-    being converted and then failing in its first forward."""
+    and whose fully qualified name contains none of ``filter_fqns``.  (The FP8 GEMM takes any such
+    ``in_features``: a K that is not a multiple of its 128-wide step runs with the last step masked.)"""
     if not isinstance(mod, nn.Linear):
         return False
     out_features, in_features = mod.weight.shape
     if out_features % 16 or in_features % 16:
         return False
-    if in_features % FP8_GEMM_K_STEP:
-        return False
     return not any(f in fqn for f in filter_fqns)
-
-
-FP8_GEMM_K_STEP = 128  # K of one FP8 MFMA step: in_features of a converted layer is a multiple of it
 
 
 def is_gfx950_available() -> bool:

@@ -88,8 +88,12 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     tn = in / gsz;
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32, bool SCALE_VEC>
+// KTAIL (rowwise only): K is a multiple of 16 but not of 128.  The last K step then ends inside its 128 bytes: lanes
+// whose 16-byte chunk lies past K fetch chunk 0 of their row instead (nothing is read outside a row) and store zeros
+// to LDS, for both operands, so the step's products are those of the K that exists.
+template <int BM, int BN, int WM, int WN, int MODE, bool OUT_F32, bool SCALE_VEC, bool KTAIL = false>
 __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const GemmArgs p) {
+    static_assert(!KTAIL || MODE == kRowwise, "a K tail has no block scale of its own");
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
     constexpr int TM = WTM / 16, TN = WTN / 16;  // MFMA tiles per wave
@@ -118,7 +122,7 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave % WM, wn = wave / WM;
     const int lrow = lane & 15, quarter = lane >> 4;
-    const int KT = p.K >> 7;
+    const int KT = KTAIL ? (p.K + 127) >> 7 : p.K >> 7;
 
     // global -> register staging of one K step.  One wave-wide load covers 8 rows x
     // 128 bytes (8 full cache lines): lane = pair * 16 + row8 * 2 + half reads chunk
@@ -134,6 +138,8 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     // than 2^32 bytes for any leading dimension below 2^24).
     i32x4 ra[A_IT], rb[B_IT];
     uint32_t oa[A_IT], ob[B_IT];
+    const bool chunk_in_k = !KTAIL || st_c * 16 < (p.K & 127);  // this lane's chunk of the last K step lies inside K
+    const uint32_t tail_back = chunk_in_k ? 0u : (uint32_t)st_c * 16u;  // what takes the lane back to chunk 0 there
     const uint8_t* const abase = p.a + (int64_t)m0 * p.ld_a;
     const uint8_t* const bbase = bptr + (int64_t)n0 * p.ld_b;
 #pragma unroll
@@ -152,24 +158,26 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
         const int64_t k = (int64_t)(kt < KT ? kt : KT - 1) << 7;
         const uint8_t* const ak = abase + k;
         const uint8_t* const bk = bbase + k;
+        const uint32_t back = KTAIL && kt >= KT - 1 ? tail_back : 0u;
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const i32x4*>(ak + oa[i]);
+        for (int i = 0; i < A_IT; ++i) ra[i] = *reinterpret_cast<const i32x4*>(ak + (oa[i] - back));
 #pragma unroll
-        for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const i32x4*>(bk + ob[i]);
+        for (int i = 0; i < B_IT; ++i) rb[i] = *reinterpret_cast<const i32x4*>(bk + (ob[i] - back));
     };
-    // LDS stores number `first` .. `last`-1 of the A_IT + B_IT that make up one staged tile
-    auto store_part = [&](int stage, int first, int last) {
+    // LDS stores number `first` .. `last`-1 of the A_IT + B_IT that make up one staged tile, which is K step `kt`
+    auto store_part = [&](int stage, int first, int last, int kt) {
+        const int keep = KTAIL && kt >= KT - 1 && !chunk_in_k ? 0 : -1;
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) {
             const int r = (wave + NW * i) * 8 + st_row8;
             if (i >= first && i < last && (A_BLK % NW == 0 || r < BM))
-                *reinterpret_cast<i32x4*>(As(stage) + lds_chunk_offset(r, st_c)) = ra[i];
+                *reinterpret_cast<i32x4*>(As(stage) + lds_chunk_offset(r, st_c)) = KTAIL ? ra[i] & keep : ra[i];
         }
 #pragma unroll
         for (int i = 0; i < B_IT; ++i) {
             const int r = (wave + NW * i) * 8 + st_row8;
             if (A_IT + i >= first && A_IT + i < last && (B_BLK % NW == 0 || r < BN))
-                *reinterpret_cast<i32x4*>(Bs(stage) + lds_chunk_offset(r, st_c)) = rb[i];
+                *reinterpret_cast<i32x4*>(Bs(stage) + lds_chunk_offset(r, st_c)) = KTAIL ? rb[i] & keep : rb[i];
         }
     };
     constexpr int ST_ALL = A_IT + B_IT;
@@ -230,7 +238,7 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
     sg_load(0);
     float s_n = load_sn(0);
     __builtin_amdgcn_sched_barrier(0);  // weight scale before tile kt+1, as in the loop: one wait count fits both
-    store_part(0, 0, ST_ALL);
+    store_part(0, 0, ST_ALL, 0);
     sg_store(0);
     load_tile(1);
     __syncthreads();
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
             if (j < TM) {
                 i32x8 fb_next = fb;
                 if (j + 1 < TM) fb_next = lds_frag(As(cur), wm * WTM + (j + 1) * 16 + lrow, quarter);
-                if (j < HALF) store_part(cur ^ 1, ST_ALL * j / HALF, ST_ALL * (j + 1) / HALF);
+                if (j < HALF) store_part(cur ^ 1, ST_ALL * j / HALF, ST_ALL * (j + 1) / HALF, kt + 1);
                 if (MODE != kRowwise && j == HALF - 1 && (kt & 7) == 7) sg_store((kt >> 3) + 1);
 #pragma unroll
                 for (int i = 0; i < TN; ++i) {
@@ -1891,7 +1899,7 @@ __global__ __launch_bounds__(256) void linear_gemv_fused_kernel(const uint4* __r
 
 // whether the one-launch kernel above takes the call
 static bool fused_gemv_applies(int64_t M, int64_t K, const void* x, int64_t ld_x) {
-    return M >= 1 && M <= 4 && K <= 4096 && aligned16(x) && ld_x % 8 == 0;
+    return M >= 1 && M <= 4 && K <= 4096 && K % 128 == 0 && aligned16(x) && ld_x % 8 == 0;
 }
 template <int MR>
 static int launch_linear_gemv_fused_mr(const void* x, int64_t ld_x, GemmArgs& p, int out_dtype, hipStream_t st) {
@@ -2178,6 +2186,28 @@ static int launch_rowwise_skinny(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (per == 6) return launch_rowwise_skinny_cfg<TM, 6>(p, out_dtype, st);
     if (per == 7 || per == 8) return launch_rowwise_skinny_cfg<TM, 8>(p, out_dtype, st);
     return launch_rowwise_skinny_cfg<TM, 5>(p, out_dtype, st);  // 5, and everything that takes several rounds anyway
+}
+
+// rowwise, K a multiple of 16 that is not one of 128: the generic kernel's form with a masked last K step
+template <int BM, int BN, int WM, int WN>
+static int launch_cfg_ktail(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    constexpr int NT = WM * WN * 64;
+    constexpr size_t lds = (size_t)2 * (BM + BN) * 128;
+    static_assert(lds <= 64 * 1024, "the K-tail form stays within the default LDS limit");
+    {
+        char name[64];
+        snprintf(name, sizeof(name), "gemm_kernel<%d,%d,%d,%d,rowwise,ktail>", BM, BN, WM, WN);
+        if (!note_launch(name, (unsigned)blocks, NT, lds)) return CFP8_OK;
+    }
+    if (out_dtype == CFP8_OUT_F32)
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, kRowwise, true, false, true>), dim3((unsigned)blocks), dim3(NT), lds, st, p);
+    else
+        hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, kRowwise, false, false, true>), dim3((unsigned)blocks), dim3(NT), lds, st, p);
+    return check_launch("gemm");
 }
 
 template <int BM, int BN, int WM, int WN, int MODE>
@@ -2720,6 +2750,12 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
             return launch_cfg<128, 256, 2, 4, kGrouped>(p, out_dtype, st);
         return launch_cfg<128, 128, 2, 2, kGrouped>(p, out_dtype, st);
     }
+    if (MODE == kRowwise && (p.K & 127)) {
+        // K = 16 k with a last step shorter than 128: only the generic kernel masks it
+        if (p.M <= 16) return launch_cfg_ktail<16, 64, 1, 4>(p, out_dtype, st);
+        if (p.M <= 64) return launch_cfg_ktail<64, 64, 1, 4>(p, out_dtype, st);
+        return launch_cfg_ktail<128, 128, 2, 2>(p, out_dtype, st);
+    }
     if (MODE == kRowwise && p.M <= 16) return launch_rowwise_gemv(p, out_dtype, st);
     if (MODE == kRowwise && p.M <= 128) {
         // a narrow weight with a long K is cut into K slices (the skinny kernels, at most 64 tokens); everything else
@@ -2799,12 +2835,13 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
 
 static int check_common(const char* who, const void* a, const void* b, const float* sa, const float* sb,
                         const void* out, int64_t ld_a, int64_t ld_b, int64_t ld_out, int out_dtype, int64_t M,
-                        int64_t N, int64_t K) {
+                        int64_t N, int64_t K, int k_unit = 128) {
     if (M < 0 || N < 0 || K < 0) return set_error(CFP8_EINVAL, "%s: negative shape", who);
     if (M == 0 || N == 0) return CFP8_OK;  // nothing to compute: pointers may be null
     if (!a || !b || !sa || !sb || !out) return set_error(CFP8_EINVAL, "%s: null pointer", who);
-    if (K == 0 || K % 128 || N % 16)
-        return set_error(CFP8_EINVAL, "%s: K=%lld must be a positive multiple of 128 and N=%lld a multiple of 16", who, (long long)K, (long long)N);
+    // (block scales cover 128 columns of K; the rowwise forms take any multiple of 16, the last K step then masked)
+    if (K == 0 || K % k_unit || N % 16)
+        return set_error(CFP8_EINVAL, "%s: K=%lld must be a positive multiple of %d and N=%lld a multiple of 16", who, (long long)K, k_unit, (long long)N);
     // the kernels index rows with 32-bit integers and tile-local byte offsets with 32 bits
     if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || ld_a >= (1ll << 24) || ld_b >= (1ll << 24))
         return set_error(CFP8_EINVAL, "%s: shape beyond the supported range (M, N, K < 2^31, leading dimensions < 2^24)", who);
@@ -2827,7 +2864,8 @@ extern "C" int cfp8_gemm_dispatch_info(int kind, int64_t M, int64_t N, int64_t K
     using namespace cfp8;
     if (!buf || buf_bytes == 0) return set_error(CFP8_EINVAL, "gemm_dispatch_info: no buffer");
     buf[0] = 0;
-    if (M <= 0 || N <= 0 || K <= 0 || K % 128 || N % 16 || M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || cus <= 0)
+    const bool rowwise_kind = kind == CFP8_DISPATCH_ROWWISE || kind == CFP8_DISPATCH_LINEAR;
+    if (M <= 0 || N <= 0 || K <= 0 || K % (rowwise_kind ? 16 : 128) || N % 16 || M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || cus <= 0)
         return set_error(CFP8_EINVAL, "gemm_dispatch_info: bad shape or compute-unit count");
     if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "gemm_dispatch_info: unknown out_dtype %d", out_dtype);
     // operands that pass every alignment test; nothing dereferences them
@@ -2892,7 +2930,7 @@ extern "C" int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* 
                                       const float* sb, void* out, int64_t ld_out, int out_dtype, int64_t M,
                                       int64_t N, int64_t K, void* stream) {
     using namespace cfp8;
-    if (int rc = check_common("scaled_mm_rowwise", a, b, sa, sb, out, ld_a, ld_b, ld_out, out_dtype, M, N, K)) return rc;
+    if (int rc = check_common("scaled_mm_rowwise", a, b, sa, sb, out, ld_a, ld_b, ld_out, out_dtype, M, N, K, 16)) return rc;
     if (M == 0 || N == 0) return CFP8_OK;
     if (K == 0) return set_error(CFP8_EINVAL, "scaled_mm_rowwise: K must be positive");
     if (int rc = check_device()) return rc;
@@ -2931,7 +2969,7 @@ extern "C" int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, i
     if (!x || !aligned16(x) || ld_x % 8 || ld_x < K) return set_error(CFP8_EINVAL, "linear_rowwise: bad activation pointer or leading dimension");
     uint8_t* qx = static_cast<uint8_t*>(workspace);
     float* sx = reinterpret_cast<float*>(qx + (((size_t)M * (size_t)K + 255) & ~(size_t)255));
-    if (int rc = check_common("linear_rowwise", qx, w, sx, w_scale, out, K, ld_w, ld_out, out_dtype, M, N, K)) return rc;
+    if (int rc = check_common("linear_rowwise", qx, w, sx, w_scale, out, K, ld_w, ld_out, out_dtype, M, N, K, 16)) return rc;
     if (int rc = check_device()) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (fused_gemv_applies(M, K, x, ld_x)) {

@@ -321,7 +321,9 @@ int cfp8_dequant_block128(const void* q, const float* scales, int64_t rows, int6
  * the reference passes -, sa [M], sb [N], out [M, N] (ld_out).
  * Replaces torch._scaled_mm(qx, w.t(), scale_a, scale_b, out_dtype=bf16) reached
  * through cosmos_rl/rollout/vllm_rollout/monkey_patch_for_fp8.py:26-34.
- * K % 128 == 0, N % 16 == 0. */
+ * K % 16 == 0, N % 16 == 0 (the dimensions module_filter_fn of cosmos_rl/utils/fp8/fp8_util.py:62-87 lets
+ * through).  The tuned kernels take K % 128 == 0; any other K runs the generic tile kernel with its last K step
+ * masked. */
 int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* sa,
                            const void* b, int64_t ld_b, const float* sb,
                            void* out, int64_t ld_out, int out_dtype,
@@ -334,7 +336,7 @@ int cfp8_scaled_mm_rowwise(const void* a, int64_t ld_a, const float* sa,
  * cfp8_linear_workspace_bytes_split(M, N, K) >= that is the size with which the call may also
  * cut K into slices for weights with few rows and a long K at 17..64 tokens (a decode-time
  * down projection: 3584 x 18944 runs 2-3x faster); the extra bytes hold fp32 partial sums.
- * Any size in between is valid and simply selects the unsplit kernel. */
+ * Any size in between is valid and simply selects the unsplit kernel.  K % 16 == 0, N % 16 == 0. */
 size_t cfp8_linear_workspace_bytes(int64_t M, int64_t K);
 size_t cfp8_linear_workspace_bytes_split(int64_t M, int64_t N, int64_t K);
 int cfp8_linear_rowwise(const void* x, int64_t ld_x, const void* w, int64_t ld_w,

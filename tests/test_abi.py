@@ -71,7 +71,7 @@ def test_argument_errors_need_no_device():
     buf = ctypes.create_string_buffer(4096)
     ptr = (ctypes.addressof(buf) + 255) & ~255
     assert lib.cfp8_scaled_mm_rowwise(ptr, 128, ptr, ptr, 128, ptr, ptr, 64, 0, 16, 64, 0, None) == _lib.EINVAL   # K = 0
-    assert "positive multiple of 128" in _lib.last_error()
+    assert "positive multiple of 16" in _lib.last_error()
     assert lib.cfp8_scaled_mm_rowwise(ptr, 1 << 24, ptr, ptr, 128, ptr, ptr, 64, 0, 16, 64, 128, None) == _lib.EINVAL
     assert "supported range" in _lib.last_error()
     # weighted combine: topk range, mode / dtype pairing, row width

@@ -74,13 +74,17 @@ def test_dispatch_limits_of_the_walking_forms():
     assert "256p" not in info(ROW, 2048, 4608, 3584)                                                  # no more tiles than CUs
     assert "256p" in info(ROW, 2048, 4608, 3584, L.OUT_BF16, 64)                                      # ... unless the GPU is smaller
     assert "swiglu" in info(SWI, 256, 512, 256)
+    # a K that is a multiple of 16 only: the generic kernel with its masked last step, whatever the shape
+    for M, N, K in ((1, 18944, 3600), (64, 512, 80), (8192, 18944, 2880)):
+        assert "ktail" in info(ROW, M, N, K) and "ktail" in info(LIN, M, N, K)
 
 
 def test_dispatch_info_rejects_bad_arguments():
     lib = L.load()
     import ctypes
     buf = ctypes.create_string_buffer(64)
-    assert lib.cfp8_gemm_dispatch_info(ROW, 128, 128, 100, 0, 256, 0, buf, 64) == L.EINVAL      # K % 128
+    assert lib.cfp8_gemm_dispatch_info(ROW, 128, 128, 100, 0, 256, 0, buf, 64) == L.EINVAL      # K % 16
+    assert lib.cfp8_gemm_dispatch_info(BLK, 128, 128, 144, 0, 256, 0, buf, 64) == L.EINVAL      # block scales: K % 128
     assert lib.cfp8_gemm_dispatch_info(9, 128, 128, 128, 0, 256, 0, buf, 64) == L.EINVAL        # kind
     assert lib.cfp8_gemm_dispatch_info(GRP, 100, 256, 128, 0, 256, 0, buf, 64) == L.EINVAL      # grouped M % 128
     assert lib.cfp8_gemm_dispatch_info(ROW, 128, 128, 128, 0, 256, 0, None, 0) == L.EINVAL

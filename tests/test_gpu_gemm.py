@@ -74,6 +74,36 @@ def test_scaled_mm_rowwise(dev, M, N, K):
     check_bf16(out16, ref, f"rowwise {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 16, 16), (5, 48, 80), (16, 64, 144), (17, 200 * 16, 1200), (64, 96, 2880), (100, 528, 1200),
+                                   (300, 272, 80), (513, 1024, 2192), (2, 18944, 3600)])
+def test_rowwise_k_not_a_multiple_of_128(dev, M, N, K):
+    """K = 16 k (what module_filter_fn lets through, cosmos_rl/utils/fp8/fp8_util.py:62-87) with a last K step shorter
+    than 128: scaled mm and the fused linear against the oracle; operands in pitched buffers whose bytes beyond K are
+    NaN patterns, which a kernel that read past K would turn into NaN outputs."""
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
+    ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
+    kp = (K + 127) // 128 * 128 + 128
+    abuf = torch.full((M, kp), 0x7F, dtype=torch.uint8, device=dev)
+    bbuf = torch.full((N, kp), 0x7F, dtype=torch.uint8, device=dev)
+    abuf[:, :K] = qx.to(dev)
+    bbuf[:, :K] = qw.to(dev)
+    a, b = abuf.view(torch.float8_e4m3fn)[:, :K], bbuf.view(torch.float8_e4m3fn)[:, :K]
+    out32 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    assert bool(torch.isfinite(out32).all())
+    assert O.rel_frobenius(out32.cpu(), ref) <= TIGHT
+    same = ops.scaled_mm(f8(qx, dev), f8(qw, dev).t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+    assert torch.equal(out32, same)
+    out16 = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.bfloat16)
+    check_bf16(out16, ref, f"rowwise {M}x{N}x{K}")
+    lin = ops.fp8_linear(x.to(dev), b.t(), sw.to(dev), out_dtype=torch.float32)
+    assert O.rel_frobenius(lin.cpu(), O.fp8_linear_rowwise(x, qw, sw, accum=torch.float64)) <= TIGHT
+    # a NaN weight byte in column 0 of row 1 reaches output column 1 only
+    if N > 2:
+        bbuf[1, 0] = 0x7F
+        out = ops.scaled_mm(a, b.t(), sx.to(dev), sw.to(dev).t(), out_dtype=torch.float32)
+        assert bool(torch.isnan(out[:, 1]).all()) and torch.equal(out[:, 2:], out32[:, 2:]) and torch.equal(out[:, 0], out32[:, 0])
+
+
 @pytest.mark.parametrize("M,N,K", [(768, 512, 384), (1024, 768, 1024)])
 def test_scaled_mm_rowwise_pitched_operands(dev, M, N, K):
     """The 256x256 kernel fetches its tiles with per-lane addresses built from the leading dimensions: operands that are

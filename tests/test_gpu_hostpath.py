@@ -171,6 +171,7 @@ def test_float8_linear_recipes(dev):
         def __init__(self):
             super().__init__()
             self.up = nn.Linear(512, 1024, bias=True)
+            self.odd = nn.Linear(1200, 48, bias=True)    # multiples of 16 only: the GEMM's masked last K step
             self.lm_head = nn.Linear(512, 256, bias=False)
 
         def fqn_filter_for_quantization(self):
@@ -195,6 +196,14 @@ def test_float8_linear_recipes(dev):
             ref = O.scaled_mm_rowwise(qx, sx.expand(40, 1), qw, sw.expand(1024, 1), accum=torch.float64)
         ref = (ref.to(torch.bfloat16) + b).float()
         assert y.dtype == torch.bfloat16 and O.rel_frobenius(y.float().cpu(), ref) <= 2e-3
+        if recipe == "rowwise":
+            assert isinstance(net.odd, fp8_util.Float8Linear)
+            x2 = O.make_activation(33, 1200, seed=6)
+            with torch.no_grad():
+                y2 = net.odd(x2.to(dev))
+            qw2, sw2 = O.quant_rowwise(net.odd.weight.detach().cpu())
+            ref2 = (O.fp8_linear_rowwise(x2, qw2, sw2, accum=torch.float64).to(torch.bfloat16) + net.odd.bias.detach().cpu()).float()
+            assert O.rel_frobenius(y2.float().cpu(), ref2) <= 2e-3
 
 
 def test_ds_group_gemm_strategy(dev):

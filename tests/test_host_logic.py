@@ -248,9 +248,8 @@ def test_recipes_filter_and_converter(monkeypatch):
     assert f(nn.Linear(128, 64), "model.layers.0.mlp.up_proj", ["lm_head"])
     assert not f(nn.Linear(128, 64), "lm_head", ["lm_head"])
     assert not f(nn.Linear(120, 64), "x", []) and not f(nn.Linear(128, 40), "x", [])
-    # multiples of 16 that the FP8 GEMM cannot take (K must be a multiple of 128) stay nn.Linear instead of
-    # converting and then failing in their first forward
-    assert not f(nn.Linear(80, 64), "x", []) and not f(nn.Linear(1200, 64), "x", []) and f(nn.Linear(1280, 48), "x", [])
+    # every multiple of 16 converts, as in the reference: the GEMM masks a last K step shorter than 128
+    assert f(nn.Linear(80, 64), "x", []) and f(nn.Linear(1200, 64), "x", []) and f(nn.Linear(1280, 48), "x", [])
     assert not f(nn.LayerNorm(32), "x", [])
 
     def cfg(**kw):
@@ -284,7 +283,7 @@ def test_recipes_filter_and_converter(monkeypatch):
     assert isinstance(net.body[0], fp8_util.Float8Linear) and net.body[0].quant_recipe == "tensorwise"
     assert net.body[0].weight is w_before
     assert type(net.body[2]) is nn.Linear            # 24 is not a multiple of 16
-    assert type(net.body[3]) is nn.Linear            # in_features 80: a multiple of 16 but not of the GEMM's K step
+    assert isinstance(net.body[3], fp8_util.Float8Linear)  # in_features 80: a multiple of 16, not of the GEMM's K step
     assert type(net.lm_head) is nn.Linear            # filtered by FQN
     assert conv.post_optimizer_hook(net) is None
     with pytest.raises(NotImplementedError):         # forward direction only
