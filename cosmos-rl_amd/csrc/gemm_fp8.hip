@@ -1467,6 +1467,247 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void g
 }
 
 // ---------------------------------------------------------------------------
+// Block-scaled GEMM on 256 x 256 tiles: eight wavefronts (two per SIMD), each a 128 x 64 block = 8 x tiles times 4 w
+// tiles, so a K step moves two thirds of the operand bytes per flop through the load path and three quarters through
+// the fragment reads of the 64 x 64 blocks of gemm_block_w8_kernel.  128 accumulator registers per wave leave no room
+// to hold a step's products apart for the rescale, so the accumulator of a row is kept in the units of the running
+// step's scale: before step k it is multiplied by s(k-1) / s(k) (s = activation scale of the row x weight scale of the
+// block), the MFMAs of the step then accumulate straight into it, and the epilogue multiplies by the last s.  In exact
+// arithmetic that is sum_k dot_k * s(k); in fp32 it adds one rounding per element and step to the rescale and the
+// rounding of the quotient, which is why results differ from the other kernel forms in the last bits.
+// Two activation and two weight stages (128 KiB), loads go straight to LDS; a step is six groups of 4 MFMAs (x tiles
+// 0..5, each fragment read two groups ahead), the barrier, and a w-major tail on x tiles 6 and 7 whose MFMAs use
+// fragments already in registers while the next step's w tiles, x tiles 0 and 1 and scales are read and the tiles after
+// next requested.  Requires M % 256 == 0, N % 256 == 0, K / 128 <= 1024.
+// ---------------------------------------------------------------------------
+template <bool OUT_F32, bool SCALE_VEC>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_256_kernel(const GemmArgs p) {
+    constexpr int BM = 256, BN = 256, NB = 2;
+    constexpr int XS = BM * 128, WS = BN * 128;
+    constexpr int WBASE = 2 * XS;
+    constexpr int SBASE = WBASE + 2 * WS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    int tm, tn;
+    tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave & 1, wn = wave >> 1;  // rows wm * 128 .. + 127, columns wn * 64 .. + 63 of the tile
+    const int lrow = lane & 15, quarter = lane >> 4;
+    const int KT = p.K >> 7;
+    const int last = KT - 1;
+
+    // global -> LDS directly: load i of an operand's K step covers rows (wave + 8 i) * 8 .. + 7 of its tile
+    uint64_t a_wave = reinterpret_cast<uint64_t>(p.a) + ((uint64_t)m0 + (uint64_t)wave * 8) * (uint64_t)p.ld_a;
+    uint64_t b_wave = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
+    uint32_t a_step = 64u * (uint32_t)p.ld_a, b_step = 64u * (uint32_t)p.ld_b;
+    asm volatile("" : "+s"(a_wave), "+s"(b_wave), "+s"(a_step), "+s"(b_step));
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t va_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_a + chunk;
+    const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
+    typedef __attribute__((address_space(3))) void lds_void;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(a_wave), 0, 0xFFFFFFFF, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(b_wave), 0, 0xFFFFFFFF, 0x00020000);
+    auto dma_x = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_void*)(smem + stage * XS + (wave + 8 * i) * 1024), 16, va_lane,
+                                                 (uint32_t)i * a_step + ((uint32_t)kt << 7), 0, 0);
+    };
+    auto dma_w = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (lds_void*)(smem + WBASE + stage * WS + (wave + 8 * i) * 1024), 16, vb_lane,
+                                                 (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 0);
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_x(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_x(1 < last ? 1 : last, 1, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(1 < last ? 1 : last, 1, i);
+
+    // activation scales: 8 K steps of this tile's rows per fetch, 4 consecutive floats per thread
+    float* const sg_buf = reinterpret_cast<float*>(smem + SBASE);  // [2][8][BM]
+    float* const sn_lds = sg_buf + 2 * 8 * BM;                         // [KT][NB]
+    const int sg_row = t >> 1, sg_half = t & 1;
+    const float* const sg_ptr = p.sa + (int64_t)(m0 + sg_row) * KT;
+    f32x4 sg = {0.f, 0.f, 0.f, 0.f};
+    auto sg_load = [&](int g) {
+        const int k0 = 8 * g + 4 * sg_half;
+        if (SCALE_VEC) {
+            sg = *reinterpret_cast<const f32x4*>(sg_ptr + (k0 + 4 <= KT ? k0 : KT - 4));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sg[e] = sg_ptr[(k0 + e) < KT ? (k0 + e) : (KT - 1)];
+        }
+    };
+    auto sg_store = [&](int g) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sg_buf[((g & 1) * 8 + 4 * sg_half + e) * BM + sg_row] = sg[e];
+    };
+
+    f32x4 acc[4][8];  // [w tile][x tile], in units of the running step's scale of the row
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int fsw = (lrow >> 1) & 7;
+    const int x_off = (wm * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int x_off2 = (wm * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    const int w_off = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
+    const int w_off2 = WBASE + (wn * 64 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
+    auto frag = [&](int stage_bytes, int off, int off2, int tile16) {
+        const uint8_t* base = smem + stage_bytes + tile16 * 2048;
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(base + off);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(base + off2);
+        i32x8 r;
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+        r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+        return r;
+    };
+    i32x8 W[4], X[4];       // x tile j of a step lives in X[j & 3]
+    float s_run[8];         // scale the accumulators of x tile j are expressed in
+    float s_nxt[8];         // scales of the step whose fragments are being read
+    auto read_scales = [&](int kt) {
+        const int k = kt < last ? kt : last;
+        const float* const sgk = sg_buf + (((k >> 3) & 1) * 8 + (k & 7)) * BM + wm * 128 + lrow;
+        const float s_n = sn_lds[k * NB + (wn >> 1)];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s_nxt[j] = sgk[j * 16] * s_n;
+    };
+
+    sg_load(0);
+    for (int idx = t; idx < KT * NB; idx += 512) {
+        const int k = idx / NB, nb = idx - k * NB;
+        sn_lds[idx] = p.sb[(int64_t)((n0 >> 7) + nb) * p.sb_stride_n + (int64_t)k * p.sb_stride_k];
+    }
+    sg_store(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    X[0] = frag(0, x_off, x_off2, 0);
+    CFP8_PHASE_END();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        W[i] = frag(0, w_off, w_off2, i);
+        CFP8_PHASE_END();
+    }
+    X[1] = frag(0, x_off, x_off2, 1);
+    read_scales(0);
+    CFP8_PHASE_END();
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s_run[j] = s_nxt[j];
+
+// the accumulators of x tile j go from the previous step's units to this step's
+#define CFP8_RESCALE256(j, rho)                                                                 \
+    {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                         \
+            _Pragma("unroll") for (int e = 0; e < 4; ++e) acc[i][j][e] = acc[i][j][e] * (rho); \
+            asm volatile("" : "+v"(acc[i][j]));                                                 \
+        }                                                                                       \
+    }
+#define CFP8_MMA256(i, j) \
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(W[i], X[(j)&3], acc[i][j], 0, 0, 0, 0, 0, 0)
+
+    for (int kt = 0; kt < KT; ++kt) {
+        const int xs_cur = (kt & 1) * XS, xs_nxt = xs_cur ^ XS;
+        const int ws_nxt = ((kt & 1) ^ 1) * WS;
+        const int kn = kt + 2 < last ? kt + 2 : last;  // past the end: the last tile again, never consumed
+        // s_nxt holds this step's scales: the factors that take every x tile's accumulators to them
+        float rho[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            rho[j] = s_run[j] * __builtin_amdgcn_rcpf(s_nxt[j]);
+            s_run[j] = s_nxt[j];
+        }
+        CFP8_RESCALE256(0, rho[0]);
+        // x tiles 0 .. 5: fragment of tile g + 2 read, MFMAs of tile g, rescale of tile g + 1
+#pragma unroll
+        for (int g = 0; g < 6; ++g) {
+            X[(g + 2) & 3] = frag(xs_cur, x_off, x_off2, g + 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) CFP8_MMA256(i, g);
+            CFP8_RESCALE256(g + 1, rho[g + 1]);
+            CFP8_PHASE_END();
+        }
+        CFP8_RESCALE256(7, rho[7]);
+        CFP8_WAIT_BARRIER(0);  // the tiles of step kt + 1 have landed, everyone is done reading this step's stages
+        CFP8_PHASE_END();
+        // tail (the next group's activation scales are stored before this step's loads are requested: an LDS store the
+        // compiler knows of waits for every direct-to-LDS load in flight)
+        if ((kt & 7) == 6) sg_store((kt >> 3) + 1);
+        X[0] = frag(xs_nxt, x_off, x_off2, 0);  // after the last step: stale data, unused
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma_x(kn, kt & 1, i);
+        if ((kt & 7) == 5) sg_load((kt >> 3) + 1);
+        CFP8_PHASE_END();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            CFP8_MMA256(i, 6);
+            CFP8_MMA256(i, 7);
+            CFP8_PHASE_END();
+            W[i] = frag(WBASE - WBASE + ws_nxt, w_off, w_off2, i);
+            dma_w(kn, kt & 1, i);
+            CFP8_PHASE_END();
+        }
+        X[1] = frag(xs_nxt, x_off, x_off2, 1);
+        read_scales(kt + 1);
+        CFP8_PHASE_END();
+    }
+#undef CFP8_RESCALE256
+#undef CFP8_MMA256
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in the stages: the epilogue reuses them
+    // back to plain units: the last step's scale of each row
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][e] *= s_run[j];
+
+    // epilogue: lane holds out[m][n .. n+3] for every (i, j)
+    if (OUT_F32) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int m = m0 + wm * 128 + j * 16 + lrow;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + wn * 64 + i * 16 + quarter * 4;
+                __builtin_nontemporal_store(acc[i][j], reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n));
+            }
+        }
+        return;
+    }
+    // bf16: turn the wave's 128 x 64 block through LDS in four parts of 32 rows (row stride 144 B), so that global
+    // stores are 16 bytes per lane and 128 contiguous bytes per row, non-temporal
+    constexpr int EST = 144;
+    uint8_t* const ebuf = smem + wave * (32 * EST);
+    const int rd_row = lane >> 3, rd_chunk = lane & 7;
+    __syncthreads();  // all waves are done reading the operand stages
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int j = h * 2 + jj;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 v = acc[i][j];
+                *reinterpret_cast<uint2*>(ebuf + (jj * 16 + lrow) * EST + (i * 16 + quarter * 4) * 2) =
+                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        }
+        // written and read by the same wave: LDS operations of one wave complete in order
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = r * 8 + rd_row;  // 0..31 within the part
+            const int m = m0 + wm * 128 + h * 32 + row;
+            const i32x4 d = *reinterpret_cast<const i32x4*>(ebuf + row * EST + rd_chunk * 16);
+            __builtin_nontemporal_store(
+                d, reinterpret_cast<i32x4*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n0 + wn * 64 + rd_chunk * 8));
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Launch record.  cfp8_gemm_dispatch_info walks the very dispatch code below with launching switched off and
 // gets back which kernels a problem would run, with grid, workgroup size and LDS bytes - so a test can pin, on
 // a machine without a GPU, that a shape still takes the kernel form its parity tests cover.
@@ -2692,6 +2933,29 @@ static int launch_block_w8(GemmArgs& p, int out_dtype, hipStream_t st) {
     return check_launch("gemm");
 }
 
+static int launch_block_256(GemmArgs& p, int out_dtype, hipStream_t st) {
+    p.tiles_m = p.M / 256;
+    p.tiles_n = p.N / 256;
+    const int64_t blocks = (int64_t)p.tiles_m * p.tiles_n;
+    if (blocks > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "gemm: too many tiles for one launch");
+    // two activation and two weight stages, the turned activation scales of two groups of 8 K steps, the tile's weight scales
+    const size_t lds = (size_t)4 * 256 * 128 + 2 * 8 * 256 * sizeof(float) + (size_t)(p.K >> 7) * 2 * sizeof(float);
+    const bool vec = (p.K >> 7) % 4 == 0 && (reinterpret_cast<uintptr_t>(p.sa) & 15u) == 0;
+    using Kern = void (*)(const GemmArgs);
+    const Kern table[2][2] = {{gemm_block_256_kernel<false, false>, gemm_block_256_kernel<true, false>},
+                              {gemm_block_256_kernel<false, true>, gemm_block_256_kernel<true, true>}};
+    const int f32 = out_dtype == CFP8_OUT_F32;
+    const Kern kern = table[vec][f32];
+    constexpr size_t lds_max = (size_t)4 * 256 * 128 + 2 * 8 * 256 * sizeof(float) + 1024 * 2 * sizeof(float);
+    static std::atomic<bool> done[65][2][2];  // zero-initialised
+    const int slot = device_slot();
+    if (slot == 64) done[64][vec][f32].store(false, std::memory_order_relaxed);
+    if (int rc = raise_lds_limit(reinterpret_cast<const void*>(kern), lds_max, done[slot][vec][f32])) return rc;
+    if (!note_launch("gemm_block_256", (unsigned)blocks, 512, lds)) return CFP8_OK;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), lds, st, p);
+    return check_launch("gemm");
+}
+
 // grouped GEMM over interleaved gate / up weights with the SwiGLU + 1x128 quantisation epilogue
 static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     constexpr int BM = 128, BN = 256;
@@ -2731,6 +2995,11 @@ static int launch_grouped_swiglu(GemmArgs& p, hipStream_t st) {
     return check_launch("gemm");
 }
 
+// the kernels that store 16 bytes per lane need every output row 16-byte aligned
+static bool out_dtype_pitch_ok(const GemmArgs& p, int out_dtype) {
+    return (p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0;
+}
+
 template <int MODE>
 static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) {
@@ -2767,6 +3036,28 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     // block scaling, large M: one 8-wave workgroup per CU on a 256 x 128 tile reads a quarter fewer operand
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
+    // block scaling from 12 K steps on, enough 256 x 256 tiles to fill the CUs in rounds that are at least 4/5 full:
+    // the 256 x 256 kernel (4096 x 18432 x K behind a flush: K = 1536 179 against 194 us, 4096 300 against 333, 7168 503
+    // against 534, 16384 x 7168 x 18432 2.01 against 2.41 ms; below 12 steps the walking 256 x 128 form is ahead, 108
+    // against 101 us at K = 1024, and 288 tiles on 256 CUs take two rounds, 208 against 186 us).  A last round that is at
+    // most half full goes to the 256 x 128 kernel as a launch of its own, as in the rowwise dispatch below.
+    if (MODE == kBlock && p.M % 256 == 0 && p.N % 256 == 0 && (p.K >> 7) >= 12 && (p.K >> 7) <= 1024 && out_dtype_pitch_ok(p, out_dtype)) {
+        const int64_t tm = p.M / 256, tn = p.N / 256, cus = cu_count(), tiles = tm * tn, rem = tiles % cus;
+        const int64_t cut = rem > 0 && rem * 2 <= cus ? (rem + tm - 1) / tm : 0;  // tile-columns that hold the partial round
+        const int64_t head = tm * (tn - cut), rounds = (head + cus - 1) / cus;
+        if (head >= cus && head * 5 >= rounds * cus * 4) {
+            if (cut == 0) return launch_block_256(p, out_dtype, st);
+            GemmArgs h = p;
+            h.N = (int)((tn - cut) * 256);
+            if (int rc = launch_block_256(h, out_dtype, st)) return rc;
+            GemmArgs tail = p;
+            tail.N = (int)(cut * 256);
+            tail.b = p.b + (int64_t)h.N * p.ld_b;
+            tail.sb = p.sb + (int64_t)(h.N >> 7) * p.sb_stride_n;
+            tail.out = static_cast<uint8_t*>(p.out) + (int64_t)h.N * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+            return launch_block_w8<256, 128, kBlock>(tail, out_dtype, st);  // at most cus tiles of 256 x 128: one round
+        }
+    }
     if (MODE == kBlock && p.M > 512 && p.M % 256 == 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
         (p.K >> 7) <= kMaxTileWeightScales)
     {

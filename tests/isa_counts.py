@@ -25,7 +25,7 @@ sys.path.insert(0, str(ROOT / "cosmos-rl_amd"))
 from cosmos_rl_amd import _build  # noqa: E402
 
 WALKING = ("gemm_rowwise_256p_kernel", "gemm_block_w8p_kernel", "gemm_mxfp4_256_kernel", "gemm_mxfp4_128_kernel",
-           "gemm_mxfp4_128x512_kernel", "gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel")
+           "gemm_mxfp4_128x512_kernel", "gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel", "gemm_block_256_kernel")
 SOURCES = ("gemm_fp8.hip", "gemm_mxfp4.hip")
 _VMEM = re.compile(r"^\s+((?:buffer|global|flat|scratch)_(?:load|store|atomic)\w*)\b(.*)")
 _PAIR = re.compile(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)")

@@ -17,6 +17,10 @@ def w8p_lds(bm, bn, kt):
     return (2 * bm + 3 * bn) * 128 + 2 * 8 * bm * 4 + 8 * 16 * 144 + 2 * 128 * 4 + 2 * ((kt * (bn // 128) + 63) & ~63) * 4
 
 
+def b256_lds(kt):
+    return 4 * 256 * 128 + 2 * 8 * 256 * 4 + kt * 2 * 4
+
+
 def w8_lds(bm, bn, kt):
     return (2 * bm + 3 * bn) * 128 + 2 * 8 * bm * 4 + kt * (bn // 128) * 4
 
@@ -39,8 +43,14 @@ CASES = [
     ("down projection M=64, split-K workspace", (LIN, 64, 3584, 18944, L.OUT_BF16, 256, True),
      "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_skinny<4,4> k_slices=4 grid=224 block=512 lds=131072; splitk_reduce grid=224 block=256 lds=0"),
     # benchmark config 4 and the short-K block shape
-    ("cfg4", (BLK, 4096, 18432, 7168), f"gemm_block_w8<256,128,block> grid=2304 block=512 lds={w8_lds(256, 128, 56)}"),
-    ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 12)}"),
+    # (1152 tiles of 256 x 256 on 256 CUs: four full rounds on the 256 x 256 kernel, the last 8 tile-columns as one round
+    # of 256 x 128 tiles)
+    ("cfg4", (BLK, 4096, 18432, 7168),
+     f"gemm_block_256 grid=1024 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=256 block=512 lds={w8_lds(256, 128, 56)}"),
+    ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_256 grid=1536 block=512 lds={b256_lds(12)}"),
+    ("block 11 K steps: the walking 256 x 128 form", (BLK, 4096, 24576, 1408), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 11)}"),
+    ("block, 288 tiles: one round of 256 x 256 tiles and the last 8 tile-columns on 256 x 128 tiles", (BLK, 1024, 18432, 7168),
+     f"gemm_block_256 grid=256 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=64 block=512 lds={w8_lds(256, 128, 56)}"),
     # benchmark config 5 (73600 padded rows)
     ("cfg5 gate_up", (GRP, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
     ("cfg5 gate_up + SwiGLU", (SWI, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped,swiglu> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),

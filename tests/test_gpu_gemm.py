@@ -271,6 +271,41 @@ def test_gemm_block128(dev, M, N, K):
     check_bf16(out16, ref, f"block {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 1536), (4096, 4352, 1664), (2048, 8192, 2048)])
+def test_gemm_block128_256x256_tiles(dev, M, N, K):
+    """The 256 x 256 block-scaled kernel (12 K steps or more, at least 256 such tiles; 4096 x 4352 also cuts the last
+    tile-column off for the 256 x 128 kernel).  It keeps a row's accumulators in the units of the running step's scale,
+    so the scales are made to jump: activation groups that are zero, tiny or a thousand times the rest, a zero and a
+    large weight block."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = (torch.randn(M, K, generator=g) * 2).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16)
+    x[:, :128] *= 1000.0
+    x[100:300, 128:256] = 0.0
+    x[:, 384:512] *= 1e-6
+    x[700:900, K - 128:] = 0.0
+    w[256:384, 256:384] = 0.0
+    w[:128, 512:640] *= 300.0
+    w[N - 128:, :128] = 0.0
+    qx, sx = O.quant_group128(x)
+    qw, sw = O.quant_block128(w)
+    ref = O.scaled_mm_block128(qx, sx, qw, sw, accum=torch.float64)
+    out32 = torch.empty(M, N, dtype=torch.float32, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out32)
+    assert bool(torch.isfinite(out32).all())
+    err = O.rel_frobenius(out32.cpu(), ref)
+    assert err <= TIGHT, f"fp32 epilogue rel Frobenius {err:.3e}"
+    # row by row as well: a row whose scales jump must be as good as the others
+    row_err = (out32.cpu().double() - ref).norm(dim=1) / ref.norm(dim=1).clamp_min(1e-30)
+    assert float(row_err.max()) <= 10 * TIGHT, f"worst row {int(row_err.argmax())}: {float(row_err.max()):.3e}"
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), out16)
+    check_bf16(out16, ref, f"block 256x256 {M}x{N}x{K}")
+    again = torch.empty_like(out32)
+    ops.gemm_fp8_fp8_bf16_nt((f8(qx, dev), sx.to(dev)), (f8(qw, dev), sw.to(dev)), again)
+    assert torch.equal(again, out32)
+
+
 def test_gemm_block128_kn_weight_layout(dev):
     """Config 4 layout: weight given [K, N], quantised with the transposing quantiser; scales stay
     [K/128, N/128].  y = x @ W."""
