@@ -258,7 +258,7 @@ def summarise_top_level(extra):
           "vendor_scaled_mm": "vendor_torch_scaled_mm_rowwise_cfg3_M8192",
           "qkv_M2048": "linear_rowwise_qkv_4608x3584_M2048", "o_M2048": "linear_rowwise_o_3584x3584_M2048",
           "gate_up_M2048": "linear_rowwise_gate_up_37888x3584_M2048", "down_M2048": "linear_rowwise_down_3584x18944_M2048"})
-    gemm("roofline_gemm_cfg4", "gemm_block128_cfg4_4096x18432x7168_incl_act_quant", "gemm_block_w8_kernel<256,128> (+ 1x128 quantiser)",
+    gemm("roofline_gemm_cfg4", "gemm_block128_cfg4_4096x18432x7168_incl_act_quant", "gemm_block_256_kernel (+ the last 8 tile-columns on gemm_block_w8_kernel<256,128>, + 1x128 quantiser)",
          "configs[3]: [4096,7168] x [7168,18432], 128x128 weight blocks, 1x128 activation groups",
          {"short_k_1536": "gemm_block128_short_k_4096x24576x1536_gemm_only"})
     gemm("roofline_gemm_cfg5", "grouped_cfg5_mlp_quant_gateup_swiglu_down", "gemm_block_w8p_kernel<128,256,grouped,SwiGLU> + gemm_block_w8_kernel<128,256,grouped>",

@@ -3036,12 +3036,12 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     // block scaling, large M: one 8-wave workgroup per CU on a 256 x 128 tile reads a quarter fewer operand
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
-    // block scaling from 12 K steps on, enough 256 x 256 tiles to fill the CUs in rounds that are at least 4/5 full:
-    // the 256 x 256 kernel (4096 x 18432 x K behind a flush: K = 1536 179 against 194 us, 4096 300 against 333, 7168 503
-    // against 534, 16384 x 7168 x 18432 2.01 against 2.41 ms; below 12 steps the walking 256 x 128 form is ahead, 108
+    // block scaling from 16 K steps on, enough 256 x 256 tiles to fill the CUs in rounds that are at least 4/5 full:
+    // the 256 x 256 kernel (4096 x 18432 x K behind a flush: K = 2048 171 against 180 us, 4096 300 against 333, 7168 503
+    // against 534, 16384 x 7168 x 18432 2.01 against 2.41 ms; at 12 steps the two are level, below that the walking 256 x 128 form is ahead, 108
     // against 101 us at K = 1024, and 288 tiles on 256 CUs take two rounds, 208 against 186 us).  A last round that is at
     // most half full goes to the 256 x 128 kernel as a launch of its own, as in the rowwise dispatch below.
-    if (MODE == kBlock && p.M % 256 == 0 && p.N % 256 == 0 && (p.K >> 7) >= 12 && (p.K >> 7) <= 1024 && out_dtype_pitch_ok(p, out_dtype)) {
+    if (MODE == kBlock && p.M % 256 == 0 && p.N % 256 == 0 && (p.K >> 7) >= 16 && (p.K >> 7) <= 1024 && out_dtype_pitch_ok(p, out_dtype)) {
         const int64_t tm = p.M / 256, tn = p.N / 256, cus = cu_count(), tiles = tm * tn, rem = tiles % cus;
         const int64_t cut = rem > 0 && rem * 2 <= cus ? (rem + tm - 1) / tm : 0;  // tile-columns that hold the partial round
         const int64_t head = tm * (tn - cut), rounds = (head + cus - 1) / cus;

@@ -47,8 +47,9 @@ CASES = [
     # of 256 x 128 tiles)
     ("cfg4", (BLK, 4096, 18432, 7168),
      f"gemm_block_256 grid=1024 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=256 block=512 lds={w8_lds(256, 128, 56)}"),
-    ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_256 grid=1536 block=512 lds={b256_lds(12)}"),
-    ("block 11 K steps: the walking 256 x 128 form", (BLK, 4096, 24576, 1408), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 11)}"),
+    ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 12)}"),
+    ("block 15 K steps: still the walking 256 x 128 form", (BLK, 4096, 24576, 1920), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 15)}"),
+    ("block 16 K steps: 256 x 256 tiles", (BLK, 4096, 24576, 2048), f"gemm_block_256 grid=1536 block=512 lds={b256_lds(16)}"),
     ("block, 288 tiles: one round of 256 x 256 tiles and the last 8 tile-columns on 256 x 128 tiles", (BLK, 1024, 18432, 7168),
      f"gemm_block_256 grid=256 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=64 block=512 lds={w8_lds(256, 128, 56)}"),
     # benchmark config 5 (73600 padded rows)

@@ -271,9 +271,9 @@ def test_gemm_block128(dev, M, N, K):
     check_bf16(out16, ref, f"block {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4096, 1536), (4096, 4352, 1664), (2048, 8192, 2048)])
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 2048), (4096, 4352, 2176), (2048, 8192, 2560)])
 def test_gemm_block128_256x256_tiles(dev, M, N, K):
-    """The 256 x 256 block-scaled kernel (12 K steps or more, at least 256 such tiles; 4096 x 4352 also cuts the last
+    """The 256 x 256 block-scaled kernel (16 K steps or more, at least 256 such tiles; 4096 x 4352 also cuts the last
     tile-column off for the 256 x 128 kernel).  It keeps a row's accumulators in the units of the running step's scale,
     so the scales are made to jump: activation groups that are zero, tiny or a thousand times the rest, a zero and a
     large weight block."""
