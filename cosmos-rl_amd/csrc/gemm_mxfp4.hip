@@ -1522,6 +1522,27 @@ static int ensure_lds(const void* fn, size_t lds, std::atomic<bool> (&raised)[64
     return CFP8_OK;
 }
 
+// compute units of the current device (256 if the query fails), cached per device ordinal
+static int mx4_cu_count() {
+    static std::atomic<int> cached[64];  // zero-initialised
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < 64) {
+        const int c = cached[dev].load(std::memory_order_relaxed);
+        if (c > 0) return c;
+    }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
 static int launch_mx4_256(Mx4Args p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 256;
     p.tiles_n = p.N / 256;
@@ -1797,8 +1818,25 @@ extern "C" int cfp8_gemm_mxfp4(const void* a, int64_t ld_a, const float* sa, con
     // 256 x 256 tiles of the direct-to-LDS pipeline once they fill at least half of the GPU
     const bool out16 = (reinterpret_cast<uintptr_t>(out) & 15u) == 0 && (ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2)) % 16 == 0;
     if (!m_indices && M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && ld_ws % 4 == 0 && (reinterpret_cast<uintptr_t>(ws) & 3u) == 0 &&
-        out16 && (M / 256) * (N / 256) >= 128 && (M / 256) * (N / 256) <= 0x7FFFFFFFll)
+        out16 && (M / 256) * (N / 256) >= 128 && (M / 256) * (N / 256) <= 0x7FFFFFFFll) {
+        // One workgroup per CU and equal tiles: the launch runs in rounds of as many tiles as there are CUs, and a last
+        // round that is at most half full costs a whole round.  Then the last tile-columns go to a second launch on
+        // smaller tiles and the first launch ends on a full round.
+        const int64_t tm = M / 256, tn = N / 256, cus = mx4_cu_count(), rem = (tm * tn) % cus;
+        const int64_t cut = (rem + tm - 1) / tm;  // tile-columns that hold the partial round
+        if (tm * tn > cus && rem > 0 && rem * 2 <= cus && cut < tn) {
+            Mx4Args head = p;
+            head.N = (int)((tn - cut) * 256);
+            if (int rc = launch_mx4_256(head, out_dtype, st)) return rc;
+            Mx4Args tail = p;
+            tail.N = (int)(cut * 256);
+            tail.w = p.w + (int64_t)head.N * ld_w;
+            tail.ws = p.ws + (int64_t)head.N * ld_ws;
+            tail.out = static_cast<uint8_t*>(out) + (int64_t)head.N * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+            return launch_mx4_128(tail, out_dtype, st);
+        }
         return launch_mx4_256(p, out_dtype, st);
+    }
     // every other shape with enough 128 x 256 tiles, and the grouped layout: the same pipeline with edges
     // (128 x 512 tiles when that still gives every CU a tile and wastes under an eighth of the last tile-column)
     // (its byte offsets inside a tile reach 463 weight rows: the pitch must stay below 2^23 for 32 bits)

@@ -172,7 +172,9 @@ def _rel(got, want):
                                    (2048, 4096, 384), (4096, 8192, 128), (2048, 4096, 256), (2560, 3328, 1152),
                                    (2000, 2064, 2880), (1025, 4112, 160), (8192, 272, 128), (130, 16400, 416), (1024, 4096, 3552),
                                    (4000, 4112, 160), (8192, 2544, 416), (4100, 4096, 2880),
-                                   (100, 10480, 2880), (128, 16400, 160), (17, 12272, 4256), (65, 10256, 128), (90, 18944, 3584), (40, 20016, 1184)])
+                                   (100, 10480, 2880), (128, 16400, 160), (17, 12272, 4256), (65, 10256, 128), (90, 18944, 3584), (40, 20016, 1184),
+                                   # 272 and 320 tiles of 256 x 256: one full round, the last tile-columns as a second launch
+                                   (4096, 4352, 256), (2048, 10240, 384)])
 def test_gemm_mxfp4_against_oracle(dev, M, N, K):
     """fp32 output within 1e-4 (relative Frobenius; the fp32 accumulation of the matrix pipe) of the exact sum, bf16 output within 1e-3 of the bf16-rounded
     exact sum; rows and columns beyond M and N of a padded output stay untouched."""
