@@ -117,6 +117,26 @@ def test_graph_fp8_linear(dev, M, N, K):
     _replay_matches_eager(dev, inputs, fn)
 
 
+def test_graph_block_gemm_256x256_tiles(dev):
+    """1x128 activation quantiser + the block-scaled GEMM on 256 x 256 tiles with its last tile-column as a second
+    launch (272 tiles), and a K that is a multiple of 16 only through the rowwise linear's masked last step."""
+    M, N, K = 4096, 4352, 2048
+    qw, sw = ops.per_block_cast_to_fp8(_bf16(dev, 6, N, K, std=0.02))
+    w2 = _bf16(dev, 7, 512, 1200, std=0.02)
+    qw2, sw2 = ops.quant_rowwise(w2)
+
+    def inputs(seed):
+        return [_bf16(dev, seed, M, K), _bf16(dev, seed + 100, 100, 1200)]
+
+    def fn(x, x2):
+        qx, sx = ops.groupwise_activation_quant(x)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+        ops.gemm_fp8_fp8_bf16_nt((qx, sx), (qw, sw), out)
+        return (out, ops.fp8_linear(x2, qw2.t(), sw2))
+
+    _replay_matches_eager(dev, inputs, fn)
+
+
 def test_graph_moe_chain(dev):
     from cosmos_rl_amd import _lib
     from cosmos_rl_amd.policy.kernel.moe.moe import combine_expert_outputs, route_tokens
