@@ -3036,6 +3036,20 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (p.M <= 64) return launch_cfg<64, 64, 1, 4, MODE>(p, out_dtype, st);
     // block scaling, large M: one 8-wave workgroup per CU on a 256 x 128 tile reads a quarter fewer operand
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
+    // block scaling, any number of tokens above 512: the first M / 256 * 256 rows take the full-tile kernels below, the
+    // last < 256 rows are a small problem of their own (rows are independent, so the split changes no row's result)
+    if (MODE == kBlock && p.M > 512 && p.M % 256 != 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
+        (p.K >> 7) <= kMaxTileWeightScales) {
+        GemmArgs body = p;
+        body.M = p.M / 256 * 256;
+        if (int rc = launch_gemm<MODE>(body, out_dtype, st)) return rc;
+        GemmArgs rest = p;
+        rest.M = p.M - body.M;
+        rest.a = p.a + (int64_t)body.M * p.ld_a;
+        rest.sa = p.sa + (int64_t)body.M * (p.K >> 7);
+        rest.out = static_cast<uint8_t*>(p.out) + (int64_t)body.M * p.ld_out * (out_dtype == CFP8_OUT_F32 ? 4 : 2);
+        return launch_gemm<MODE>(rest, out_dtype, st);
+    }
     // block scaling from 16 K steps on, enough 256 x 256 tiles to fill the CUs in rounds that are at least 4/5 full:
     // the 256 x 256 kernel (4096 x 18432 x K behind a flush: K = 2048 171 against 180 us, 4096 300 against 333, 7168 503
     // against 534, 16384 x 7168 x 18432 2.01 against 2.41 ms; at 12 steps the two are level, below that the walking 256 x 128 form is ahead, 108

@@ -50,6 +50,9 @@ CASES = [
     ("block short K", (BLK, 4096, 24576, 1536), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 12)}"),
     ("block 15 K steps: still the walking 256 x 128 form", (BLK, 4096, 24576, 1920), f"gemm_block_w8p<256,128,block> grid=256 block=512 lds={w8p_lds(256, 128, 15)}"),
     ("block 16 K steps: 256 x 256 tiles", (BLK, 4096, 24576, 2048), f"gemm_block_256 grid=1536 block=512 lds={b256_lds(16)}"),
+    ("block, 4000 tokens: 3840 rows on full tiles, 160 as a problem of their own", (BLK, 4000, 18432, 7168),
+     f"gemm_block_256 grid=1020 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=120 block=512 lds={w8_lds(256, 128, 56)}; "
+     "gemm_kernel<128,128,2,2,block> grid=288 block=256 lds=73728"),
     ("block, 288 tiles: one round of 256 x 256 tiles and the last 8 tile-columns on 256 x 128 tiles", (BLK, 1024, 18432, 7168),
      f"gemm_block_256 grid=256 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=64 block=512 lds={w8_lds(256, 128, 56)}"),
     # benchmark config 5 (73600 padded rows)

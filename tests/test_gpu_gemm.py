@@ -255,7 +255,10 @@ def block_operands(M, N, K, seed):
                                    (1024, 12288, 640), (768, 16384, 128), (1024, 12416, 1152), (1280, 10240, 2176),
                                    # the same with 16-byte scale loads: K of 8 and 12 steps (one group of eight steps, one and
                                    # a half); 516 tiles (two full rounds of one tile per CU and a short one) with K of 3 steps
-                                   (1024, 12288, 1024), (1024, 12288, 1536), (768, 22016, 384)])
+                                   (1024, 12288, 1024), (1024, 12288, 1536), (768, 22016, 384),
+                                   # a token count that is no multiple of 256: full tiles for the first 768 / 1024 rows, the
+                                   # last 232 / 1 as a launch of their own
+                                   (1000, 16384, 640), (1025, 12288, 384)])
 def test_gemm_block128(dev, M, N, K):
     # the last two shapes have >= 384 tiles of 256 x 128 and take the 8-wave 256 x 128 kernel: one with a
     # ragged last tile-row and K/128 not a multiple of 4 (scalar scale loads), one with 16-byte scale loads
