@@ -3093,6 +3093,9 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
         // multiple of 256
         const int64_t t256 = (int64_t)(p.M / 256) * ((p.N + 255) / 256);
         if (p.N % 256 != 0 || t256 <= 128) return launch_rowwise_256x128(p, out_dtype, st);
+        // 512 rows on a wide weight: 129 .. 256 tiles of 256 x 256, one round of the direct-to-LDS kernel (config 3's
+        // weight: 58 against 67 us for the register-staged 256 x 256 configuration below)
+        if (p.M == 512) return launch_rowwise_256(p, out_dtype, st);
     }
     // 257..512 rows 7 % faster on 256 x 256 tiles than on 128 x 128
     if (MODE == kRowwise && p.M > 128 && p.M <= 256) return launch_cfg<256, 128, 4, 2, kRowwise>(p, out_dtype, st);

@@ -34,6 +34,7 @@ CASES = [
      "gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
     ("cfg3 M=1024", (ROW, 1024, 18944, 3584),
      f"gemm_rowwise_256 grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=160 block=256 lds=65536"),
+    ("cfg3 M=512: one round of 256 x 256 tiles", (ROW, 512, 18944, 3584), f"gemm_rowwise_256 grid=148 block=256 lds={LDS_ROW}"),
     ("cfg3 M=64", (LIN, 64, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),
     ("cfg3 M=17", (LIN, 17, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),
     ("cfg3 M=128", (LIN, 128, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<128,5> grid=237 block=256 lds=143360"),

@@ -61,7 +61,9 @@ def rowwise_operands(M, N, K, seed, dev):
                                    (18, 24592, 256), (50, 28688, 128), (32, 40976, 128),
                                    # 65..128 tokens: its 128-row form, ring of five stages, K of 1, 3, 5, 9 and 28 steps
                                    (65, 12272, 384), (128, 16400, 1152), (100, 20016, 128), (127, 10480, 640), (96, 18944, 3584),
-                                   (128, 4608, 896)])
+                                   (128, 4608, 896),
+                                   # 512 tokens on a wide weight: one round of 256 x 256 tiles of the direct-to-LDS kernel
+                                   (512, 16640, 384)])
 def test_scaled_mm_rowwise(dev, M, N, K):
     x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=M + N + K, dev=dev)
     ref = O.scaled_mm_rowwise(qx, sx, qw, sw, accum=torch.float64)
