@@ -15,6 +15,7 @@ OUT_BF16 = 0
 OUT_F32 = 1
 GROUP_MODE_DIV = 0
 GROUP_MODE_DEEPEP = 1
+SCALE_F32, SCALE_E8M0 = 0, 1
 TENSORWISE_AMAX_SLOTS = 64
 TENSORWISE_STATIC_MAX_TENSORS = 512
 IN_BF16, IN_F16, IN_F32 = 0, 1, 2
@@ -42,6 +43,8 @@ SIGNATURES = {
     "cfp8_quant_tensorwise_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise_multi_static": (c_int, [POINTER(TensorDesc), c_int64, c_void_p]),
     "cfp8_tensorwise_resident": (c_int, [c_int]),
+    "cfp8_tensorwise_status": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+    "cfp8_tensorwise_resident_tuning": (c_int, [c_int64, c_int]),
     "cfp8_tensorwise_amax_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_tensorwise_cast_multi": (c_int, [POINTER(TensorDesc), c_int64, c_void_p, c_void_p]),
     "cfp8_quant_tensorwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -63,6 +66,7 @@ SIGNATURES = {
     "cfp8_scatter_quant_group128": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64,
                                             c_void_p, c_void_p]),
     "cfp8_dequant_block128": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "cfp8_dequant_group128": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int, c_int64, c_int64, c_void_p, c_int64, c_int, c_void_p]),
     "cfp8_scaled_mm_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                        c_int, c_int64, c_int64, c_int64, c_void_p]),
     "cfp8_linear_workspace_bytes": (c_size_t, [c_int64, c_int64]),

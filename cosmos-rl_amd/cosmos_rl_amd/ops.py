@@ -7,6 +7,7 @@ must live on the GPU; nothing here computes on the CPU.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import List, Optional, Sequence, Tuple
 
@@ -169,12 +170,28 @@ def quant_rowwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Ten
     return qs, ss
 
 
-def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.Tensor], torch.Tensor]:
+@contextlib.contextmanager
+def gpu_is_mine():
+    """While active, ``quant_tensorwise_multi`` may use the launch that reads large tensors once and needs every
+    compute unit of the GPU at the same time (``cfp8_tensorwise_resident``).  For a process that owns the GPU while
+    it quantises, e.g. a trainer casting its weights; process-wide, restores the previous setting on exit."""
+    lib = _lib.load()
+    prev = lib.cfp8_tensorwise_resident(1)
+    try:
+        yield
+    finally:
+        lib.cfp8_tensorwise_resident(prev)
+
+
+def quant_tensorwise_multi(tensors: Sequence[torch.Tensor], return_status: bool = False):
     """Tensorwise dynamic quantisation of a list of bf16 tensors in two launches per
-    batch.  Returns (list of fp8 tensors shaped like the inputs, fp32 scales [n])."""
+    batch.  Returns (list of fp8 tensors shaped like the inputs, fp32 scales [n]); with ``return_status`` also a
+    device int32 scalar, the number of tensors that the read-once launch (see ``gpu_is_mine``) gave up and the
+    two ordinary passes redid - nonzero means that the GPU was not the caller's alone; results are right either way."""
     n = len(tensors)
     if n == 0:
-        return [], torch.empty(0, dtype=torch.float32)
+        empty = ([], torch.empty(0, dtype=torch.float32))
+        return (*empty, torch.zeros((), dtype=torch.int32)) if return_status else empty
     _need_gpu(*tensors)
     dev = tensors[0].device
     scales = torch.empty(n, dtype=torch.float32, device=dev)
@@ -195,6 +212,10 @@ def quant_tensorwise_multi(tensors: Sequence[torch.Tensor]) -> Tuple[List[torch.
         descs[i].scale = sbase + 4 * i
         descs[i].numel = tc.numel()
     _lib.check(_lib.load().cfp8_quant_tensorwise_multi(descs, n, amax_ws.data_ptr(), _stream()))
+    if return_status:
+        given_up = torch.empty((), dtype=torch.int32, device=dev)
+        _lib.check(_lib.load().cfp8_tensorwise_status(amax_ws.data_ptr(), n, given_up.data_ptr(), _stream()))
+        return outs, scales, given_up
     return outs, scales
 
 
@@ -393,6 +414,34 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """``per_token_cast_to_fp8`` of the reference's tests/test_deepep.py:75-85, including its
     formula ``x * (448 / amax.clamp(1e-4))`` with scales ``amax / 448``."""
     return _group128(x, _lib.GROUP_MODE_DEEPEP)
+
+
+def per_token_cast_back(x_fp8: torch.Tensor, x_scales: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``per_token_cast_back`` of the reference's tests/test_deepep.py:86-108: ``bf16(fp32(x_fp8) * scale)`` with one
+    scale per row and group of 128 columns.  ``x_scales`` is fp32 ``[m, ceil(n / 128)]`` or, as in the reference's
+    ``x_scales.dtype == torch.int`` branch (:97-99), int32 holding four E8M0 exponent bytes each, lowest byte first
+    (``[m, ceil(n / 128) / 4]``)."""
+    if x_fp8.numel() == 0:
+        return x_fp8.to(out_dtype)
+    _need_gpu(x_fp8, x_scales)
+    assert x_fp8.dim() == 2 and x_fp8.dtype == FP8_DTYPE
+    m, n = x_fp8.shape
+    groups = -(-n // BLOCK)
+    q = x_fp8 if x_fp8.is_contiguous() else x_fp8.contiguous()
+    if x_scales.dtype == torch.int32:
+        sc = x_scales.contiguous().view(torch.uint8).view(m, -1)
+        kind = _lib.SCALE_E8M0
+    elif x_scales.dtype == torch.float32:
+        sc = x_scales.contiguous().view(m, -1)
+        kind = _lib.SCALE_F32
+    else:
+        raise ValueError(f"scales must be float32 or packed int32, got {x_scales.dtype}")
+    if sc.shape[1] < groups:
+        raise ValueError(f"{sc.shape[1]} scales per row do not cover {n} columns")
+    y = torch.empty((m, n), dtype=out_dtype, device=x_fp8.device)
+    _lib.check(_lib.load().cfp8_dequant_group128(q.data_ptr(), n, sc.data_ptr(), sc.shape[1], kind, m, n, y.data_ptr(), n,
+                                                _out_code(out_dtype), _stream()))
+    return y
 
 
 def weight_dequant(x: torch.Tensor, s: torch.Tensor, block_size: int = 128,

@@ -34,13 +34,27 @@ class GroupGEMMStrategy:
 
 
 class TorchBF16GroupGEMM(GroupGEMMStrategy):
-    """bf16 baseline: one matmul per expert group (the reference uses ``torch._grouped_mm``)."""
+    """bf16 baseline (group_gemms.py:80-118): ``torch._grouped_mm`` with int32 ``m_offsets``, which stay on the
+    device; where this torch build has no grouped kernel for the operands (the CPU, notably) one matmul per
+    expert group, which reads the offsets back."""
+
+    _native = None  # None: not tried yet; True / False: torch._grouped_mm works / does not for these operands
 
     def arrange_expert_weights(self, all_weights, submod_name, module):
         return torch.stack(all_weights)
 
-    @staticmethod
-    def _grouped(x, w, m_offsets):
+    @classmethod
+    def _grouped(cls, x, w, m_offsets):
+        if cls._native is not False and x.is_cuda and hasattr(torch, "_grouped_mm"):
+            offs = m_offsets if m_offsets.dtype == torch.int32 else m_offsets.to(torch.int32)
+            try:
+                out = torch._grouped_mm(x, w.transpose(-2, -1), offs, out_dtype=torch.bfloat16)
+                cls._native = True
+                return out
+            except (RuntimeError, NotImplementedError):
+                if cls._native:
+                    raise
+                cls._native = False
         out = torch.zeros(x.shape[0], w.shape[1], dtype=torch.bfloat16, device=x.device)
         start = 0
         for e, end in enumerate(m_offsets.tolist()):

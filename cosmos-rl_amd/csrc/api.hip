@@ -48,6 +48,6 @@ int check_device() {
 
 }  // namespace cfp8
 
-extern "C" int cfp8_version(void) { return 100; }
+extern "C" int cfp8_version(void) { return 101; }
 
 extern "C" const char* cfp8_last_error(void) { return cfp8::g_err; }

@@ -206,6 +206,46 @@ __device__ __forceinline__ uint2 cast8(const uint4& v, const Divider& d) {
     return make_uint2(o[0], o[1]);
 }
 
+// cast8 for a scale that need not come from the data's own maximum: the quotient saturates at +-448 before the
+// conversion, like the reference's clamp in front of its cast.  The decision is taken on the first product
+// x * (1 / s): beyond 460 in magnitude (infinite included: a huge x over a small s, or x = +-inf, where the
+// correction step would produce inf - inf) the result is +-448 with that sign; up to 460 the corrected quotient
+// is below 464 and the conversion rounds it to at most 448 by itself.  A vector that holds a NaN is converted
+// element by element, the NaN elements to the byte 0x7F (the hardware conversion of a NaN is not relied on).
+__device__ __forceinline__ u32 absmax8(u32 acc, const uint4& v);
+__device__ __forceinline__ uint2 cast8_clamped(const uint4& v, const Divider& d) {
+    if (!d.finite) return cast8(v, d);
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+    auto q = [&](float x) {
+        const float q0 = x * d.r;
+        const float e = __builtin_fmaf(q0, d.s, -x);
+        const float y = __builtin_fmaf(-e, d.r, q0);
+        return __builtin_fabsf(q0) > 460.0f ? __builtin_copysignf(kE4M3Max, q0) : y;
+    };
+    u32 o[2];
+    if (pk_fold(absmax8(0u, v)) > 0x7F80u) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            u32 bytes = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const u32 word = w[2 * i + (e >> 1)];
+                const float x = (e & 1) ? bf16_hi(word) : bf16_lo(word);
+                const u32 b = x != x ? 0x7Fu : (cvt2<false>(q(x), 0.0f, 0u) & 0xFFu);
+                bytes |= b << (8 * e);
+            }
+            o[i] = bytes;
+        }
+        return make_uint2(o[0], o[1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        u32 p = cvt2<false>(q(bf16_lo(w[2 * i])), q(bf16_hi(w[2 * i])), 0u);
+        o[i] = cvt2<true>(q(bf16_lo(w[2 * i + 1])), q(bf16_hi(w[2 * i + 1])), p);
+    }
+    return make_uint2(o[0], o[1]);
+}
+
 __device__ __forceinline__ u32 absmax8(u32 acc, const uint4& v) {
     acc = pk_absmax(acc, v.x);
     acc = pk_absmax(acc, v.y);

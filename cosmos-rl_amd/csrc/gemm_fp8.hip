@@ -3038,7 +3038,8 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     // bytes than two 128 x 128 workgroups, as long as there are enough tiles to fill the 256 CUs
     // block scaling, any number of tokens above 512: the first M / 256 * 256 rows take the full-tile kernels below, the
     // last < 256 rows are a small problem of their own (rows are independent, so the split changes no row's result)
-    if (MODE == kBlock && p.M > 512 && p.M % 256 != 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
+    // (from 768 rows on: a body of 512 rows would fall below the `M > 512` of the full-tile forms it is cut out for)
+    if (MODE == kBlock && p.M >= 768 && p.M % 256 != 0 && p.N % 128 == 0 && (int64_t)(p.M / 256) * (p.N / 128) >= 384 &&
         (p.K >> 7) <= kMaxTileWeightScales) {
         GemmArgs body = p;
         body.M = p.M / 256 * 256;

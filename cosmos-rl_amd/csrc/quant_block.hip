@@ -213,6 +213,54 @@ __global__ __launch_bounds__(256) void dequant_block128_kernel(const uint8_t* __
     }
 }
 
+// ---------------------------------------------------------------------------
+// 1x128 group dequantiser: y[i, j] = fp8[i, j] * s[i, j / 128], the inverse of group128_kernel.  The thread layout of
+// the block dequantiser (one 8-column vector of four consecutive rows per thread), with a scale per row and group.
+// E8M0: the scales are one exponent byte per group, value 2^(byte - 127) formed as the fp32 bit pattern byte << 23
+// (byte 0 gives +0 and byte 255 +infinity, as that shift does).
+// ---------------------------------------------------------------------------
+template <bool F32, bool E8M0>
+__global__ __launch_bounds__(256) void dequant_group128_kernel(const uint8_t* __restrict__ q, int64_t ld_q,
+                                                               const void* __restrict__ s, int64_t ld_s, int64_t rows,
+                                                               int nvec_row, void* __restrict__ y, int64_t ld_y) {
+    const int cv = blockIdx.x * blockDim.x + threadIdx.x;
+    if (cv >= nvec_row) return;
+    for (int64_t r0 = ((int64_t)blockIdx.y * blockDim.y + threadIdx.y) * 4; r0 < rows;
+         r0 += (int64_t)gridDim.y * blockDim.y * 4) {
+        uint2 w[4];
+        float sc[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t r = r0 + k < rows ? r0 + k : rows - 1;
+            const u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + r * ld_q + (int64_t)cv * 8));
+            w[k] = make_uint2(t[0], t[1]);
+            if (E8M0) sc[k] = __uint_as_float((u32) static_cast<const uint8_t*>(s)[r * ld_s + (cv >> 4)] << 23);
+            else sc[k] = static_cast<const float*>(s)[r * ld_s + (cv >> 4)];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (r0 + k >= rows) break;
+            float f[8];
+            f32x2 p;
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].x, false); f[0] = p[0]; f[1] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].x, true);  f[2] = p[0]; f[3] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].y, false); f[4] = p[0]; f[5] = p[1];
+            p = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[k].y, true);  f[6] = p[0]; f[7] = p[1];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] *= sc[k];
+            const int64_t at = (r0 + k) * ld_y + (int64_t)cv * 8;
+            if (F32) {
+                uint4* o = reinterpret_cast<uint4*>(static_cast<float*>(y) + at);
+                st16<true>(o, make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])));
+                st16<true>(o + 1, make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]), __float_as_uint(f[7])));
+            } else {
+                st16<true>(reinterpret_cast<uint4*>(static_cast<uint16_t*>(y) + at),
+                           make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])));
+            }
+        }
+    }
+}
+
 // SwiGLU fused with the 1x128 quantiser: h = bf16(bf16(silu(g)) * u) is formed in registers from the
 // two bf16 GEMM outputs and quantised like group128_kernel<DIV> does; h never exists in memory.
 // The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors (swiglu_pair).
@@ -480,4 +528,35 @@ extern "C" int cfp8_dequant_block128(const void* q, const float* scales, int64_t
         hipLaunchKernelGGL(dequant_block128_kernel<false>, grid, block, 0, st, static_cast<const uint8_t*>(q), scales, rows, cols,
                            (int)nvec_row, tc, y);
     return check_launch("dequant_block128");
+}
+
+extern "C" int cfp8_dequant_group128(const void* q, int64_t ld_q, const void* scales, int64_t ld_scales, int scale_kind,
+                                     int64_t rows, int64_t cols, void* y, int64_t ld_y, int out_dtype, void* stream) {
+    using namespace cfp8;
+    if (rows < 0 || cols < 0) return set_error(CFP8_EINVAL, "dequant_group128: negative shape");
+    if (rows == 0 || cols == 0) return CFP8_OK;
+    if (!q || !scales || !y) return set_error(CFP8_EINVAL, "dequant_group128: null pointer");
+    if (out_dtype != CFP8_OUT_BF16 && out_dtype != CFP8_OUT_F32) return set_error(CFP8_EINVAL, "dequant_group128: unknown out_dtype %d", out_dtype);
+    if (scale_kind != CFP8_SCALE_F32 && scale_kind != CFP8_SCALE_E8M0) return set_error(CFP8_EINVAL, "dequant_group128: unknown scale_kind %d", scale_kind);
+    const int64_t ngroups = (cols + 127) / 128;
+    if (cols % 8 || ld_q % 8 || ld_q < cols || ld_y < cols || ld_y % (out_dtype == CFP8_OUT_F32 ? 4 : 8) || ld_scales < ngroups)
+        return set_error(CFP8_EINVAL, "dequant_group128: cols=%lld ld_q=%lld ld_y=%lld ld_scales=%lld: cols and ld_q must be multiples of 8, "
+                         "rows of y 16-byte aligned, and every pitch at least its row", (long long)cols, (long long)ld_q, (long long)ld_y, (long long)ld_scales);
+    if ((reinterpret_cast<uintptr_t>(q) & 7u) || !aligned16(y) || (scale_kind == CFP8_SCALE_F32 && (reinterpret_cast<uintptr_t>(scales) & 3u)))
+        return set_error(CFP8_EINVAL, "dequant_group128: misaligned pointer");
+    const int64_t nvec_row = cols / 8;
+    const int bx = nvec_row > 128 ? 256 : nvec_row > 64 ? 128 : 64, by = 256 / bx;
+    int64_t gx = (nvec_row + bx - 1) / bx, gy = (rows + 4 * by - 1) / (4 * by);
+    if (gx > 0x7FFFFFFFll) return set_error(CFP8_EINVAL, "dequant_group128: shape exceeds the grid limits");
+    if (gy > 65535) gy = 65535;  // the kernel strides over the remaining row quads
+    if (int rc = check_device()) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)gx, (unsigned)gy), block(bx, by);
+    const uint8_t* qp = static_cast<const uint8_t*>(q);
+    const bool f32 = out_dtype == CFP8_OUT_F32, e8 = scale_kind == CFP8_SCALE_E8M0;
+    if (f32 && e8) hipLaunchKernelGGL((dequant_group128_kernel<true, true>), grid, block, 0, st, qp, ld_q, scales, ld_scales, rows, (int)nvec_row, y, ld_y);
+    else if (f32) hipLaunchKernelGGL((dequant_group128_kernel<true, false>), grid, block, 0, st, qp, ld_q, scales, ld_scales, rows, (int)nvec_row, y, ld_y);
+    else if (e8) hipLaunchKernelGGL((dequant_group128_kernel<false, true>), grid, block, 0, st, qp, ld_q, scales, ld_scales, rows, (int)nvec_row, y, ld_y);
+    else hipLaunchKernelGGL((dequant_group128_kernel<false, false>), grid, block, 0, st, qp, ld_q, scales, ld_scales, rows, (int)nvec_row, y, ld_y);
+    return check_launch("dequant_group128");
 }

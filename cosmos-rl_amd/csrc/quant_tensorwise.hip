@@ -11,7 +11,9 @@
 //                  so the 64 slots are two cache lines, and one atomic per 32 KiB
 //                  holds a 1 GB tensor at 5.2 TB/s where the same loads without
 //                  the atomic reach 6.9: a large launch therefore gives every
-//                  workgroup up to 8 chunks (one atomic per 256 KiB).
+//                  workgroup up to 8 chunks (one atomic per 256 KiB).  The maxima
+//                  use slots 0 .. kAmaxSlots - 2; the last slot is the tensor's
+//                  status word (see the resident kernel below), zero here.
 //   pass 2 (cast)  reads 2 B and writes 1 B per element; every workgroup folds
 //                  the tensor's slots and forms the scale on its own.
 // The table of tensors travels in the kernel arguments (scalar loads), so the
@@ -27,6 +29,8 @@ namespace cfp8 {
 constexpr int kMaxBatch = 48;
 constexpr int kChunkVecs = 256 * 8;  // 16-byte vectors per workgroup: 32 KiB of bf16
 constexpr int kAmaxSlots = CFP8_TENSORWISE_AMAX_SLOTS;  // one wavefront reads them in one load
+constexpr int kMaxSlots = kAmaxSlots - 1;                // slots that hold maxima; slot kStatusSlot is the status word
+constexpr int kStatusSlot = kAmaxSlots - 1;
 constexpr int kMaxDevices = 64;  // device ordinals with per-device state of their own
 
 struct TensorTable {
@@ -92,11 +96,15 @@ __global__ __launch_bounds__(256) void tensorwise_amax_kernel(const TensorTable 
     __syncthreads();
     if (threadIdx.x == 0) {
         m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;  // fp32 bit pattern of the workgroup's amax
-        if (m) atomicMax(tb.amax[t] + (local & (kAmaxSlots - 1)), m);  // result unused: the wave does not wait
+        if (m) atomicMax(tb.amax[t] + local % (unsigned)kMaxSlots, m);  // result unused: the wave does not wait
     }
 }
 
-template <bool LDNT, bool STNT>
+// CLAMP: the quotient is clamped to +-448 before the conversion.  The fused call needs no clamp (the scale comes
+// from the maximum of the very data that is cast, so no quotient exceeds 448 by more than one fp32 step and the
+// conversion rounds that to 448 by itself); the split-phase cast takes the caller's slots, which an all-reduce or
+// a stale workspace may have left smaller than the tensor's own maximum, and saturates like the reference's cast.
+template <bool LDNT, bool STNT, bool CLAMP>
 __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable tb) {
     const int t = find_tensor(tb, blockIdx.x);
     const unsigned local = blockIdx.x - tb.first_block[t];
@@ -106,21 +114,23 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
     uint2* q = tb.q[t] + base;
     const int64_t left = nvec - base;
     static_assert(kAmaxSlots == 64, "one slot per lane");
-    const float amax = __uint_as_float(wave_max(tb.amax[t][threadIdx.x & 63]));
+    const int slot = threadIdx.x & 63;
+    const float amax = __uint_as_float(wave_max(slot < kMaxSlots ? tb.amax[t][slot] : 0u));
     const float scale = scale_from_amax(amax);
     if (local == 0 && threadIdx.x == 0) *tb.scale[t] = scale;
     const Divider d(scale);
+    auto cast = [&](const uint4& v) { return CLAMP ? cast8_clamped(v, d) : cast8(v, d); };
     uint4 v[8];
     if (left >= kChunkVecs) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = ld16<LDNT>(x + threadIdx.x + 256 * i);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) st8<STNT>(q + threadIdx.x + 256 * i, cast8(v[i], d));
+        for (int i = 0; i < 8; ++i) st8<STNT>(q + threadIdx.x + 256 * i, cast(v[i]));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             int idx = threadIdx.x + 256 * i;
-            if (idx < left) st8<STNT>(q + idx, cast8(ld16<LDNT>(x + idx), d));
+            if (idx < left) st8<STNT>(q + idx, cast(ld16<LDNT>(x + idx)));
         }
     }
 }
@@ -139,14 +149,27 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
 // wave runs per tensor is 30 KB of straight line, shared by the CU's twelve waves and small enough to stay in
 // the instruction cache from one tensor to the next (with one wave per SIMD and all 512 registers it was 350 KB
 // and the kernel spent its time fetching it).
-// The wait at the counter is bounded by the wall clock, so every wave leaves the kernel whatever happens; a
-// workgroup that gives up poisons the tensor's scale and bytes with NaN.  The launch needs all its workgroups
-// resident at once: the grid is one workgroup per CU and a workgroup takes a whole CU, so on a GPU that no
-// other grid holds they are.  Two such launches on different streams of one GPU could each hold part of the
-// CUs and wait for the rest until the bound expires: callers that run this path from several streams at once
-// switch it off (cfp8_tensorwise_resident).
+// The launch needs all its workgroups resident at once: the grid is one workgroup per CU and a workgroup takes a
+// whole CU, so on a GPU that no other grid holds they are.  Where they are not (another stream's or process's
+// kernel holds CUs, a second launch of this kind, a CU mask) the meeting cannot complete, so the wait at the
+// counter is bounded by the wall clock and every wave leaves the kernel whatever happens.  The counter makes the
+// outcome of a tensor the same for every workgroup: its low half counts arrivals, its high half counts
+// workgroups that gave up.  A workgroup gives up by a compare-and-swap that adds to the high half of a value it
+// has just read with an incomplete count; from then on no value of the counter is both complete and clean, so no
+// workgroup can take the tensor for met, and before that none could.  A tensor that was given up is left alone by
+// every workgroup (no byte, no scale), its status word (slot kStatusSlot of its amax slots) and those of the
+// tensors behind it in the launch are set, and the kernel ends.  The two repair kernels that follow every
+// resident launch on the same stream redo exactly the tensors whose status word is set as two ordinary passes
+// (a few microseconds when there is none), so the call's results are right either way; the status words stay
+// set in the caller's workspace until its next use and cfp8_tensorwise_status counts them.
+// The form is opt-in (cfp8_tensorwise_resident): a process switches it on when it has the GPU to itself while it
+// quantises.
 // ---------------------------------------------------------------------------
-static std::atomic<int> g_resident_enabled{1};
+static std::atomic<int> g_resident_enabled{0};
+static std::atomic<unsigned> g_resident_wait_us{20000};   // bound of a workgroup's wait at a tensor's counter
+static std::atomic<unsigned> g_resident_extra_arrivals{0};  // test hook: arrivals expected beyond the grid (never come)
+constexpr u32 kGaveUp = 1u << 16;  // a workgroup that gives up adds this to the tensor's counter
+
 
 constexpr int kResWaves = 12;     // per workgroup
 constexpr int kResRegVecs = 32;
@@ -161,9 +184,10 @@ struct ResidentTable {
     uint2* q[kMaxBatch];
     float* scale[kMaxBatch];
     unsigned nchunks[kMaxBatch];  // 64-vector chunks (the tensor is a whole number of them)
-    u32* amax[kMaxBatch];         // slot 0: arrival counter, slots 1 .. 63: maxima of the workgroups
+    u32* amax[kMaxBatch];         // slot 0: arrival counter, slots 1 .. 62: maxima of the workgroups, slot 63: status
     int n;
     unsigned wait_ticks;  // bound of the wait at the counter, in ticks of the 100 MHz wall clock
+    unsigned arrivals;    // count at which a tensor's meeting is complete: the grid size (a test asks for more)
 };
 
 // atomic max that has been performed when the function returns (the wave waits for the value it returns)
@@ -174,7 +198,7 @@ __device__ __forceinline__ void publish_max(u32* slot, u32 bits) {
 
 __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tensorwise_resident_kernel(const ResidentTable tb) {
     extern __shared__ __attribute__((aligned(16))) uint4 res_lds[];  // [waves][kResLdsVecs][64 lanes], then the give-up flag
-    u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);
+    u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);  // this tensor's verdict
     u32* const red = gave_up + 1;  // [kResWaves]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -255,7 +279,7 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             const u32 w = wave_max(pk_fold(m));
             if (lane == 0) red[wave] = w;
         }
-        // ---- the workgroup's maximum goes to one of the tensor's slots 1 .. 63 with one atomic (thousands of atomics on
+        // ---- the workgroup's maximum goes to one of the tensor's slots 1 .. 62 with one atomic (thousands of atomics on
         // one address serialise at the memory side: one per wave cost 30 us per tensor); slot 0 counts the workgroups
         // that have done so.  A workgroup is counted once its atomic max has been performed (thread 0 has waited for
         // the value it returns); counter and maxima are only ever touched by device-scope atomics, which act at the
@@ -266,25 +290,41 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             u32 w = 0;
 #pragma unroll
             for (int k = 0; k < kResWaves; ++k) w = umax(w, red[k]);
-            if (w) publish_max(tb.amax[t] + 1 + blockIdx.x % (kAmaxSlots - 1), w << 16);  // fp32 bit pattern
+            if (w) publish_max(tb.amax[t] + 1 + blockIdx.x % (kMaxSlots - 1), w << 16);  // fp32 bit pattern
             u32* const counter = tb.amax[t];
-            __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u32 v = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
             const uint64_t since = __builtin_amdgcn_s_memrealtime();
-            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gridDim.x) {
+            // met: a clean counter with every arrival.  Given up: any value with a set high half.
+            while (v < kGaveUp && v < tb.arrivals) {
                 if (__builtin_amdgcn_s_memrealtime() - since > (uint64_t)tb.wait_ticks) {
-                    *gave_up = 1u;
-                    break;
+                    // give up, unless the count completes or somebody else gives up first (v is then re-read)
+                    if (__hip_atomic_compare_exchange_strong(counter, &v, v + kGaveUp, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT))
+                        v += kGaveUp;
+                    continue;
                 }
                 __builtin_amdgcn_s_sleep(2);
+                v = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (v >= kGaveUp) {
+                // the same verdict reaches every workgroup: this tensor and the ones behind it go to the repair kernels
+                *gave_up = 1u;
+                for (int u = t; u < tb.n; ++u)
+                    __hip_atomic_store(tb.amax[u] + kStatusSlot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
         __syncthreads();
+        if (*gave_up != 0u) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS loads still on their way
+            break;
+        }
         // ---- cast what is held and store it; every slot that has been stored is requested anew at once with the next
         // tensor's chunk, so the stores of this tensor and the loads of the next share the memory system.  Behind the
         // last tensor the loads go through a descriptor of no bytes: they fetch nothing.
         static_assert(kAmaxSlots == 64, "one slot per lane");
-        const float amax = __uint_as_float(wave_max(lane ? __hip_atomic_load(tb.amax[t] + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u));
-        const float scale = *gave_up != 0u ? __uint_as_float(kCanonNaN) : scale_from_amax(amax);
+        const float amax = __uint_as_float(
+            wave_max(lane >= 1 && lane < kStatusSlot ? __hip_atomic_load(tb.amax[t] + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u));
+        const float scale = scale_from_amax(amax);
         if (gw == 0 && lane == 0) *tb.scale[t] = scale;
         const Divider d(scale);
         const __amdgpu_buffer_rsrc_t rq = rsrc(tb.q[t]);
@@ -339,6 +379,83 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
         for (int l = 0; l < kResLdsVecs; ++l) m = absmax8(m, my_lds[l * 64]);
     }
+}
+
+// ---------------------------------------------------------------------------
+// The two passes over exactly those tensors of a resident launch whose status word says that the launch gave them
+// up.  Small fixed grids behind every resident launch: a workgroup reads the status words of the launch's tensors
+// with one wave-wide load and leaves at once when none is set, which is the normal case.  Maxima go to slots
+// 1 .. 62 (slot 0 holds the resident kernel's counter; what that kernel's workgroups published there before giving
+// up are maxima of parts of the same tensor and do no harm).
+// ---------------------------------------------------------------------------
+constexpr int kRepairBlocksPerCu = 8;
+
+__device__ __forceinline__ uint64_t repair_mask(const ResidentTable& tb) {  // bit t: tensor t was given up
+    const int lane = threadIdx.x & 63;
+    u32 st = 0;
+    if (lane < tb.n) st = tb.amax[lane][kStatusSlot];
+    return __builtin_amdgcn_ballot_w64(st != 0u);
+}
+
+__global__ __launch_bounds__(256) void tensorwise_repair_amax_kernel(const ResidentTable tb) {
+    __shared__ u32 red[4];
+    uint64_t mask = repair_mask(tb);
+    while (mask) {
+        const int t = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        const int64_t nvec = (int64_t)tb.nchunks[t] * 64;
+        const uint4* const x = tb.x[t];
+        u32 m = 0;
+        for (int64_t base = (int64_t)blockIdx.x * kChunkVecs; base < nvec; base += (int64_t)gridDim.x * kChunkVecs) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t idx = base + threadIdx.x + 256 * i;
+                if (idx < nvec) m = absmax8(m, ld16<true>(x + idx));
+            }
+        }
+        m = wave_max(pk_fold(m));
+        __syncthreads();  // red is free again
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            m = umax(umax(red[0], red[1]), umax(red[2], red[3])) << 16;
+            if (m) atomicMax(tb.amax[t] + 1 + blockIdx.x % (unsigned)(kMaxSlots - 1), m);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void tensorwise_repair_cast_kernel(const ResidentTable tb) {
+    uint64_t mask = repair_mask(tb);
+    while (mask) {
+        const int t = __builtin_ctzll(mask);
+        mask &= mask - 1;
+        const int slot = threadIdx.x & 63;
+        const float amax = __uint_as_float(wave_max(slot >= 1 && slot < kStatusSlot ? tb.amax[t][slot] : 0u));
+        const float scale = scale_from_amax(amax);
+        if (blockIdx.x == 0 && threadIdx.x == 0) *tb.scale[t] = scale;
+        const Divider d(scale);
+        const int64_t nvec = (int64_t)tb.nchunks[t] * 64;
+        const uint4* const x = tb.x[t];
+        uint2* const q = tb.q[t];
+        for (int64_t base = (int64_t)blockIdx.x * kChunkVecs; base < nvec; base += (int64_t)gridDim.x * kChunkVecs) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t idx = base + threadIdx.x + 256 * i;
+                if (idx < nvec) st8<true>(q + idx, cast8(ld16<true>(x + idx), d));
+            }
+        }
+    }
+}
+
+// how many of the n tensors of a workspace carry a set status word
+__global__ __launch_bounds__(256) void tensorwise_status_kernel(const u32* slots, int64_t n, int32_t* out) {
+    __shared__ int red[4];
+    int c = 0;
+    for (int64_t i = threadIdx.x; i < n; i += 256) c += slots[i * kAmaxSlots + kStatusSlot] != 0u;
+    for (int off = 32; off; off >>= 1) c += __shfl_xor(c, off);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) *out = red[0] + red[1] + red[2] + red[3];
 }
 
 enum : int { kPhaseAmax = 1, kPhaseCast = 2 };
@@ -397,7 +514,8 @@ static void two_pass(const cfp8_tensor_desc* descs, int64_t n, u32* slots, int p
             }
             tb.first_block[count] = blocks;
             if (phase == kPhaseAmax) hipLaunchKernelGGL(tensorwise_amax_kernel<true>, dim3(blocks), dim3(256), 0, st, tb);
-            else hipLaunchKernelGGL((tensorwise_cast_kernel<true, true>), dim3(blocks), dim3(256), 0, st, tb);
+            else if (phases == kPhaseCast) hipLaunchKernelGGL((tensorwise_cast_kernel<true, true, true>), dim3(blocks), dim3(256), 0, st, tb);
+            else hipLaunchKernelGGL((tensorwise_cast_kernel<true, true, false>), dim3(blocks), dim3(256), 0, st, tb);
         }
     }
 }
@@ -412,7 +530,7 @@ static int resident_cus() {  // compute units of the current device, 0 if unknow
     }
     int c = cached[dev].load(std::memory_order_relaxed);
     if (c > 0) return c;
-    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0) {
+    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0 || c > 32768) {
         (void)hipGetLastError();
         return 0;
     }
@@ -455,10 +573,14 @@ static void resident_all(const cfp8_tensor_desc* descs, int64_t n, u32* slots, i
         }
         if (count == 0) break;
         tb.n = count;
-        tb.wait_ticks = 100u * 1000u * 1000u;  // one second of the 100 MHz clock
+        tb.wait_ticks = g_resident_wait_us.load(std::memory_order_relaxed) * 100u;  // the wall clock runs at 100 MHz
+        tb.arrivals = (unsigned)cus + g_resident_extra_arrivals.load(std::memory_order_relaxed);
         // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
         // GPU that no other grid holds they are
         hipLaunchKernelGGL(tensorwise_resident_kernel, dim3((unsigned)cus), dim3(kResWaves * 64), kResLdsBytes, st, tb);
+        // tensors that the launch gave up (none, normally) are redone as two ordinary passes
+        hipLaunchKernelGGL(tensorwise_repair_amax_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
+        hipLaunchKernelGGL(tensorwise_repair_cast_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
     }
 }
 
@@ -552,6 +674,28 @@ extern "C" int cfp8_quant_tensorwise_multi_static(const cfp8_tensor_desc* descs,
 extern "C" int cfp8_tensorwise_resident(int enable) {
     if (enable < 0) return cfp8::g_resident_enabled.load(std::memory_order_relaxed);
     return cfp8::g_resident_enabled.exchange(enable ? 1 : 0, std::memory_order_relaxed);
+}
+
+extern "C" int cfp8_tensorwise_resident_tuning(int64_t wait_us, int extra_arrivals) {
+    if (wait_us > 0) cfp8::g_resident_wait_us.store((unsigned)(wait_us < 30000000 ? wait_us : 30000000), std::memory_order_relaxed);
+    if (extra_arrivals >= 0) cfp8::g_resident_extra_arrivals.store((unsigned)(extra_arrivals < 1024 ? extra_arrivals : 1024), std::memory_order_relaxed);
+    return CFP8_OK;
+}
+
+extern "C" int cfp8_tensorwise_status(const float* amax_ws, int64_t n, int32_t* given_up, void* stream) {
+    using namespace cfp8;
+    if (n < 0 || n > (1ll << 24)) return set_error(CFP8_EINVAL, "tensorwise_status: bad tensor count");
+    if (!given_up) return set_error(CFP8_EINVAL, "tensorwise_status: null pointer");
+    if (int rc = check_device()) return rc;
+    const u32* slots = reinterpret_cast<const u32*>(amax_ws);
+    if (!slots) {  // the library's own slots, those of cfp8_quant_tensorwise_multi_static
+        if (n > kStaticMaxTensors) return set_error(CFP8_EINVAL, "tensorwise_status: the library's own slots hold %d tensors", kStaticMaxTensors);
+        u32* own = nullptr;
+        if (int rc = static_slots(&own)) return rc;
+        slots = own;
+    }
+    hipLaunchKernelGGL(tensorwise_status_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream), slots, n, given_up);
+    return check_launch("tensorwise_status");
 }
 
 extern "C" int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n, float* amax_ws, void* stream) {

@@ -101,10 +101,10 @@ int cfp8_quant_rowwise_multi(const cfp8_rowwise_desc* descs, int64_t n, void* st
  * The descriptor array lives in HOST memory; amax_ws is a device array of
  * n * CFP8_TENSORWISE_AMAX_SLOTS floats (scratch, overwritten).
  * numel % 8 == 0 for every tensor.
- * Tensors that fill three quarters or more of the GPU's registers and LDS and still fit (106-141 MB of
- * bf16 on a 256-CU MI355X, numel % 512 == 0: the MLP weights of a 7-8 B model) are read once: one
- * launch of one workgroup per CU keeps them on the chip between the two passes, the workgroups meeting
- * at a counter in amax_ws in between.  That launch wants the GPU to itself - see cfp8_tensorwise_resident.
+ * With the read-once form switched on (cfp8_tensorwise_resident, off by default), tensors that fill three quarters
+ * or more of the GPU's registers and LDS and still fit (106-141 MB of bf16 on a 256-CU MI355X, numel % 512 == 0:
+ * the MLP weights of a 7-8 B model) are read once: one launch of one workgroup per CU keeps them on the chip
+ * between the two passes, the workgroups meeting at a counter in amax_ws in between.
  * The order in which the tensors of a call are quantised is unspecified; the results do not depend on it. */
 #define CFP8_TENSORWISE_AMAX_SLOTS 64
 typedef struct cfp8_tensor_desc {
@@ -117,23 +117,44 @@ typedef struct cfp8_tensor_desc {
 int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
                                 float* amax_ws, void* stream);
 
-/* Switch for the read-once form of cfp8_quant_tensorwise_multi (and _multi_static): enable != 0 allows it
- * (the default), 0 makes every tensor take the two separate passes, a negative value only queries.  Returns
- * the previous setting.  The read-once launch needs all its workgroups on the GPU at the same time, one per
- * CU; two of them issued on different streams of one GPU can each hold part of the CUs and wait for the
- * rest until a one-second bound expires and the affected tensors come out as NaN.  A process that
- * quantises from several streams at once, or that runs with part of the CUs masked off, switches it off.
- * No counterpart in the reference. */
+/* Switch for the read-once form of cfp8_quant_tensorwise_multi (and _multi_static): enable != 0 allows it, 0 (the
+ * default) makes every tensor take the two separate passes, a negative value only queries.  Returns the previous
+ * setting.  The read-once launch needs all its workgroups on the GPU at the same time, one per CU, so it is for a
+ * process that has the GPU to itself while it quantises (the trainer's cast of its weights; not a rollout worker
+ * that quantises on a copy stream beside generation, cosmos_rl/rollout/worker/rollout_control.py:1312-1317).
+ * Where the workgroups cannot all be resident (another stream's or process's kernel holds CUs, two such launches
+ * at once, a CU mask) the meeting of a tensor cannot complete: every workgroup waits at most the bound below, all
+ * of them then leave that tensor and the ones behind it in the launch untouched, and two small kernels that
+ * follow every such launch on the same stream quantise exactly those tensors as two ordinary passes.  The call's
+ * results are therefore the same bits either way; what a failed meeting costs is the wait.  It is recorded: the
+ * last of a tensor's CFP8_TENSORWISE_AMAX_SLOTS slots in amax_ws is its status word, nonzero when the read-once
+ * launch gave the tensor up, until the workspace is next used.  No counterpart in the reference. */
 int cfp8_tensorwise_resident(int enable);
 
+/* *given_up (device int32) = how many of the n tensors of the last call on amax_ws carry a set status word.
+ * amax_ws NULL: the library's own slots, those of cfp8_quant_tensorwise_multi_static.
+ * One small launch on `stream`; nothing is read back by the library.  A caller that finds a nonzero count
+ * after synchronising knows that the read-once form does not have the GPU to itself and switches it off. */
+int cfp8_tensorwise_status(const float* amax_ws, int64_t n, int32_t* given_up, void* stream);
+
+/* Tuning and test hook of the read-once form (process-wide; negative or zero arguments leave a value as it is):
+ * wait_us > 0 sets the bound of a workgroup's wait at a tensor's meeting (default 20000 us); extra_arrivals >= 0
+ * makes every meeting expect that many arrivals more than the grid has workgroups - with 1, no meeting can
+ * complete and every tensor of a read-once launch is given up and repaired, which is how the test suite drives
+ * that path with every wave leaving its kernel normally.  0 restores the real count. */
+int cfp8_tensorwise_resident_tuning(int64_t wait_us, int extra_arrivals);
+
 /* Split-phase forms of the above.  Pass 1 alone leaves partial maxima of |x| of
- * tensor i in amax_ws[i*SLOTS .. i*SLOTS+SLOTS-1] (non-negative fp32 bit
+ * tensor i in amax_ws[i*SLOTS .. i*SLOTS+SLOTS-2] (non-negative fp32 bit
  * patterns, a NaN pattern if the tensor holds one; their maximum as unsigned
- * integers is the tensor's amax); pass 2 alone folds those slots, writes scale and
- * bytes.  Between the two a caller may combine amax_ws across devices with an
- * elementwise all-reduce max over the uint32 view - the tensor-parallel Float8 case of
- * cosmos_rl/policy/model/gpt/parallelize.py:268-280.  q and scale may be null
- * in pass 1. */
+ * integers is the tensor's amax) and zero in the last slot, the status word; pass 2
+ * alone folds those slots, writes scale and bytes.  Between the two a caller may
+ * combine amax_ws across devices with an elementwise all-reduce max over the uint32
+ * view - the tensor-parallel Float8 case of
+ * cosmos_rl/policy/model/gpt/parallelize.py:268-280.  The slots pass 2 finds need not
+ * hold the maximum of the very tensor it casts (another rank's data went into them):
+ * a quotient beyond +-448 saturates to +-448, as the reference's clamp in front of
+ * its cast does.  q and scale may be null in pass 1. */
 int cfp8_tensorwise_amax_multi(const cfp8_tensor_desc* descs, int64_t n,
                                float* amax_ws, void* stream);
 int cfp8_tensorwise_cast_multi(const cfp8_tensor_desc* descs, int64_t n,
@@ -314,6 +335,20 @@ int cfp8_scatter_quant_group128(const void* x, int64_t ld_x, int64_t tokens, int
  * cosmos_rl/policy/model/deepseek_v3/weight_mapper.py:246-259. */
 int cfp8_dequant_block128(const void* q, const float* scales, int64_t rows, int64_t cols,
                           void* y, int out_dtype, void* stream);
+
+/* 1x128 group dequantisation, the inverse of cfp8_quant_group128: y[i, j] = fp8[i, j] * scale[i, j / 128].
+ * q fp8 [rows, cols] (pitch ld_q bytes); y bf16 or fp32 [rows, cols] (pitch ld_y elements, rows 16-byte aligned);
+ * cols % 8 == 0, not necessarily a multiple of 128 (the last group is then short).
+ * scale_kind CFP8_SCALE_F32: scales fp32 [rows, ceil(cols/128)], pitch ld_scales floats.
+ * scale_kind CFP8_SCALE_E8M0: one exponent byte per group, [rows, ceil(cols/128)] with pitch ld_scales bytes, value
+ *   2^(byte - 127) formed as the bit pattern byte << 23 - what viewing the reference's packed int32 scales as uint8
+ *   and shifting gives (four groups per int32, lowest byte first).
+ * Replaces per_token_cast_back of tests/test_deepep.py:86-108 (float scales, and its `x_scales.dtype == torch.int`
+ * branch :97-99); the product is formed in fp32 and rounded once, to nearest even, for bf16. */
+#define CFP8_SCALE_F32 0
+#define CFP8_SCALE_E8M0 1
+int cfp8_dequant_group128(const void* q, int64_t ld_q, const void* scales, int64_t ld_scales, int scale_kind,
+                          int64_t rows, int64_t cols, void* y, int64_t ld_y, int out_dtype, void* stream);
 
 /* Rowwise scaled mm on quantised operands:
  *   out[m, n] = (sum_k a[m,k] b[n,k]) * sa[m] * sb[n]

@@ -235,6 +235,22 @@ def group128_dequant(q_u8: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
     return e4m3_to_f32(q_u8) * se
 
 
+def per_token_cast_back(q_u8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """``per_token_cast_back`` (tests/test_deepep.py:86-108) in full: the columns are padded to a multiple of 128, a
+    scale tensor of dtype int32 holds four E8M0 exponent bytes per element (viewed as uint8 and shifted into the
+    exponent field of an fp32, :97-99), the product is formed in fp32 and cast to bf16."""
+    m, n = q_u8.shape
+    if q_u8.numel() == 0:
+        return torch.empty(m, n, dtype=torch.bfloat16)
+    aligned = (n + BLOCK - 1) // BLOCK * BLOCK
+    x = torch.zeros(m, aligned, dtype=torch.float32)
+    x[:, :n] = e4m3_to_f32(q_u8)
+    if scales.dtype == torch.int32:
+        scales = (scales.contiguous().view(torch.uint8).to(torch.int32) << 23).view(torch.float32)
+    sc = scales.reshape(m, -1, 1)
+    return (x.view(m, -1, BLOCK) * sc).view(m, aligned).to(torch.bfloat16)[:, :n].contiguous()
+
+
 def rowwise_dequant(q_u8: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
     return e4m3_to_f32(q_u8) * s.reshape(-1, 1)
 

@@ -56,6 +56,8 @@ CASES = [
      "gemm_kernel<128,128,2,2,block> grid=288 block=256 lds=73728"),
     ("block, 288 tiles: one round of 256 x 256 tiles and the last 8 tile-columns on 256 x 128 tiles", (BLK, 1024, 18432, 7168),
      f"gemm_block_256 grid=256 block=512 lds={b256_lds(56)}; gemm_block_w8<256,128,block> grid=64 block=512 lds={w8_lds(256, 128, 56)}"),
+    ("block, 600 tokens on a wide weight: below 768 rows nothing is cut off, one launch of 256 x 128 tiles", (BLK, 600, 24576, 1024),
+     "gemm_kernel<256,128,4,2,block> grid=576 block=512 lds=114688"),
     # benchmark config 5 (73600 padded rows)
     ("cfg5 gate_up", (GRP, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
     ("cfg5 gate_up + SwiGLU", (SWI, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped,swiglu> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),

@@ -310,7 +310,8 @@ def test_tensorwise_read_once_launch(dev):
     NaN and an infinity (the scale is then not finite and the bytes take the integer path), through the entry
     point that allocates nothing, and with the launch switched off."""
     lib = _lib.load()
-    assert lib.cfp8_tensorwise_resident(-1) == 1
+    assert lib.cfp8_tensorwise_resident(-1) == 0          # opt-in: off until a caller says the GPU is its own
+    lib.cfp8_tensorwise_resident(1)
     g = torch.Generator(device=dev).manual_seed(77)
     shapes = [(18944, 3584), (512, 3584), (14336, 4096), (3584, 3584), (3584, 18944), (13568, 4096), (17280, 4096)]
     ws = [(torch.randn(sh, generator=g, device=dev) * (0.01 * (i + 1))).to(torch.bfloat16) for i, sh in enumerate(shapes)]
@@ -323,7 +324,8 @@ def test_tensorwise_read_once_launch(dev):
     ws[4][11, 18000] = float("nan")
     ws[5].zero_()                             # amax 0: the scale floor
     ws[6][17279, 4095] = 300.0               # exactly the capacity of 256 CUs; the maximum in the last element of the last chunk
-    qs, scales = ops.quant_tensorwise_multi(ws)
+    qs, scales, given_up = ops.quant_tensorwise_multi(ws, return_status=True)
+    assert int(given_up) == 0                             # every meeting of the read-once launch completed
     q2, s2 = _two_pass(ws, dev)
     for i in range(len(ws)):
         assert torch.equal(u8(qs[i]), u8(q2[i])), f"tensor {i}: bytes differ from the two separate passes"
@@ -346,11 +348,117 @@ def test_tensorwise_read_once_launch(dev):
     assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, outs)) and torch.equal(bits(scales), bits(sc))
     # switched off: every tensor takes the two separate passes; same results
     assert lib.cfp8_tensorwise_resident(0) == 1
-    try:
-        qs_c, scales_c = ops.quant_tensorwise_multi(ws)
-    finally:
-        assert lib.cfp8_tensorwise_resident(1) == 0
+    qs_c, scales_c = ops.quant_tensorwise_multi(ws)
     assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, qs_c)) and torch.equal(bits(scales), bits(scales_c))
+    with ops.gpu_is_mine():
+        assert lib.cfp8_tensorwise_resident(-1) == 1
+    assert lib.cfp8_tensorwise_resident(-1) == 0
+
+
+def test_tensorwise_read_once_launch_gives_up_and_is_repaired(dev):
+    """The read-once launch when its workgroups cannot meet.  Forced from the host: every meeting expects one arrival
+    more than the grid has workgroups and waits 1 ms, so no meeting completes, every workgroup gives the first
+    tensor up and leaves its kernel normally; the repair kernels behind the launch redo the given-up tensors as two
+    ordinary passes.  Results must be the bits of the two-pass path, the status count must name the large tensors,
+    and with the real arrival count restored the same call reports none."""
+    lib = _lib.load()
+    g = torch.Generator(device=dev).manual_seed(78)
+    shapes = [(18944, 3584), (512, 3584), (3584, 18944), (64, 64), (13568, 4096)]
+    ws = [(torch.randn(sh, generator=g, device=dev) * (0.01 * (i + 1))).to(torch.bfloat16) for i, sh in enumerate(shapes)]
+    ws[2][5, 5] = float("nan")
+    want_q, want_s = _two_pass(ws, dev)
+    prev = lib.cfp8_tensorwise_resident(1)
+    try:
+        _lib.check(lib.cfp8_tensorwise_resident_tuning(1000, 1))
+        torch.cuda.synchronize()
+        qs, scales, given_up = ops.quant_tensorwise_multi(ws, return_status=True)
+        torch.cuda.synchronize()
+        assert int(given_up) == 3, f"{int(given_up)} tensors reported as given up, 3 took the read-once launch"
+        assert torch.equal(bits(scales), bits(want_s)), "scales after repair differ from the two passes"
+        for i in range(len(ws)):
+            assert torch.equal(u8(qs[i]), u8(want_q[i])), f"tensor {i}: bytes after repair differ from the two passes"
+        # the library's own slots: same path, status read with a null workspace
+        outs = [torch.empty(w.shape, dtype=torch.float8_e4m3fn, device=dev) for w in ws]
+        sc = torch.empty(len(ws), dtype=torch.float32, device=dev)
+        ops.quant_tensorwise_multi_static(ws, outs, sc)
+        cnt = torch.zeros((), dtype=torch.int32, device=dev)
+        _lib.check(lib.cfp8_tensorwise_status(None, len(ws), cnt.data_ptr(), torch.cuda.current_stream().cuda_stream))
+        assert int(cnt) == 3
+        assert all(torch.equal(u8(a), u8(b)) for a, b in zip(outs, want_q)) and torch.equal(bits(sc), bits(want_s))
+    finally:
+        _lib.check(lib.cfp8_tensorwise_resident_tuning(20000, 0))
+    try:
+        qs, scales, given_up = ops.quant_tensorwise_multi(ws, return_status=True)
+        assert int(given_up) == 0
+        assert torch.equal(bits(scales), bits(want_s)) and all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, want_q))
+    finally:
+        lib.cfp8_tensorwise_resident(prev)
+
+
+def test_tensorwise_split_phase_cast_saturates(dev):
+    """The split-phase cast with slots that hold LESS than the tensor's own maximum (another rank's data, a stale
+    workspace): quotients beyond 448 saturate to +-448 like the reference's clamp, infinities too, NaN stays NaN."""
+    g = torch.Generator().manual_seed(79)
+    x = (torch.randn(300, 1024, generator=g) * 0.02).to(torch.bfloat16)
+    x[0, 0], x[0, 1], x[0, 2], x[0, 3], x[0, 4] = 5.0, -7.0, float("inf"), float("-inf"), float("nan")
+    x[1, 0], x[1, 1] = 3.0e38, -3.0e38
+    xd = x.to(dev)
+    n = 1
+    q = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=dev)
+    sc = torch.empty(n, dtype=torch.float32, device=dev)
+    ws = torch.zeros(n * _lib.TENSORWISE_AMAX_SLOTS, dtype=torch.float32, device=dev)
+    amax = torch.tensor(0.05, dtype=torch.float32)           # smaller than the data's maximum
+    ws[3] = amax
+    d = (_lib.TensorDesc * n)()
+    d[0].x, d[0].q, d[0].scale, d[0].numel = xd.data_ptr(), q.data_ptr(), sc.data_ptr(), xd.numel()
+    _lib.check(_lib.load().cfp8_tensorwise_cast_multi(d, n, ws.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    scale = amax / 448.0
+    assert torch.equal(bits(sc), scale.view(torch.int32).reshape(1))
+    want = O._cast_with_scale(x.float(), scale)
+    assert_bytes(q, want, "saturating split-phase cast")
+    assert [int(v) for v in u8(q)[0, :5]] == [0x7E, 0xFE, 0x7E, 0xFE, 0x7F] and [int(v) for v in u8(q)[1, :2]] == [0x7E, 0xFE]
+
+
+def test_tensorwise_qwen25_7b_full_pass(dev):
+    """The benchmark's headline call itself: all 197 linear weights of a Qwen2.5-7B-shaped decoder (7.07e9 elements) in
+    one cfp8_quant_tensorwise_multi call with the read-once launch allowed, i.e. two resident launches of 48 + 36
+    tensors and the two passes over the other 113.  Every scale against the closed form of torch's amax, and for
+    every tensor four sampled rows of bytes against the oracle's cast with that scale; then the same through the
+    entry point that allocates nothing."""
+    lib = _lib.load()
+    shapes = [((3584, 3584), 28), ((3584, 3584), 28), ((512, 3584), 28), ((512, 3584), 28), ((18944, 3584), 28),
+              ((18944, 3584), 28), ((3584, 18944), 28), ((152064, 3584), 1)]
+    g = torch.Generator(device=dev).manual_seed(1236)
+    tensors = []
+    for k, (sh, mult) in enumerate(shapes):
+        for j in range(mult):
+            t = torch.empty(sh, dtype=torch.bfloat16, device=dev)
+            t.normal_(0.0, 0.02 * (1 + (k + j) % 3), generator=g)   # neighbouring tensors differ in scale
+            tensors.append(t)
+    n = len(tensors)
+    assert n == 197 and sum(t.numel() for t in tensors) == 7_070_285_824
+    amax = torch.stack([t.abs().amax().float() for t in tensors]).cpu()
+    want_scales = O.scale_from_amax(amax)
+
+    def check(outs, scales, what):
+        assert_scales(scales, want_scales, f"{what}: scales")
+        for i, (t, q) in enumerate(zip(tensors, outs)):
+            rows = torch.tensor([0, t.shape[0] // 3, (2 * t.shape[0]) // 3 + 1, t.shape[0] - 1])
+            want = O._cast_with_scale(t[rows.to(dev)].cpu(), want_scales[i])
+            assert_bytes(q.view(torch.uint8)[rows.to(dev)], want, f"{what}: tensor {i} {tuple(t.shape)} rows {rows.tolist()}")
+
+    prev = lib.cfp8_tensorwise_resident(1)
+    try:
+        outs, scales, given_up = ops.quant_tensorwise_multi(tensors, return_status=True)
+        assert int(given_up) == 0
+        check(outs, scales, "workspace entry")
+        for q in outs:
+            q.view(torch.uint8).fill_(0x55)
+        sc = torch.full((n,), -1.0, dtype=torch.float32, device=dev)
+        ops.quant_tensorwise_multi_static(tensors, outs, sc)
+        check(outs, sc, "no-allocation entry")
+    finally:
+        lib.cfp8_tensorwise_resident(prev)
 
 
 def test_tensorwise_full_size_properties(dev):
@@ -452,6 +560,44 @@ def test_group128_deepep_formula(dev, shape):
     qo, so = O.group128_cast_deepep(x)
     assert_scales(s, so, f"deepep {shape} scales")
     assert_bytes(q, qo, f"deepep {shape} bytes")
+
+
+@pytest.mark.parametrize("shape", [(4, 128), (33, 896), (7, 200), (1, 8), (129, 2048), (4096, 7168), (1048700, 8)])
+def test_per_token_cast_back(dev, shape):
+    """per_token_cast_back (tests/test_deepep.py:86-108) with float scales: bit-equal to the oracle in bf16 (NaN
+    bytes compare as NaN), the round trip through the quantiser stays within half an e4m3 step, fp32 output too."""
+    m, n = shape
+    g = torch.Generator().manual_seed(m * 13 + n)
+    q = torch.randint(0, 256, (m, n), generator=g, dtype=torch.uint8)
+    s = torch.rand(m, (n + 127) // 128, generator=g) * 3e-3 + 1e-6
+    want = O.per_token_cast_back(q, s)
+    got = ops.per_token_cast_back(q.to(dev).view(torch.float8_e4m3fn), s.to(dev)).cpu()
+    nan = want.isnan()
+    assert torch.equal(got.isnan(), nan) and torch.equal(got[~nan].view(torch.int16), want[~nan].view(torch.int16))
+    got32 = ops.per_token_cast_back(q.to(dev).view(torch.float8_e4m3fn), s.to(dev), out_dtype=torch.float32).cpu()
+    want32 = O.group128_dequant(q, s)
+    assert torch.equal(got32[~nan], want32[~nan])
+    if m <= 4096:
+        x = O.make_activation(m, n, seed=m + n)
+        qx, sx = ops.per_token_cast_to_fp8(x.to(dev))
+        back = ops.per_token_cast_back(qx, sx).float().cpu()
+        step = sx.cpu().repeat_interleave(128, 1)[:, :n] * 16.0          # half an e4m3 step at the top binade
+        assert bool(((back - x.float()).abs() <= step * 1.01 + x.float().abs() * 2 ** -8).all())
+
+
+def test_per_token_cast_back_packed_e8m0_scales(dev):
+    """The reference's `x_scales.dtype == torch.int` branch: four exponent bytes per int32, lowest byte first."""
+    g = torch.Generator().manual_seed(5)
+    m, n = 37, 1000                                        # eight groups (two int32 per row), the last one 104 columns
+    q = torch.randint(0, 256, (m, n), generator=g, dtype=torch.uint8)
+    e = torch.randint(100, 140, (m, 8), generator=g, dtype=torch.uint8)
+    e[0, 0], e[1, 1], e[2, 2] = 0, 255, 1                    # zero, infinity, the smallest normal scale
+    packed = e.view(torch.int32)
+    want = O.per_token_cast_back(q, packed)
+    got = ops.per_token_cast_back(q.to(dev).view(torch.float8_e4m3fn), packed.to(dev)).cpu()
+    nan = want.isnan()
+    assert torch.equal(got.isnan(), nan) and torch.equal(got[~nan].view(torch.int16), want[~nan].view(torch.int16))
+    assert ops.per_token_cast_back(torch.empty(0, 16, dtype=torch.float8_e4m3fn, device=dev), torch.empty(0, 1, device=dev)).shape == (0, 16)
 
 
 def test_group128_edges(dev):

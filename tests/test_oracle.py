@@ -192,6 +192,56 @@ def test_deepep_formula_matches_in_tree_statement():
     assert bool(((back - x.float()).abs() <= s.repeat_interleave(128, 1)[:, :200] * 16 * 1.01).all())
 
 
+def test_per_token_cast_back_closed_forms():
+    """per_token_cast_back (tests/test_deepep.py:86-108) pinned without retyping it: element by element against
+    python floats (decode table x scale, one rounding to bf16 through struct), the E8M0 bytes against math.ldexp,
+    the byte order of the packed int32 scales against an explicit little-endian pack, a ragged last group, and
+    the empty case."""
+    import math
+    import struct
+    g = torch.Generator().manual_seed(3)
+    m, n = 3, 200                                     # two groups, the second 72 columns wide
+    q = torch.randint(0, 256, (m, n), generator=g, dtype=torch.uint8)
+    q[q == 0x7F] = 0x10
+    q[q == 0xFF] = 0x90                               # no NaN bytes in the closed-form comparison
+    table = [float(v) for v in O.e4m3_to_f32(torch.arange(256, dtype=torch.uint8))]
+
+    def f32(v):                                       # a python float rounded to fp32 (overflow gives infinity)
+        try:
+            return struct.unpack("<f", struct.pack("<f", v))[0]
+        except OverflowError:
+            return math.copysign(math.inf, v)
+
+    def bf16_rne(f):                                  # round an fp32 value to bf16, ties to even, as a python float
+        if math.isinf(f):
+            return f
+        u = struct.unpack("<I", struct.pack("<f", f))[0]
+        u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+        return struct.unpack("<f", struct.pack("<I", u))[0]
+
+    # fp32 scales
+    sc = torch.rand(m, 2, generator=g) * 0.01 + 1e-4
+    got = O.per_token_cast_back(q, sc)
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    for i in range(m):
+        for j in range(0, n, 7):
+            prod = f32(table[int(q[i, j])] * float(sc[i, j // 128]))
+            assert float(got[i, j]) == bf16_rne(prod), (i, j)
+    assert torch.equal(got.float(), O.group128_dequant(q, sc).to(torch.bfloat16).float())
+    # packed E8M0 scales: int32 [m, 1] holds the bytes of groups 0..3, lowest byte first (the reference's view
+    # needs as many scales as groups, so four groups here, the last one 72 columns wide)
+    n = 456
+    q = torch.randint(0, 120, (m, n), generator=g, dtype=torch.uint8)
+    e = torch.tensor([[120, 131, 90, 140], [127, 100, 127, 126], [1, 254, 3, 200]], dtype=torch.uint8)
+    packed = torch.tensor([[int.from_bytes(bytes(row.tolist()), "little", signed=True)] for row in e], dtype=torch.int32)
+    got8 = O.per_token_cast_back(q, packed)
+    for i in range(m):
+        for j in range(0, n, 11):
+            want = bf16_rne(f32(table[int(q[i, j])] * math.ldexp(1.0, int(e[i, j // 128]) - 127)))
+            assert float(got8[i, j]) == want, (i, j)
+    assert O.per_token_cast_back(torch.empty(0, 16, dtype=torch.uint8), torch.empty(0, 1)).shape == (0, 16)
+
+
 def test_nan_and_inf_policy():
     x = torch.zeros(3, 16, dtype=torch.bfloat16)
     x[0, 1] = float("nan"); x[0, 2] = 1.0
