@@ -18,7 +18,11 @@ LIB_DIR = PKG_DIR / "lib"
 LIB_PATH = LIB_DIR / "libcosmosfp8.so"
 OBJ_DIR = CSRC_DIR / "build"
 
-SOURCES = ["api.hip", "quant_rowwise.hip", "quant_tensorwise.hip", "quant_block.hip", "gemm_fp8.hip", "moe_indices.hip", "quant_mxfp4.hip", "gemm_mxfp4.hip"]
+SOURCES = ["api.hip", "quant_rowwise.hip", "quant_tensorwise.hip", "quant_block.hip", "gemm_fp8.hip", "gemm_grouped_xres.hip", "moe_indices.hip",
+           "quant_mxfp4.hip", "gemm_mxfp4.hip"]
+
+# Per-file flags.  gemm_grouped_xres.hip: matrix instructions write ordinary vector registers (see the file's header).
+EXTRA_FLAGS = {"gemm_grouped_xres.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 # -packed-fp32-ops: hipcc must not form v_pk_{add,mul,fma}_f32 (they have returned
 # wrong results on some machines).  -ffp-contract=off: the quantisers rely on
@@ -40,7 +44,7 @@ def hipcc() -> str:
 
 def _compile(src: str) -> Path:
     obj = OBJ_DIR / (src.replace(".hip", ".o"))
-    cmd = [hipcc(), *HIPCC_FLAGS, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", str(CSRC_DIR / src), "-o", str(obj)]
+    cmd = [hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", str(CSRC_DIR / src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

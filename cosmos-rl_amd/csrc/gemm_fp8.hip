@@ -24,33 +24,14 @@
 //             running sum as acc += part * (sa[m, kb] * sb[n / 128, kb]).
 #include <atomic>
 #include <stdio.h>
+#include <stdlib.h>
 #include <type_traits>
 
 #include "cfp8_common.h"
+#include "gemm_internal.h"
 
 namespace cfp8 {
 
-enum : int { kRowwise = 0, kBlock = 1, kGrouped = 2 };
-
-struct GemmArgs {
-    const uint8_t* a;   // activations fp8 [M, K]
-    const uint8_t* b;   // weights fp8 [N, K] (grouped: [E, N, K])
-    const float* sa;    // rowwise [M]; block [M, K/128]
-    const float* sb;    // rowwise [N]; block: see strides
-    const int32_t* m_indices;
-    void* out;
-    int64_t ld_a, ld_b, ld_out;
-    int64_t sb_stride_n, sb_stride_k, sb_stride_e;
-    int M, N, K;
-    int tiles_m, tiles_n;
-    // split-K (rowwise, at most 64 tokens): fp32 partial sums [k_slices, M, N] in caller-provided memory
-    float* partial;
-    size_t partial_bytes;
-    int k_slices, slice_steps;
-    // grouped GEMM with the SwiGLU + 1x128 quantisation epilogue: scales of the quantised product [M, N / 256]
-    float* h_scales;
-    int64_t ld_hs;
-};
 
 __device__ __forceinline__ int lds_chunk_offset(int row, int c) {
     return ((row >> 4) << 11) + (c << 8) + ((((row & 15) ^ ((c & 1) << 3))) << 4);
@@ -440,11 +421,6 @@ __global__ __launch_bounds__(WM * WN * 64) __attribute__((amdgpu_waves_per_eu(2)
 // Requires M % 256 == 0 and N % 256 == 0 (every address is then a per-lane part
 // plus a wave-uniform part).
 // ---------------------------------------------------------------------------
-#define CFP8_PHASE_END() __builtin_amdgcn_sched_barrier(0)
-// Wait until at most `vm` of this wave's loads are outstanding and its LDS reads are done, then the workgroup barrier.
-// Written out as instructions: in front of a barrier it knows of, the compiler waits for every load it has issued,
-// including the direct-to-LDS loads that are meant to stay in flight across the barrier.
-#define CFP8_WAIT_BARRIER(vm) asm volatile("s_waitcnt vmcnt(" #vm ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define CFP8_MMA2(wb, wh, xb, xh, g)                                                                   \
     {                                                                                                  \
         _Pragma("unroll") for (int e = 0; e < 2; ++e) {                                                \
@@ -1719,9 +1695,9 @@ struct LaunchRecord {
     size_t len = 0;
 };
 static thread_local LaunchRecord g_rec;
-static bool dry_run() { return g_rec.dry; }
+bool dry_run() { return g_rec.dry; }
 // returns true when the kernel is to be launched for real
-static bool note_launch(const char* kernel, unsigned grid, unsigned block, size_t lds) {
+bool note_launch(const char* kernel, unsigned grid, unsigned block, size_t lds) {
     if (!g_rec.dry) return true;
     const int n = snprintf(g_rec.text + g_rec.len, sizeof(g_rec.text) - g_rec.len, "%s%s grid=%u block=%u lds=%zu", g_rec.len ? "; " : "",
                            kernel, grid, block, lds);
@@ -1732,21 +1708,21 @@ static int launched(const char* what) { return dry_run() ? CFP8_OK : check_launc
 
 // Kernels that use more than 64 KiB of LDS need the limit raised once per device and function.
 // `flag` is that (device, function) pair's once-flag; a race on the first call raises it twice, harmlessly.
-static int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag) {
+int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag) {
     if (dry_run() || flag.load(std::memory_order_relaxed)) return CFP8_OK;
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return set_error(CFP8_ELAUNCH, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
     flag.store(true, std::memory_order_relaxed);
     return CFP8_OK;
 }
-static int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached) beyond
+int device_slot() {  // 0..63 for the first 64 ordinals, 64 (never cached) beyond
     if (dry_run()) return 64;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) dev = 64;
     return dev >= 0 && dev < 64 ? dev : 64;
 }
 
-static int cu_count() {  // compute units of the current device
+int cu_count() {  // compute units of the current device
     if (dry_run()) return g_rec.cus;
     static std::atomic<int> cached[64];  // zero-initialised
     const int slot = device_slot();
@@ -2492,14 +2468,6 @@ static int launch_cfg(GemmArgs& p, int out_dtype, hipStream_t st) {
 // ---------------------------------------------------------------------------
 constexpr int kPersistentBlockSteps = 32;  // K steps up to which the dispatch sends a problem here (LDS would hold 384)
 
-// One int of a table that no kernel writes, by a scalar load.  Behind the first store of a kernel the compiler turns
-// such a read into a vector load, and then waits for every load in flight, the direct-to-LDS ones included.
-__device__ __forceinline__ int scalar_table_load(const int32_t* table, int index) {
-    const int32_t* const ptr = table + index;  // uniform
-    int v;
-    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ptr) : "memory");
-    return v;
-}
 
 template <int BM, int BN, int MODE, bool OUT_F32, bool SWIGLU = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void gemm_block_w8p_kernel(const GemmArgs p) {
@@ -3005,6 +2973,11 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
     if (MODE == kGrouped) {
         // groups are 128-row aligned, so a tile is 128 rows; 256 columns per workgroup (8 waves) read a
         // quarter fewer operand bytes per flop than 128
+        // 5 or 6 K steps (a down projection) and at least a tile per CU: the kernel that keeps the activation
+        // fragments of a tile row in registers (73472 rows, N = 2048, K = 768: 176 against 241 us on the kernel below)
+        if (p.M % 128 == 0 && p.N % 256 == 0 && (p.K >> 7) >= 5 && (p.K >> 7) <= 6 && p.sb_stride_k == 1 && p.ld_out < (1 << 21) &&
+            (int64_t)(p.M / 128) * (p.N / 256) >= cu_count() && out_dtype_pitch_ok(p, out_dtype) && grouped_xres_pays(p))
+            return launch_grouped_xres(p, out_dtype, st);
         if (p.M % 128 == 0 && p.N % 256 == 0 && (int64_t)(p.M / 128) * (p.N / 256) >= 384 && (p.K >> 7) * 2 <= kMaxTileWeightScales) {
             // 7 to 32 K steps: one workgroup per CU that walks its tiles (73600 rows, N = 2048: K = 896 196 against 215 us,
             // K = 1024 206 against 233 us, K = 1408 271 against 300 us; K = 2048, N = 7168: 1258 against 1360 us; K = 768:

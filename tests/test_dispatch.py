@@ -61,7 +61,10 @@ CASES = [
     # benchmark config 5 (73600 padded rows)
     ("cfg5 gate_up", (GRP, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
     ("cfg5 gate_up + SwiGLU", (SWI, 73600, 1536, 2048), f"gemm_block_w8p<128,256,grouped,swiglu> grid=256 block=512 lds={w8p_lds(128, 256, 16)}"),
-    ("cfg5 down", (GRP, 73600, 2048, 768), f"gemm_block_w8<128,256,grouped> grid=4600 block=512 lds={w8_lds(128, 256, 6)}"),
+    ("cfg5 down", (GRP, 73600, 2048, 768), "gemm_grouped_xres<6> parts=4 grid=256 block=256 lds=151552"),
+    ("down K=640", (GRP, 73600, 2048, 640), "gemm_grouped_xres<5> parts=4 grid=256 block=256 lds=151552"),
+    ("down, few tile rows", (GRP, 9600, 4096, 768), "gemm_grouped_xres<6> parts=3 grid=225 block=256 lds=151552"),
+    ("down, half a round of tile rows", (GRP, 16768, 2048, 768), f"gemm_block_w8<128,256,grouped> grid=1048 block=512 lds={w8_lds(128, 256, 6)}"),
     # the shapes of the walking-kernel parity tests (tests/test_gpu_gemm.py): each must take the walking form
     ("walk rowwise 2304x11520x512", (ROW, 2304, 11520, 512), f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}"),
     ("walk rowwise 8192x7680x896", (ROW, 8192, 7680, 896), f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}"),
@@ -85,6 +88,8 @@ def test_dispatch_limits_of_the_walking_forms():
     """K range of the walking forms and the tile count above which they apply."""
     info = L.gemm_dispatch_info
     assert "w8p" in info(GRP, 73600, 2048, 896) and "w8p" not in info(GRP, 73600, 2048, 768)          # grouped: from 7 K steps
+    assert "xres" in info(GRP, 73600, 2048, 640) and "xres" not in info(GRP, 73600, 2048, 512) and "xres" not in info(GRP, 73600, 2048, 896)
+    assert "xres" not in info(GRP, 73600, 2048 + 128, 768) and "xres" not in info(GRP, 73600, 2048, 768, cus=8 * 4600)   # N % 256; a tile per CU
     assert "w8p" in info(GRP, 73600, 2048, 4096) and "w8p" not in info(GRP, 73600, 2048, 4224)        # ... to 32
     assert "w8p" in info(BLK, 4096, 24576, 384) and "w8p" not in info(BLK, 4096, 24576, 256)          # block: from 3
     assert "256p" in info(ROW, 8192, 18944, 384) and "256p" not in info(ROW, 8192, 18944, 256)        # rowwise: K >= 384

@@ -605,6 +605,44 @@ def test_walking_grouped_kernels_repeatable_and_equal_to_sliced_calls(dev):
         assert torch.equal(outs[0][0].view(torch.uint8)[valid], q0.view(torch.uint8)[valid]) and torch.equal(outs[0][1][valid], s0[valid])
 
 
+def test_grouped_short_k_kernel_equal_to_sliced_calls(dev):
+    """5 or 6 K steps (an expert's down projection): the kernel that keeps a tile row's activation fragments in
+    registers and walks the row's tiles.  Against the same problem cut along N into calls of 256 columns (the
+    one-tile-per-workgroup kernels: same arithmetic, other schedule): same bits, bf16 and fp32, with an expert without
+    tokens, fewer tile rows than CUs (every row cut into pieces) and more (whole rows first, then pieces); the rows of
+    padding keep what the output held; five runs agree."""
+    from cosmos_rl_amd import _lib
+    E = 7
+    for K, N, T, topk in ((768, 4096, 4700, 2), (640, 4096, 4700, 2), (768, 2048, 8300, 4)):
+        qx, sx, mi, valid = _grouped_problem(dev, T, E, K, topk, seed=K + T)
+        rows = qx.shape[0]
+        qw, sw = ops.per_block_cast_to_fp8(O.make_weight((E, N, K), seed=8, std=0.05).to(dev))
+        for dt, code in ((torch.bfloat16, _lib.OUT_BF16), (torch.float32, _lib.OUT_F32)):
+            assert "gemm_grouped_xres" in _lib.gemm_dispatch_info(_lib.DISPATCH_GROUPED, rows, N, K, out_dtype=code), (rows, N, K)
+            assert "gemm_grouped_xres" not in _lib.gemm_dispatch_info(_lib.DISPATCH_GROUPED, rows, 256, K, out_dtype=code)
+            runs = []
+            for _ in range(5):
+                o = torch.full((rows, N), 7.0, dtype=dt, device=dev)
+                ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qw, sw), o, mi)
+                runs.append(o)
+            assert all(torch.equal(runs[0], r) for r in runs[1:]), f"K={K} N={N} {dt}: runs differ"
+            parts = []
+            for n0 in range(0, N, 256):
+                o = torch.full((rows, 256), 7.0, dtype=dt, device=dev)
+                ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qw[:, n0:n0 + 256].contiguous(), sw[:, n0 // 128:n0 // 128 + 2].contiguous()), o, mi)
+                parts.append(o)
+            assert torch.equal(torch.cat(parts, 1), runs[0]), f"K={K} N={N} {dt}: differs from the sliced calls"
+            assert bool((runs[0][~valid] == 7.0).all()) and not bool((runs[0][valid] == 7.0).all(1).any())
+        # an output with a row pitch, through the C entry point: the columns beyond N keep their contents
+        wide = torch.full((rows, N + 64), 3.0, dtype=torch.bfloat16, device=dev)
+        lib = _lib.load()
+        _lib.check(lib.cfp8_gemm_grouped_block128(qx.data_ptr(), K, sx.data_ptr(), qw.data_ptr(), sw.data_ptr(), mi.data_ptr(), wide.data_ptr(), N + 64,
+                                                  _lib.OUT_BF16, rows, N, K, E, torch.cuda.current_stream().cuda_stream))
+        ref = torch.full((rows, N), 3.0, dtype=torch.bfloat16, device=dev)
+        ops.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((qx, sx), (qw, sw), ref, mi)
+        assert torch.equal(wide[:, :N], ref) and bool((wide[:, N:] == 3.0).all())
+
+
 def test_walking_kernels_equal_to_sliced_calls(dev):
     """Rowwise and block-scaled: a problem with more tiles than CUs (the walking kernels) against the same problem cut
     along N into calls that fit one round of workgroups (one tile per workgroup, or the generic kernel): same bits."""
