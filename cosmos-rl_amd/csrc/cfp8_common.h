@@ -296,31 +296,42 @@ __device__ __forceinline__ float silu32_det(float x) {
     return x / (1.0f + exp32_det(-x));
 }
 
-// SiLU for a result that is rounded to bf16 right away.  The defining arithmetic is silu32_det (about 40
-// VALU operations, most of them the IEEE division and the polynomial); what the caller keeps of it is the
-// bf16 rounding, 8 significant bits.  The hardware exponential and reciprocal (v_exp_f32, v_rcp_f32, one ulp
-// each) give x / (1 + exp(-x)) within a few fp32 ulps in a fifth of the instructions, and two floats that
-// close round to the same bf16 unless a rounding boundary of bf16 lies between them, i.e. unless the low 16
-// bits of the fast result are within kSiluTieMargin of 0x8000.  Only then - and for |x| > 16, where the
-// argument of the exponential loses accuracy, infinities and NaN - the defining sequence runs (a wave-level
-// branch, taken for about one wave-wide element slot in sixteen).  That the bf16 result equals the defining one
-// for every one of the 65536 bf16 inputs is checked exhaustively on the GPU by the test suite; measured over all
-// inputs with |x| <= 16 the fast value is within 14 fp32 ulps of the defining one (within 1 for 99 % of them).
-constexpr u32 kSiluTieMargin = 32;
-__device__ __forceinline__ float silu32_for_bf16(float x) {
-    const float e = __builtin_amdgcn_exp2f(x * -1.44269502162933349609375f);
-    float y = x * __builtin_amdgcn_rcpf(1.0f + e);
-    const u32 low = __float_as_uint(y) & 0xFFFFu;
-    const bool near_tie = low - (0x8000u - kSiluTieMargin) <= 2u * kSiluTieMargin;
-    if (near_tie || !(__builtin_fabsf(x) <= 16.0f)) y = silu32_det(x);
-    return y;
+// SiLU for results that are rounded to bf16 right away, four at a time.  The defining arithmetic is silu32_det (about 40
+// VALU operations, most of them the IEEE division and the polynomial); what the caller keeps of it is the bf16
+// rounding, 8 significant bits.  The hardware exponential and reciprocal (v_exp_f32, v_rcp_f32, one ulp each) give
+// x / (1 + exp(-x)) in a fifth of the instructions, within a few fp32 ulps plus the rounding of the exponent
+// t = -x log2(e), which weighs |t| ulps of t: measured over all bf16 inputs with |x| <= 16 the fast value is within
+// 14 fp32 ulps of the defining one, within 1 for 99 % of them.  Two floats that close round to the same bf16 unless
+// a rounding boundary of bf16 lies between them, i.e. unless the low 16 bits of the fast result are within
+// 4 + |t| of 0x8000.  Only then - and for |x| > 16, infinities and NaN - the defining sequence runs: one wave-level
+// test for the four values (the fast sequences of the four interleave, and the rare case lies out of line), then per
+// flagged value.  That the bf16 result equals the defining one for every one of the 65536 bf16 inputs is checked
+// exhaustively on the GPU by the test suite.
+__device__ __forceinline__ void silu32x4_for_bf16(const float (&x)[4], float (&y)[4]) {
+    bool redo[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float t = x[i] * -1.44269502162933349609375f;
+        y[i] = x[i] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
+        const u32 margin = 4u + (u32)__builtin_fabsf(t);  // (the conversion saturates; NaN gives 0)
+        const u32 low = __float_as_uint(y[i]) & 0xFFFFu;
+        redo[i] = low - (0x8000u - margin) <= 2u * margin || !(__builtin_fabsf(x[i]) <= 16.0f);
+    }
+    if (__builtin_expect(redo[0] || redo[1] || redo[2] || redo[3], 0)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (redo[i]) y[i] = silu32_det(x[i]);
+    }
 }
 
-// two packed bf16 gate values and two up values -> two packed bf16 of bf16(bf16(silu(g)) * u)
-__device__ __forceinline__ u32 swiglu_pair(u32 g, u32 u) {
-    const float s0 = silu32_for_bf16(bf16_lo(g)), s1 = silu32_for_bf16(bf16_hi(g));
-    const u32 s = pack_bf16x2(s0, s1);
-    return pack_bf16x2(bf16_lo(s) * bf16_lo(u), bf16_hi(s) * bf16_hi(u));
+// four gate values (two words of two packed bf16) and four up values -> four packed bf16 of bf16(bf16(silu(g)) * u)
+__device__ __forceinline__ void swiglu_quad(u32 g0, u32 g1, u32 u0, u32 u1, u32& h0, u32& h1) {
+    const float x[4] = {bf16_lo(g0), bf16_hi(g0), bf16_lo(g1), bf16_hi(g1)};
+    float y[4];
+    silu32x4_for_bf16(x, y);
+    const u32 s0 = pack_bf16x2(y[0], y[1]), s1 = pack_bf16x2(y[2], y[3]);
+    h0 = pack_bf16x2(bf16_lo(s0) * bf16_lo(u0), bf16_hi(s0) * bf16_hi(u0));
+    h1 = pack_bf16x2(bf16_lo(s1) * bf16_lo(u1), bf16_hi(s1) * bf16_hi(u1));
 }
 
 }  // namespace cfp8

@@ -125,10 +125,10 @@ __global__ __launch_bounds__(256) void gemm_grouped_xres_kernel(const GemmArgs p
     };
 
     // weight tiles: global -> LDS directly, load i of a K step covers rows (wave + 4 i) * 8 .. + 7 of the tile
-    // (row-major stage, 16-byte chunks XOR-ed by (row >> 1) & 7, as in gemm_rowwise_256_kernel)
+    // (row-major stage, 16-byte chunks XOR-ed by f(row), as in gemm_rowwise_256_kernel)
     uint32_t b_step = 32u * (uint32_t)p.ld_b;
     asm volatile("" : "+s"(b_step));
-    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + (lane >> 4))) << 4);
+    const uint32_t chunk = (uint32_t)(((lane & 7) ^ ((wave & 1) * 4 + ((lane >> 4) & 1))) << 4);
     const uint32_t vb_lane = (uint32_t)(lane >> 3) * (uint32_t)p.ld_b + chunk;
     auto w_rsrc = [&](int expert, int n0) {
         const uint64_t bw = reinterpret_cast<uint64_t>(p.b) + ((uint64_t)expert * (uint64_t)p.N + (uint64_t)n0 + (uint64_t)wave * 8) * (uint64_t)p.ld_b;
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void gemm_grouped_xres_kernel(const GemmArgs p
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)(smem + NBASE + ((wave * 2 + par) * 64) * 4), 4,
                                                  (uint32_t)(lane < KT ? lane : KT - 1) * 4u, 0, 0, 0);
     };
-    const int fsw = (lrow >> 1) & 7;
+    const int fsw = ((lrow >> 1) & 1) | (((lrow >> 3) & 1) << 2);
     const int w_off = (wn * 128 + lrow) * 128 + (((2 * quarter) ^ fsw) << 4);
     const int w_off2 = (wn * 128 + lrow) * 128 + (((2 * quarter + 1) ^ fsw) << 4);
     auto frag = [&](int stage, int tile16) {
@@ -483,44 +483,15 @@ __global__ __launch_bounds__(256) void gemm_grouped_xres_kernel(const GemmArgs p
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// The schedule for tiles_m tile rows of tiles_n tiles on `cus` workgroups: one workgroup per CU.  Tile rows beyond the
-// last full round of whole rows (all of them, with fewer tile rows than CUs) are cut along N into `parts` pieces; a
-// unit costs its tiles plus about one tile for loading its fragments, and `parts` is the count with the shortest last
-// round.  `fill` is the share of the run's tile slots (CUs x length of the longest workgroup's run) that hold tiles.
-struct XresPlan {
-    int parts;
-    int64_t blocks;
-    double fill;
-};
-static XresPlan xres_plan(int tiles_m, int tiles_n, int cus) {
-    const int rem = tiles_m >= cus ? tiles_m % cus : tiles_m;
-    int parts = 1;
-    int64_t span = (int64_t)(tiles_m / cus) * (tiles_n + 1);
-    if (rem) {
-        int64_t best = INT64_MAX;
-        for (int q = 1; q <= tiles_n; ++q) {
-            const int64_t rounds = ((int64_t)rem * q + cus - 1) / cus;
-            const int64_t cost = rounds * ((tiles_n + q - 1) / q + 1);
-            if (cost < best) best = cost, parts = q;
-        }
-        span += best;
-    }
-    const int64_t units = (int64_t)(tiles_m - rem) + (int64_t)rem * parts;
-    int64_t blocks = units < cus ? units : cus;
-    // (the kernel takes tiles_m / gridDim.x * gridDim.x tile rows for whole-row units: with fewer tile rows than CUs
-    // the grid must exceed the tile rows unless every unit is a whole row anyway)
-    if (tiles_m < cus && parts == 1) blocks = tiles_m;
-    return {parts, blocks, (double)tiles_m * tiles_n / ((double)cus * (double)span)};
-}
 // Worth it from about 60 % of the tile slots filled (8 experts, 131 tile rows of 8 tiles, 45 % filled: 68 us against
 // 62 us on the one-tile-per-workgroup kernel; 286 tile rows, 81 %: 100 against 124 us).
-bool grouped_xres_pays(const GemmArgs& p) { return xres_plan(p.M / 128, p.N / 256, cu_count()).fill >= 0.6; }
+bool grouped_xres_pays(const GemmArgs& p) { return unit_plan(p.M / 128, p.N / 256, cu_count(), 1).fill >= 0.6; }
 
 template <int KT>
 static int launch_grouped_xres_kt(GemmArgs& p, int out_dtype, hipStream_t st) {
     p.tiles_m = p.M / 128;
     p.tiles_n = p.N / 256;
-    const XresPlan plan = xres_plan(p.tiles_m, p.tiles_n, cu_count());
+    const UnitPlan plan = unit_plan(p.tiles_m, p.tiles_n, cu_count(), 1);
     const int parts = plan.parts;
     const int64_t blocks = plan.blocks;
     p.unit_parts = parts;

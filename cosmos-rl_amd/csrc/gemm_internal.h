@@ -39,6 +39,36 @@ int raise_lds_limit(const void* fn, size_t lds, std::atomic<bool>& flag);       
 int device_slot();                                                                // 0..63, 64 = not cached
 int cu_count();                                                                   // compute units of the current device
 
+// ---- units of the kernels in which a workgroup walks rows of tiles ----------
+// The schedule for tiles_m tile rows of tiles_n tiles on `cus` workgroups: one workgroup per CU.  Tile rows beyond the
+// last full round of whole rows (all of them, with fewer tile rows than CUs) are cut along N into `parts` pieces; a
+// unit costs its tiles plus `unit_cost` tiles for starting it, and `parts` is the count with the shortest last round.  `fill` is the share of the run's tile slots (CUs x length of the longest workgroup's run) that hold tiles.
+struct UnitPlan {
+    int parts;
+    int64_t blocks;
+    double fill;
+};
+inline UnitPlan unit_plan(int tiles_m, int tiles_n, int cus, int unit_cost) {
+    const int rem = tiles_m >= cus ? tiles_m % cus : tiles_m;
+    int parts = 1;
+    int64_t span = (int64_t)(tiles_m / cus) * (tiles_n + unit_cost);
+    if (rem) {
+        int64_t best = INT64_MAX;
+        for (int q = 1; q <= tiles_n; ++q) {
+            const int64_t rounds = ((int64_t)rem * q + cus - 1) / cus;
+            const int64_t cost = rounds * ((tiles_n + q - 1) / q + unit_cost);
+            if (cost < best) best = cost, parts = q;
+        }
+        span += best;
+    }
+    const int64_t units = (int64_t)(tiles_m - rem) + (int64_t)rem * parts;
+    int64_t blocks = units < cus ? units : cus;
+    // (the kernel takes tiles_m / gridDim.x * gridDim.x tile rows for whole-row units: with fewer tile rows than CUs
+    // the grid must exceed the tile rows unless every unit is a whole row anyway)
+    if (tiles_m < cus && parts == 1) blocks = tiles_m;
+    return {parts, blocks, (double)tiles_m * tiles_n / ((double)cus * (double)span)};
+}
+
 // gemm_grouped_xres.hip
 int launch_grouped_xres(GemmArgs& p, int out_dtype, hipStream_t st);
 bool grouped_xres_pays(const GemmArgs& p);  // enough of the CUs' tile slots would hold tiles

@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void dequant_group128_kernel(const uint8_t* __
 
 // SwiGLU fused with the 1x128 quantiser: h = bf16(bf16(silu(g)) * u) is formed in registers from the
 // two bf16 GEMM outputs and quantised like group128_kernel<DIV> does; h never exists in memory.
-// The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors (swiglu_pair).
+// The two roundings to bf16 are those of the unfused torch chain act(g) * u on bf16 tensors (swiglu_quad).
 
 __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __restrict__ gate, int64_t ldg,
                                                               const uint4* __restrict__ up, int64_t ldu, int nvec,
@@ -292,8 +292,9 @@ __global__ __launch_bounds__(256) void swiglu_group128_kernel(const uint4* __res
         if (!ok[i]) vg[i] = vu[i] = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const uint4 h = make_uint4(swiglu_pair(vg[i].x, vu[i].x), swiglu_pair(vg[i].y, vu[i].y),
-                                   swiglu_pair(vg[i].z, vu[i].z), swiglu_pair(vg[i].w, vu[i].w));
+        uint4 h;
+        swiglu_quad(vg[i].x, vg[i].y, vu[i].x, vu[i].y, h.x, h.y);
+        swiglu_quad(vg[i].z, vg[i].w, vu[i].z, vu[i].w, h.z, h.w);
         const u32 m = row16_max(pk_fold(absmax8(0u, h)));
         const float scale = scale_from_amax(amax_from_bits(m));
         const Divider d(scale);
