@@ -141,34 +141,37 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
 // the CU's LDS): a lane keeps kResRegVecs 16-byte vectors in registers and kResLdsVecs in LDS, 256 CUs x 768
 // lanes x 45 x 16 B = 141 MB.  Per tensor every wave loads its 1 KiB chunks (chunk c of the tensor goes to wave
 // c mod waves, so that at any moment the GPU reads one compact window that moves through the tensor),
-// reduces |x|, the workgroup publishes its maximum with one atomic max, the workgroups meet at a counter in
-// device memory, and every wave casts what it holds with the tensor's scale and stores it: 2 B read and 1 B
-// written per element instead of 2 + 2 + 1.  A slot that has been cast and stored is requested anew at once with
-// the next tensor's chunk (register slots by loads into the same registers, LDS slots by direct-to-LDS loads), so
-// one tensor's stores and the next one's loads are in flight together.  Every kept vector has its own registers, hence its own instructions: the code a
-// wave runs per tensor is 30 KB of straight line, shared by the CU's twelve waves and small enough to stay in
-// the instruction cache from one tensor to the next (with one wave per SIMD and all 512 registers it was 350 KB
-// and the kernel spent its time fetching it).
+// reduces |x|, the workgroup publishes its maximum, the workgroups meet (below), and every wave casts what it holds
+// with the tensor's scale and stores it: 2 B read and 1 B written per element instead of 2 + 2 + 1.  A slot that
+// has been cast and stored is requested anew at once with the next tensor's chunk (register slots by loads into
+// the same registers, LDS slots by direct-to-LDS loads), so one tensor's stores and the next one's loads are in
+// flight together.  Every kept vector has its own registers, hence its own instructions: the code a wave runs per
+// tensor is 30 KB of straight line, shared by the CU's twelve waves and small enough to stay in the instruction
+// cache from one tensor to the next (with one wave per SIMD and all 512 registers it was 350 KB and the kernel
+// spent its time fetching it).
+// The meeting.  Every workgroup owns one word per side of a small array in device memory (tensors alternate
+// sides); it writes tag << 16 | its maximum there with one atomic and then reads everybody's words until all carry
+// the tensor's tag - at which point it also holds all the maxima.  While the workgroups meet nothing is in flight,
+// so the meeting is the kernel's fixed cost per tensor; this form takes one trip to memory and one back (a counter
+// took three dependent ones: publish the maximum, count the arrival, read the maxima - about 5 us more per tensor).
 // The launch needs all its workgroups resident at once: the grid is one workgroup per CU and a workgroup takes a
 // whole CU, so on a GPU that no other grid holds they are.  Where they are not (another stream's or process's
-// kernel holds CUs, a second launch of this kind, a CU mask) the meeting cannot complete, so the wait at the
-// counter is bounded by the wall clock and every wave leaves the kernel whatever happens.  The counter makes the
-// outcome of a tensor the same for every workgroup: its low half counts arrivals, its high half counts
-// workgroups that gave up.  A workgroup gives up by a compare-and-swap that adds to the high half of a value it
-// has just read with an incomplete count; from then on no value of the counter is both complete and clean, so no
-// workgroup can take the tensor for met, and before that none could.  A tensor that was given up is left alone by
-// every workgroup (no byte, no scale), its status word (slot kStatusSlot of its amax slots) and those of the
-// tensors behind it in the launch are set, and the kernel ends.  The two repair kernels that follow every
-// resident launch on the same stream redo exactly the tensors whose status word is set as two ordinary passes
-// (a few microseconds when there is none), so the call's results are right either way; the status words stay
-// set in the caller's workspace until its next use and cfp8_tensorwise_status counts them.
+// kernel holds CUs, a second launch of this kind, a CU mask) the meeting cannot complete, so the wait is bounded
+// by the wall clock and every wave leaves the kernel whatever happens.  A workgroup that gives up sets the status
+// word (slot kStatusSlot of a tensor's amax slots) of the tensor it waited for and of every tensor behind it in
+// the launch, marks its words of the meeting array so that the others stop waiting at once, and leaves; so does a
+// workgroup that finds such a mark.  A workgroup may have seen the same meeting complete just before: it stores
+// its part of that tensor with the right scale and gives up at the next meeting.  The two repair kernels that
+// follow every resident launch on the same stream redo exactly the tensors whose status word is set, as two
+// ordinary passes (a few microseconds when there is none), and what they write is what a complete launch writes,
+// so the call's results are right either way; the status words stay set in the caller's workspace until its next
+// use and cfp8_tensorwise_status counts them.
 // The form is opt-in (cfp8_tensorwise_resident): a process switches it on when it has the GPU to itself while it
 // quantises.
 // ---------------------------------------------------------------------------
 static std::atomic<int> g_resident_enabled{0};
 static std::atomic<unsigned> g_resident_wait_us{20000};   // bound of a workgroup's wait at a tensor's counter
 static std::atomic<unsigned> g_resident_extra_arrivals{0};  // test hook: arrivals expected beyond the grid (never come)
-constexpr u32 kGaveUp = 1u << 16;  // a workgroup that gives up adds this to the tensor's counter
 
 
 constexpr int kResWaves = 12;     // per workgroup
@@ -179,27 +182,32 @@ static_assert(kResLdsVecs <= kResRegVecs, "the LDS part passes through registers
 constexpr size_t kResLdsBytes = (size_t)kResWaves * kResLdsVecs * 64 * 16 + 64;
 static_assert(kResLdsBytes <= 160 * 1024, "LDS of one CU");
 
+// The meeting array: a word per workgroup and side (tensors alternate sides), tag << 16 | bf16 bits of the workgroup's
+// maximum; cleared by a kernel in front of every resident launch.  Tags are tensor numbers 1 .. kMaxBatch; kMeetAbort
+// in a word says that its workgroup has given the launch up.
+constexpr int kMeetSlots = 1024;
+constexpr u32 kMeetAbort = 0xFFFF0000u;
+static __device__ __align__(256) u32 g_meet[2][kMeetSlots];
+
+__global__ __launch_bounds__(256) void tensorwise_meet_clear_kernel() {
+    for (int i = threadIdx.x; i < 2 * kMeetSlots; i += 256) (&g_meet[0][0])[i] = 0u;
+}
+
 struct ResidentTable {
     const uint4* x[kMaxBatch];
     uint2* q[kMaxBatch];
     float* scale[kMaxBatch];
     unsigned nchunks[kMaxBatch];  // 64-vector chunks (the tensor is a whole number of them)
-    u32* amax[kMaxBatch];         // slot 0: arrival counter, slots 1 .. 62: maxima of the workgroups, slot 63: status
+    u32* amax[kMaxBatch];         // slots 1 .. 62: maxima (the repair kernels'), slot 63: status
     int n;
-    unsigned wait_ticks;  // bound of the wait at the counter, in ticks of the 100 MHz wall clock
-    unsigned arrivals;    // count at which a tensor's meeting is complete: the grid size (a test asks for more)
+    unsigned wait_ticks;  // bound of the wait at a meeting, in ticks of the 100 MHz wall clock
+    unsigned arrivals;    // words that must carry a tensor's tag: the grid size (a test asks for more, which never come)
 };
-
-// atomic max that has been performed when the function returns (the wave waits for the value it returns)
-__device__ __forceinline__ void publish_max(u32* slot, u32 bits) {
-    const u32 old = __hip_atomic_fetch_max(slot, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("" ::"v"(old));
-}
 
 __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tensorwise_resident_kernel(const ResidentTable tb) {
     extern __shared__ __attribute__((aligned(16))) uint4 res_lds[];  // [waves][kResLdsVecs][64 lanes], then the give-up flag
     u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);  // this tensor's verdict
-    u32* const red = gave_up + 1;  // [kResWaves]
+    u32* const red = gave_up + 1;  // [kResWaves] maxima of the waves, then the tensor's maximum
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const unsigned gw = blockIdx.x * (unsigned)kResWaves + (unsigned)wave;
@@ -279,38 +287,62 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             const u32 w = wave_max(pk_fold(m));
             if (lane == 0) red[wave] = w;
         }
-        // ---- the workgroup's maximum goes to one of the tensor's slots 1 .. 62 with one atomic (thousands of atomics on
-        // one address serialise at the memory side: one per wave cost 30 us per tensor); slot 0 counts the workgroups
-        // that have done so.  A workgroup is counted once its atomic max has been performed (thread 0 has waited for
-        // the value it returns); counter and maxima are only ever touched by device-scope atomics, which act at the
-        // memory side of the XCDs' L2s, so no cache needs writing back or invalidating here (a release or acquire
-        // fence at device scope does both, tens of microseconds each).
+        // ---- the meeting.  The workgroup's maximum goes, tagged with the tensor's number, to the workgroup's own word
+        // of the meeting array (side t & 1) by one atomic whose result nobody waits for; the first wave then reads all
+        // the workgroups' words until every one carries the tag, and has the tensor's maximum in hand when they do:
+        // one trip to memory and one back, where a counter costs three in a row (publish, count, read the maxima).  All
+        // of it by device-scope atomics, which act at the memory side of the XCDs' L2s, so no cache needs writing back or
+        // invalidating (a release or acquire fence at device scope does both, tens of microseconds each).  A word is
+        // reused two tensors later, when every workgroup has long read it: nobody reaches tensor t + 2 before all have
+        // met at t + 1.
         __syncthreads();
-        if (threadIdx.x == 0) {
+        if (wave == 0) {
             u32 w = 0;
 #pragma unroll
             for (int k = 0; k < kResWaves; ++k) w = umax(w, red[k]);
-            if (w) publish_max(tb.amax[t] + 1 + blockIdx.x % (kMaxSlots - 1), w << 16);  // fp32 bit pattern
-            u32* const counter = tb.amax[t];
-            u32 v = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-            const uint64_t since = __builtin_amdgcn_s_memrealtime();
-            // met: a clean counter with every arrival.  Given up: any value with a set high half.
-            while (v < kGaveUp && v < tb.arrivals) {
-                if (__builtin_amdgcn_s_memrealtime() - since > (uint64_t)tb.wait_ticks) {
-                    // give up, unless the count completes or somebody else gives up first (v is then re-read)
-                    if (__hip_atomic_compare_exchange_strong(counter, &v, v + kGaveUp, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                                             __HIP_MEMORY_SCOPE_AGENT))
-                        v += kGaveUp;
-                    continue;
-                }
-                __builtin_amdgcn_s_sleep(2);
-                v = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const u32 tag = (u32)(t + 1) << 16;
+            u32* const side = &g_meet[t & 1][0];
+            if (lane == 0) {
+                const u32 old = __hip_atomic_fetch_max(side + blockIdx.x, tag | w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                (void)old;  // not used: the atomic is sent and forgotten
             }
-            if (v >= kGaveUp) {
-                // the same verdict reaches every workgroup: this tensor and the ones behind it go to the repair kernels
-                *gave_up = 1u;
-                for (int u = t; u < tb.n; ++u)
-                    __hip_atomic_store(tb.amax[u] + kStatusSlot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t since = __builtin_amdgcn_s_memrealtime();
+            bool met = false, lost = false;
+            u32 mx = 0;
+            for (;;) {
+                // words of workgroups that do not exist (a test asks for more arrivals than the grid has) never get a tag
+                bool all = true, any_abort = false;
+                mx = 0;
+                for (unsigned base = 0; base < tb.arrivals; base += 64) {
+                    const unsigned i = base + (unsigned)lane;
+                    const u32 v = i < tb.arrivals ? __hip_atomic_load(side + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
+                    all = all && (v & 0xFFFF0000u) == tag;
+                    any_abort = any_abort || (v & 0xFFFF0000u) == kMeetAbort;
+                    mx = umax(mx, v & 0xFFFFu);
+                }
+                met = __builtin_amdgcn_ballot_w64(!all) == 0;
+                lost = __builtin_amdgcn_ballot_w64(any_abort) != 0;
+                if (met || lost) break;
+                if (__builtin_amdgcn_s_memrealtime() - since > (uint64_t)tb.wait_ticks) {
+                    lost = true;
+                    break;
+                }
+            }
+            if (met && !lost) {
+                mx = wave_max(mx);
+                if (lane == 0) red[kResWaves] = mx;  // (a word of its own: red[0] is written again before every wave has read this)
+            } else {
+                // Given up (by this workgroup's clock or because another workgroup says so): this tensor and the ones
+                // behind it go to the repair kernels, the other workgroups are told through both sides of the meeting
+                // array, and the workgroup leaves.  A workgroup that had already seen this meeting complete goes on to
+                // store its part of the tensor - the same bytes the repair writes - and learns at the next meeting.
+                if (lane == 0) {
+                    *gave_up = 1u;
+                    for (int u = t; u < tb.n; ++u)
+                        __hip_atomic_store(tb.amax[u] + kStatusSlot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_fetch_max(&g_meet[0][blockIdx.x], kMeetAbort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_fetch_max(&g_meet[1][blockIdx.x], kMeetAbort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
         __syncthreads();
@@ -321,9 +353,12 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
         // ---- cast what is held and store it; every slot that has been stored is requested anew at once with the next
         // tensor's chunk, so the stores of this tensor and the loads of the next share the memory system.  Behind the
         // last tensor the loads go through a descriptor of no bytes: they fetch nothing.
-        static_assert(kAmaxSlots == 64, "one slot per lane");
-        const float amax = __uint_as_float(
-            wave_max(lane >= 1 && lane < kStatusSlot ? __hip_atomic_load(tb.amax[t] + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u));
+        // (Nothing is in flight here: the loads of this tensor were awaited before its maximum was formed.  Said with the
+        // builtin, which the compiler takes into account - it cannot see the waits written as instructions, and would
+        // otherwise put a wait for the kept registers' loads in front of every use of one, inside the phase below,
+        // where it would bound the stores and loads in flight.)
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters left alone
+        const float amax = amax_from_bits(red[kResWaves]);
         const float scale = scale_from_amax(amax);
         if (gw == 0 && lane == 0) *tb.scale[t] = scale;
         const Divider d(scale);
@@ -530,7 +565,7 @@ static int resident_cus() {  // compute units of the current device, 0 if unknow
     }
     int c = cached[dev].load(std::memory_order_relaxed);
     if (c > 0) return c;
-    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0 || c > 32768) {
+    if (hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || c <= 0 || c >= kMeetSlots) {
         (void)hipGetLastError();
         return 0;
     }
@@ -575,8 +610,10 @@ static void resident_all(const cfp8_tensor_desc* descs, int64_t n, u32* slots, i
         tb.n = count;
         tb.wait_ticks = g_resident_wait_us.load(std::memory_order_relaxed) * 100u;  // the wall clock runs at 100 MHz
         tb.arrivals = (unsigned)cus + g_resident_extra_arrivals.load(std::memory_order_relaxed);
+        if (tb.arrivals > (unsigned)kMeetSlots) tb.arrivals = (unsigned)kMeetSlots;
         // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
         // GPU that no other grid holds they are
+        hipLaunchKernelGGL(tensorwise_meet_clear_kernel, dim3(1), dim3(256), 0, st);
         hipLaunchKernelGGL(tensorwise_resident_kernel, dim3((unsigned)cus), dim3(kResWaves * 64), kResLdsBytes, st, tb);
         // tensors that the launch gave up (none, normally) are redone as two ordinary passes
         hipLaunchKernelGGL(tensorwise_repair_amax_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);

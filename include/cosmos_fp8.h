@@ -104,7 +104,9 @@ int cfp8_quant_rowwise_multi(const cfp8_rowwise_desc* descs, int64_t n, void* st
  * With the read-once form switched on (cfp8_tensorwise_resident, off by default), tensors that fill three quarters
  * or more of the GPU's registers and LDS and still fit (106-141 MB of bf16 on a 256-CU MI355X, numel % 512 == 0:
  * the MLP weights of a 7-8 B model) are read once: one launch of one workgroup per CU keeps them on the chip
- * between the two passes, the workgroups meeting at a counter in amax_ws in between.
+ * between the two passes; in between the workgroups meet through a small array in device memory that the library
+ * owns (one per GPU, so two read-once launches must not run on one GPU at the same time - which their need for
+ * every CU rules out anyway).
  * The order in which the tensors of a call are quantised is unspecified; the results do not depend on it. */
 #define CFP8_TENSORWISE_AMAX_SLOTS 64
 typedef struct cfp8_tensor_desc {
@@ -123,9 +125,9 @@ int cfp8_quant_tensorwise_multi(const cfp8_tensor_desc* descs, int64_t n,
  * process that has the GPU to itself while it quantises (the trainer's cast of its weights; not a rollout worker
  * that quantises on a copy stream beside generation, cosmos_rl/rollout/worker/rollout_control.py:1312-1317).
  * Where the workgroups cannot all be resident (another stream's or process's kernel holds CUs, two such launches
- * at once, a CU mask) the meeting of a tensor cannot complete: every workgroup waits at most the bound below, all
- * of them then leave that tensor and the ones behind it in the launch untouched, and two small kernels that
- * follow every such launch on the same stream quantise exactly those tensors as two ordinary passes.  The call's
+ * at once, a CU mask) the meeting of a tensor cannot complete: every workgroup waits at most the bound below,
+ * marks that tensor and the ones behind it in the launch and leaves, and two small kernels that follow every such
+ * launch on the same stream quantise exactly the marked tensors as two ordinary passes.  The call's
  * results are therefore the same bits either way; what a failed meeting costs is the wait.  It is recorded: the
  * last of a tensor's CFP8_TENSORWISE_AMAX_SLOTS slots in amax_ws is its status word, nonzero when the read-once
  * launch gave the tensor up, until the workspace is next used.  No counterpart in the reference. */

@@ -338,7 +338,7 @@ def test_tensorwise_read_once_launch(dev):
     assert [int(u8(qs[0])[i, j]) for i, j in ((0, 0), (18943, 3583), (9000, 77))] == [0x7E, 0xFE, 0x7E]
     assert float(ws[0][0, 0].float().cpu() / scales[0].cpu()) > 448.0
     assert int(u8(qs[0])[5, 5]) == 0x80 and int(u8(qs[0])[5, 6]) == 0x00
-    # the counters and maxima live in the workspace of the call: a second call starts from zero again
+    # the meeting words are cleared in front of every launch: a second call starts from zero again
     qs_b, scales_b = ops.quant_tensorwise_multi(ws)
     assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, qs_b)) and torch.equal(bits(scales), bits(scales_b))
     # the library's own slots
