@@ -310,15 +310,24 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             bool met = false, lost = false;
             u32 mx = 0;
             for (;;) {
-                // words of workgroups that do not exist (a test asks for more arrivals than the grid has) never get a tag
+                // (words of workgroups that do not exist - a test asks for more arrivals than the grid has - never get a tag)
                 bool all = true, any_abort = false;
                 mx = 0;
-                for (unsigned base = 0; base < tb.arrivals; base += 64) {
-                    const unsigned i = base + (unsigned)lane;
-                    const u32 v = i < tb.arrivals ? __hip_atomic_load(side + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
-                    all = all && (v & 0xFFFF0000u) == tag;
-                    any_abort = any_abort || (v & 0xFFFF0000u) == kMeetAbort;
-                    mx = umax(mx, v & 0xFFFFu);
+                // (256 words per round of four loads that are in flight together: one trip for a GPU of 256 CUs; an
+                // index past the last word reads the last word once more)
+                for (unsigned base = 0; base < tb.arrivals; base += 256) {
+                    u32 v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const unsigned i = base + (unsigned)(k * 64 + lane);
+                        v[k] = __hip_atomic_load(side + (i < tb.arrivals ? i : tb.arrivals - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        all = all && (v[k] & 0xFFFF0000u) == tag;
+                        any_abort = any_abort || (v[k] & 0xFFFF0000u) == kMeetAbort;
+                        mx = umax(mx, v[k] & 0xFFFFu);
+                    }
                 }
                 met = __builtin_amdgcn_ballot_w64(!all) == 0;
                 lost = __builtin_amdgcn_ballot_w64(any_abort) != 0;
