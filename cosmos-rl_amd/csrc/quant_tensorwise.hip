@@ -414,14 +414,18 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the empty loads still write LDS: none is in flight when the wave ends)
             break;
         }
-        // ---- the next tensor's maximum, slot by slot as the loads land (they return in order); the LDS slots were
-        // requested first, so they are complete once the last register slot is
+        // ---- the next tensor's maximum, slot by slot as the loads land (they return in order).  The LDS slots were
+        // requested first: of the 2 x kResVecs stores and loads of the phase at most 63 are still in flight behind the
+        // wait below, so the 2 x kResLdsVecs oldest - the LDS slots' - are done, and their part of the maximum is formed
+        // while the register slots' loads are still landing (read by instructions written out, see lds_slot)
+        static_assert(2 * kResVecs - 63 >= 2 * kResLdsVecs, "a wait for all but 63 operations covers the LDS slots");
         m = 0;
+        asm volatile("s_waitcnt vmcnt(63)" ::: "memory");
+#pragma unroll
+        for (int l = 0; l < kResLdsVecs; ++l) m = absmax8(m, lds_slot(l));
 #pragma unroll
         for (int r = 0; r < kResRegVecs; ++r) m = absmax8(m, keep[r]);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-        for (int l = 0; l < kResLdsVecs; ++l) m = absmax8(m, my_lds[l * 64]);
     }
 }
 
