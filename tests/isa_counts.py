@@ -1,7 +1,7 @@
 """Instruction census of the GEMM kernels with hand-counted waits, from hipcc's own assembly listing of
-csrc/gemm_fp8.hip and csrc/gemm_mxfp4.hip.
+csrc/gemm_fp8.hip, csrc/gemm_grouped_xres.hip and csrc/gemm_mxfp4.hip.
 
-gemm_rowwise_256p_kernel, gemm_block_w8p_kernel, the strip kernels and the direct-to-LDS kernels of gemm_mxfp4.hip order their
+gemm_rowwise_256p_kernel, gemm_block_w8p_kernel, gemm_grouped_xres_kernel, the strip kernels and the direct-to-LDS kernels of gemm_mxfp4.hip order their
 LDS traffic with hand-written
 ``s_waitcnt vmcnt(N)`` + ``s_barrier`` pairs: N is the number of vector-memory operations the author
 counted between the loads a barrier needs and the barrier.  That is right only while the compiler
@@ -25,8 +25,9 @@ sys.path.insert(0, str(ROOT / "cosmos-rl_amd"))
 from cosmos_rl_amd import _build  # noqa: E402
 
 WALKING = ("gemm_rowwise_256p_kernel", "gemm_block_w8p_kernel", "gemm_mxfp4_256_kernel", "gemm_mxfp4_128_kernel",
-           "gemm_mxfp4_128x512_kernel", "gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel", "gemm_block_256_kernel")
-SOURCES = ("gemm_fp8.hip", "gemm_mxfp4.hip")
+           "gemm_mxfp4_128x512_kernel", "gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel", "gemm_block_256_kernel",
+           "gemm_grouped_xres_kernel")
+SOURCES = ("gemm_fp8.hip", "gemm_grouped_xres.hip", "gemm_mxfp4.hip")
 _VMEM = re.compile(r"^\s+((?:buffer|global|flat|scratch)_(?:load|store|atomic)\w*)\b(.*)")
 _PAIR = re.compile(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)")
 
@@ -37,8 +38,8 @@ def assembly() -> list[str]:
     with tempfile.TemporaryDirectory() as tmp:
         for src in SOURCES:
             out = Path(tmp) / (src + ".s")
-            cmd = [_build.hipcc(), *_build.HIPCC_FLAGS, f"-I{_build.INCLUDE_DIR}", f"-I{_build.CSRC_DIR}", "--cuda-device-only", "-S",
-                   str(_build.CSRC_DIR / src), "-o", str(out)]
+            cmd = [_build.hipcc(), *_build.HIPCC_FLAGS, *_build.EXTRA_FLAGS.get(src, []), f"-I{_build.INCLUDE_DIR}", f"-I{_build.CSRC_DIR}",
+                   "--cuda-device-only", "-S", str(_build.CSRC_DIR / src), "-o", str(out)]
             res = subprocess.run(cmd, capture_output=True, text=True)
             if res.returncode != 0:
                 raise RuntimeError(f"hipcc -S failed:\n{res.stderr}")

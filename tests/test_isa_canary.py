@@ -51,6 +51,24 @@ def test_no_scratch_and_counts_add_up(census):
             assert ops["buffer_load_dword lds"] == 3 * sc + copies * sc and ops["global_load_lds_dword"] == 1, (name, ops)
             assert rec["mfma"] == copies * mfma_per_step, (name, rec)
             continue
+        if m.group(1) == "gemm_grouped_xres_kernel":
+            # <K steps, fp32 output>: one barrier in the middle of every K step; the weight loads of a step (8 per wave) are
+            # requested three steps ahead, the prologue requests three steps.  bf16: a tile leaves as 16 stores spread over
+            # steps 1 .. 4 of the next tile (4 each, in the half in front of the barrier), so a barrier may leave the 8
+            # loads of the step in between and the stores of that step and of its own in flight; fp32: 32 stores in front
+            # of the first barrier of the next tile.  The last tile's stores are issued once more behind the loop.
+            kt, f32 = args
+            stores_per_tile = 32 if f32 else 16
+            assert ops["buffer_load_dwordx4 lds"] == 3 * 8 + kt * 8, (name, ops)
+            assert ops["buffer_store_dwordx4"] == 2 * stores_per_tile, (name, ops)
+            stores_at = lambda k: 4 if 1 <= k % kt <= 4 else 0   # (python's % wraps a negative step into the tile before)
+            want = [40, 40] + [8] * (kt - 2) if f32 else [8 + stores_at(k - 1) + stores_at(k) for k in range(kt)]
+            assert rec["hand_written_vmcnt_before_barrier"] == sorted(want), (name, rec)
+            # a unit's activation fragments (two 16-byte loads each) and scales, at the kernel's start and at a unit switch
+            assert ops["buffer_load_dwordx4"] == 2 * kt * 4 * 2 and ops["buffer_load_dword"] == 2 * kt * 4, (name, ops)
+            assert rec["mfma"] == kt * 32, (name, rec)
+            assert not any(k.startswith("scratch_") for k in ops), f"{name} spills: {ops}"
+            continue
         if m.group(1) in ("gemm_rowwise_strip_kernel", "gemm_mxfp4_strip_kernel"):
             # a ring of S stages: the prologue requests S - 1 tiles, every step one more; the barrier of a step lets the
             # loads of the S - 2 tiles behind the one it needs pass
