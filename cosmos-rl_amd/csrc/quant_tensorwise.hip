@@ -183,8 +183,11 @@ constexpr size_t kResLdsBytes = (size_t)kResWaves * kResLdsVecs * 64 * 16 + 64;
 static_assert(kResLdsBytes <= 160 * 1024, "LDS of one CU");
 
 // The meeting array: a word per workgroup and side (tensors alternate sides), tag << 16 | bf16 bits of the workgroup's
-// maximum; cleared by a kernel in front of every resident launch.  Tags are tensor numbers 1 .. kMaxBatch; kMeetAbort
-// in a word says that its workgroup has given the launch up.
+// maximum; cleared by a kernel in front of every resident launch.  A tag is the launch's number (10 bits, never all
+// ones) and the tensor's number 1 .. kMaxBatch (6 bits); kMeetAbort in a word says that its workgroup has given the
+// launch up.  Two such launches at once on one GPU cannot both have every CU and disturb each other's words; because
+// their tags differ, neither can take a foreign word for an arrival: they run into the bound of the wait, and the
+// repair kernels do the work.
 constexpr int kMeetSlots = 1024;
 constexpr u32 kMeetAbort = 0xFFFF0000u;
 static __device__ __align__(256) u32 g_meet[2][kMeetSlots];
@@ -202,6 +205,7 @@ struct ResidentTable {
     int n;
     unsigned wait_ticks;  // bound of the wait at a meeting, in ticks of the 100 MHz wall clock
     unsigned arrivals;    // words that must carry a tensor's tag: the grid size (a test asks for more, which never come)
+    unsigned launch_tag;  // (launch number mod 1023) << 6: two launches that overlap on one GPU never take each other's words for theirs
 };
 
 __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tensorwise_resident_kernel(const ResidentTable tb) {
@@ -300,7 +304,7 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             u32 w = 0;
 #pragma unroll
             for (int k = 0; k < kResWaves; ++k) w = umax(w, red[k]);
-            const u32 tag = (u32)(t + 1) << 16;
+            const u32 tag = (tb.launch_tag | (u32)(t + 1)) << 16;  // this launch's number, then the tensor's
             u32* const side = &g_meet[t & 1][0];
             if (lane == 0) {
                 const u32 old = __hip_atomic_fetch_max(side + blockIdx.x, tag | w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -624,6 +628,9 @@ static void resident_all(const cfp8_tensor_desc* descs, int64_t n, u32* slots, i
         tb.wait_ticks = g_resident_wait_us.load(std::memory_order_relaxed) * 100u;  // the wall clock runs at 100 MHz
         tb.arrivals = (unsigned)cus + g_resident_extra_arrivals.load(std::memory_order_relaxed);
         if (tb.arrivals > (unsigned)kMeetSlots) tb.arrivals = (unsigned)kMeetSlots;
+        static std::atomic<unsigned> launches{0};
+        tb.launch_tag = (launches.fetch_add(1, std::memory_order_relaxed) % 1023u) << 6;
+        static_assert(kMaxBatch < 64, "a tensor's number fits six bits");
         // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
         // GPU that no other grid holds they are
         hipLaunchKernelGGL(tensorwise_meet_clear_kernel, dim3(1), dim3(256), 0, st);

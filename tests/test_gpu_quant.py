@@ -395,6 +395,36 @@ def test_tensorwise_read_once_launch_gives_up_and_is_repaired(dev):
         lib.cfp8_tensorwise_resident(prev)
 
 
+def test_tensorwise_read_once_launches_on_two_streams(dev):
+    """Two read-once calls at the same time on two streams of one process - what the entry point's contract rules out.
+    Each launch needs every CU, so they cannot both be resident, and they share the array through which workgroups
+    meet; the launch number in every meeting tag keeps either from taking the other's words for arrivals.  Whatever
+    the hardware makes of the overlap (one launch after the other, or meetings that run into the bound of the wait
+    and are repaired), both calls must return the bits of the two-pass path."""
+    lib = _lib.load()
+    g = torch.Generator(device=dev).manual_seed(80)
+    sets = [[(torch.randn(18944, 3584, generator=g, device=dev) * (0.01 * (i + 1 + 3 * k))).to(torch.bfloat16) for i in range(3)] for k in range(2)]
+    wants = [_two_pass(ws, dev) for ws in sets]
+    prev = lib.cfp8_tensorwise_resident(1)
+    try:
+        _lib.check(lib.cfp8_tensorwise_resident_tuning(3000, 0))
+        streams = [torch.cuda.Stream(device=dev) for _ in range(2)]
+        torch.cuda.synchronize()
+        got = [None, None]
+        for _ in range(3):
+            for k in range(2):
+                with torch.cuda.stream(streams[k]):
+                    got[k] = ops.quant_tensorwise_multi(sets[k])
+            torch.cuda.synchronize()
+            for k in range(2):
+                qs, scales = got[k]
+                assert torch.equal(bits(scales), bits(wants[k][1])), f"stream {k}: scales differ from the two passes"
+                assert all(torch.equal(u8(a), u8(b)) for a, b in zip(qs, wants[k][0])), f"stream {k}: bytes differ from the two passes"
+    finally:
+        _lib.check(lib.cfp8_tensorwise_resident_tuning(20000, 0))
+        lib.cfp8_tensorwise_resident(prev)
+
+
 def test_tensorwise_split_phase_cast_saturates(dev):
     """The split-phase cast with slots that hold LESS than the tensor's own maximum (another rank's data, a stale
     workspace): quotients beyond 448 saturate to +-448 like the reference's clamp, infinities too, NaN stays NaN."""
