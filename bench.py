@@ -9,7 +9,8 @@ already resident in HBM).  One step = one `cfp8_quant_tensorwise_multi` call ove
 `value` = algorithmic bytes of the two-pass algorithm (5 B/element: 2 read by the amax pass,
 2 read + 1 written by the cast pass) per second over the timed steps.  The bench owns the GPU and says so to the
 library (`cfp8_tensorwise_resident(1)`), so the 84 MLP weights (136 MB each, 81 % of the elements) take the launch
-that keeps a tensor on the chip between the passes and move 3 B/element through HBM; `value` keeps the 5 B/element
+that keeps a tensor on the chip between the passes and move 3 B/element through HBM (the 56 q / o projections too, five
+at a time: `roofline.grouped_tensors`); `value` keeps the 5 B/element
 accounting of the metric, `config.single_read_lower_bound_GBps` is the same time on 3.
 `roofline` is for the dominant kernel, that launch, on the bytes it moves: `achieved` = 3 B/element x the elements of a
 launch / its event-timed duration, `frac` = that over 8 TB/s; the same time on the metric's 5 B/element is
@@ -134,9 +135,11 @@ def main() -> int:
     headline_verified = True
 
     # ---- per-kernel timing with events on the launch stream ------------------------------
-    # The call above runs two kinds of launches: the 84 MLP weights (136 MB each) take the kernel that keeps a tensor
-    # on the chip between the passes (48 + 36 tensors = 2 launches), the other 113 tensors take pass 1 and pass 2 as
-    # launches of their own (3 batches of at most 48).  Each kind is timed here as a call on its own tensors.
+    # The call above runs three kinds of launches: the 84 MLP weights (136 MB each) take the kernel that keeps a tensor
+    # on the chip between the passes (48 + 36 tensors = 2 launches); the 56 q / o projections (26 MB each) take the same
+    # kernel five at a time, each on a fifth of the CUs (48 + 8 tensors = 2 launches); the other 57 tensors (k, v,
+    # lm_head) take pass 1 and pass 2 as launches of their own (2 batches of at most 48).  Each kind is timed here as a
+    # call on its own tensors.
     def time_phase(fn, reps):
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for a, b in evs:
@@ -157,18 +160,34 @@ def main() -> int:
         return (count + 47) // 48
 
     reps = max(3, args.steps)
-    cap_elems = cus * 12 * 45 * 512          # what the CUs hold; the library takes tensors of 3/4 of that and more
-    big = lambda t: t.numel() % 512 == 0 and cap_elems * 3 // 4 <= t.numel() <= cap_elems
-    d_big, n_big, numel_big = sub_table(big)
-    d_rest, n_rest, numel_rest = sub_table(lambda t: not big(t))
-    assert n_big == 84 and n_rest == 113
+
+    def resident_groups(t):
+        """How many tensors like t the library keeps on the chip at the same time (0: t takes the two passes): the
+        rule of quant_tensorwise.hip - the largest count up to 8 whose share of the CUs (12 waves x 45 chunks of
+        512 elements per CU) still holds the tensor, provided the tensor fills three quarters of that share."""
+        if t.numel() % 512:
+            return 0
+        chunks = t.numel() // 512
+        for g in range(8, 0, -1):
+            cap = (cus // g) * 12 * 45
+            if cap and chunks <= cap:
+                return g if chunks * 4 >= cap * 3 else 0
+        return 0
+
+    d_big, n_big, numel_big = sub_table(lambda t: resident_groups(t) == 1)
+    d_mid, n_mid, numel_mid = sub_table(lambda t: resident_groups(t) > 1)
+    d_rest, n_rest, numel_rest = sub_table(lambda t: resident_groups(t) == 0)
+    assert (n_big, n_mid, n_rest) == (84, 56, 57), (n_big, n_mid, n_rest)
     res_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_big, n_big, amax_ws.data_ptr(), stream)), reps)
+    mid_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_mid, n_mid, amax_ws.data_ptr(), stream)), reps)
     amax_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_amax_multi(d_rest, n_rest, amax_ws.data_ptr(), stream)), reps)
     cast_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_cast_multi(d_rest, n_rest, amax_ws.data_ptr(), stream)), reps)
     # the same 84 tensors as two separate passes, for comparison
     lib.cfp8_tensorwise_resident(0)
     two_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_big, n_big, amax_ws.data_ptr(), stream)), reps)
+    mid_two_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_mid, n_mid, amax_ws.data_ptr(), stream)), reps)
     lib.cfp8_tensorwise_resident(1)
+    mid_med, mid_two_med = statistics.median(mid_ms), statistics.median(mid_two_ms)
     res_med, amax_med, cast_med, two_med = (statistics.median(x) for x in (res_ms, amax_ms, cast_ms, two_ms))
     res_launches = launches_of(n_big)
     rest_launches = launches_of(n_rest)
@@ -199,6 +218,13 @@ def main() -> int:
         "note": "avg_launch_ms is the call on the 84 tensors (two read-once launches, the fill kernel in front and the two "
                 "repair launches behind each, which find nothing to do) / 2",
         "same_tensors_as_two_passes_ms": round(two_med, 4),
+        "grouped_tensors": {
+            "what": "the 56 q / o projections (12.8 M elements each): five of them on the chip at a time, each held by a fifth "
+                    "of the CUs, in the same kernel",
+            "tensors": n_mid, "launches_per_step": launches_of(n_mid), "ms": round(mid_med, 4),
+            "achieved": round(3 * numel_mid / (mid_med * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "frac": round(3 * numel_mid / (mid_med * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "same_tensors_as_two_passes_ms": round(mid_two_med, 4)},
         "other_tensors": {
             "tensors": n_rest, "launches_per_pass": rest_launches,
             "cast_kernel": {"kernel": "tensorwise_cast_kernel", "achieved": round(3 * numel_rest / (cast_med * 1e-3) / 1e9, 1), "unit": "GB/s",

@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
 
 // ---------------------------------------------------------------------------
 // Both passes in one launch, with the tensor kept on the chip in between (tensors of 106-141 MB: the MLP
-// weights of a 7-8 B model).  One workgroup of twelve waves per CU (three per SIMD, 168 registers each, all of
+// weights of a 7-8 B model; smaller ones several at a time, each held by a group of the CUs, see `groups` below).  One workgroup of twelve waves per CU (three per SIMD, 168 registers each, all of
 // the CU's LDS): a lane keeps kResRegVecs 16-byte vectors in registers and kResLdsVecs in LDS, 256 CUs x 768
 // lanes x 45 x 16 B = 141 MB.  Per tensor every wave loads its 1 KiB chunks (chunk c of the tensor goes to wave
 // c mod waves, so that at any moment the GPU reads one compact window that moves through the tensor),
@@ -204,7 +204,9 @@ struct ResidentTable {
     u32* amax[kMaxBatch];         // slots 1 .. 62: maxima (the repair kernels'), slot 63: status
     int n;
     unsigned wait_ticks;  // bound of the wait at a meeting, in ticks of the 100 MHz wall clock
-    unsigned arrivals;    // words that must carry a tensor's tag: the grid size (a test asks for more, which never come)
+    int groups;           // tensors held at the same time, each by group_wgs workgroups
+    unsigned group_wgs;
+    unsigned arrivals;    // words that must carry a tensor's tag: a group's size (a test asks for more, which never come)
     unsigned launch_tag;  // (launch number mod 1023) << 6: two launches that overlap on one GPU never take each other's words for theirs
 };
 
@@ -214,11 +216,18 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
     u32* const red = gave_up + 1;  // [kResWaves] maxima of the waves, then the tensor's maximum
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const unsigned gw = blockIdx.x * (unsigned)kResWaves + (unsigned)wave;
-    const unsigned nw = gridDim.x * (unsigned)kResWaves;
+    // Groups: the launch's workgroups are cut into tb.groups equal groups, each of which holds one tensor at a time
+    // (tensor r * groups + grp in round r) and meets only within itself: a tensor a fifth the size of the chip's
+    // registers and LDS is held by a fifth of the CUs while the other four fifths hold four more.  Workgroups beyond
+    // the last group have nothing to do.
+    const unsigned grp = blockIdx.x / tb.group_wgs;
+    if (grp >= (unsigned)tb.groups || (int)grp >= tb.n) return;  // (uniform; no barrier has been reached)
+    const unsigned first_wg = grp * tb.group_wgs;  // the group's first workgroup = its first word of the meeting array
+    const unsigned gw = (blockIdx.x - first_wg) * (unsigned)kResWaves + (unsigned)wave;  // the wave's number in its group
+    const unsigned nw = tb.group_wgs * (unsigned)kResWaves;
     uint4* const my_lds = res_lds + wave * (kResLdsVecs * 64) + lane;
     if (threadIdx.x == 0) *gave_up = 0u;
-    // Chunk i of the wave is chunk gw + i * nw of the tensor: at any moment the waves of the whole GPU read one compact
+    // Chunk i of the wave is chunk gw + i * nw of the tensor: at any moment the waves of a group read one compact
     // window that moves through the tensor, as a streaming kernel's workgroups do.  Every wave issues the same loads
     // and stores whatever its share: slots past its last chunk repeat that chunk (a wave without any repeats a chunk
     // of another wave), which changes neither the maximum nor a stored byte - branches around the loads would make
@@ -262,13 +271,13 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(wave_lds + l * 1024), 16, g.lane_vec * 16u, slot_vec(g, l) * 16u, 0, 2);
     };
     uint4 keep[kResRegVecs];
-    Geo g = geo(0);
+    Geo g = geo((int)grp);
     u32 m = 0;
     // ---- the first tensor's loads: kResDepth in flight per wave, issued in chunk order, straight into the registers
     // that keep them
     {
         constexpr int kResDepth = 8;
-        const __amdgpu_buffer_rsrc_t rx = rsrc(tb.x[0]);
+        const __amdgpu_buffer_rsrc_t rx = rsrc(tb.x[grp]);
 #pragma unroll
         for (int l = 0; l < kResDepth; ++l) keep[l] = load(rx, g, l);
 #pragma unroll
@@ -285,7 +294,7 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             if (r + kResDepth < kResRegVecs) keep[r + kResDepth] = load(rx, g, kResLdsVecs + r + kResDepth);
         }
     }
-    for (int t = 0; t < tb.n; ++t) {
+    for (int t = (int)grp, round = 0; t < tb.n; t += tb.groups, ++round) {
         // here the wave holds tensor t and m is the lane's maximum of it
         {
             const u32 w = wave_max(pk_fold(m));
@@ -305,9 +314,9 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
             for (int k = 0; k < kResWaves; ++k) w = umax(w, red[k]);
             const u32 tag = (tb.launch_tag | (u32)(t + 1)) << 16;  // this launch's number, then the tensor's
-            u32* const side = &g_meet[t & 1][0];
+            u32* const side = &g_meet[round & 1][first_wg];  // the group's words
             if (lane == 0) {
-                const u32 old = __hip_atomic_fetch_max(side + blockIdx.x, tag | w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const u32 old = __hip_atomic_fetch_max(side + (blockIdx.x - first_wg), tag | w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 (void)old;  // not used: the atomic is sent and forgotten
             }
             const uint64_t since = __builtin_amdgcn_s_memrealtime();
@@ -351,7 +360,7 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
                 // store its part of the tensor - the same bytes the repair writes - and learns at the next meeting.
                 if (lane == 0) {
                     *gave_up = 1u;
-                    for (int u = t; u < tb.n; ++u)
+                    for (int u = t - (int)grp; u < tb.n; ++u)  // from the first tensor of this round on
                         __hip_atomic_store(tb.amax[u] + kStatusSlot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_fetch_max(&g_meet[0][blockIdx.x], kMeetAbort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     __hip_atomic_fetch_max(&g_meet[1][blockIdx.x], kMeetAbort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -376,10 +385,10 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
         if (gw == 0 && lane == 0) *tb.scale[t] = scale;
         const Divider d(scale);
         const __amdgpu_buffer_rsrc_t rq = rsrc(tb.q[t]);
-        const bool more = t + 1 < tb.n;
-        const Geo gn = more ? geo(t + 1) : g;
+        const bool more = t + tb.groups < tb.n;
+        const Geo gn = more ? geo(t + tb.groups) : g;
         const __amdgpu_buffer_rsrc_t rx =
-            more ? rsrc(tb.x[t + 1]) : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(tb.x[t]), 0, 0, 0x00020000);
+            more ? rsrc(tb.x[t + tb.groups]) : __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(tb.x[t]), 0, 0, 0x00020000);
         auto lds_slot = [&](int l) {  // this tensor's LDS slot l, read before the slot is requested anew
             u32x4 v;
             asm volatile("ds_read_b128 %0, %1 offset:%2\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_lane), "n"(l * 1024) : "memory");
@@ -599,45 +608,58 @@ static int resident_cus() {  // compute units of the current device, 0 if unknow
     return c;
 }
 
-// A tensor takes the resident kernel if it is a whole number of 1 KiB chunks, fits the chip, and fills at least three
-// quarters of it: a tensor costs the resident kernel about 12 us plus 0.52 us per million elements (every wave walks
-// all its slots and the workgroups meet in the middle), the two launches 0.82 us per million, level at 50 million.
-static bool resident_fits(const cfp8_tensor_desc& d, int cus) {
-    const uint64_t cap = (uint64_t)cus * kResWaves * kResVecs, nc = (uint64_t)(d.numel / 512);
-    return d.numel % 512 == 0 && nc <= cap && nc * 4 >= cap * 3;
+// How many tensors like this one the chip holds at the same time (0: the tensor does not take the resident kernel).
+// A tensor must be a whole number of 1 KiB chunks; G of them are resident together, each held by cus / G workgroups,
+// for the largest G <= kResMaxGroups whose groups still hold the tensor, and the tensor must fill at least three
+// quarters of its group: a round of G tensors costs the resident kernel about 5 us plus 0.52 us per million elements
+// (every wave walks all its slots and the groups meet in the middle), the two launches 0.82 us per million.
+constexpr int kResMaxGroups = 8;
+static int resident_groups(const cfp8_tensor_desc& d, int cus) {
+    if (d.numel <= 0 || d.numel % 512) return 0;
+    const uint64_t nc = (uint64_t)(d.numel / 512);
+    for (int g = kResMaxGroups; g >= 1; --g) {
+        const uint64_t cap = (uint64_t)(cus / g) * kResWaves * kResVecs;
+        if (cus / g >= 1 && nc <= cap) return nc * 4 >= cap * 3 ? g : 0;
+    }
+    return 0;
 }
+static bool resident_fits(const cfp8_tensor_desc& d, int cus) { return resident_groups(d, cus) != 0; }
 
-// The tensors of the call that take the resident kernel, kMaxBatch per launch
+// The tensors of the call that take the resident kernel: one class of group count after the other, kMaxBatch per launch
 static void resident_all(const cfp8_tensor_desc* descs, int64_t n, u32* slots, int cus, hipStream_t st) {
-    int64_t i = 0;
-    while (i < n) {
-        ResidentTable tb;
-        int count = 0;
-        for (; i < n && count < kMaxBatch; ++i) {
-            const cfp8_tensor_desc& d = descs[i];
-            if (!resident_fits(d, cus)) continue;
-            tb.x[count] = static_cast<const uint4*>(d.x);
-            tb.q[count] = static_cast<uint2*>(d.q);
-            tb.scale[count] = d.scale;
-            tb.nchunks[count] = (unsigned)(d.numel / 512);
-            tb.amax[count] = slots + i * kAmaxSlots;
-            ++count;
+    for (int groups = 1; groups <= kResMaxGroups; ++groups) {
+        int64_t i = 0;
+        while (i < n) {
+            ResidentTable tb;
+            int count = 0;
+            for (; i < n && count < kMaxBatch; ++i) {
+                const cfp8_tensor_desc& d = descs[i];
+                if (resident_groups(d, cus) != groups) continue;
+                tb.x[count] = static_cast<const uint4*>(d.x);
+                tb.q[count] = static_cast<uint2*>(d.q);
+                tb.scale[count] = d.scale;
+                tb.nchunks[count] = (unsigned)(d.numel / 512);
+                tb.amax[count] = slots + i * kAmaxSlots;
+                ++count;
+            }
+            if (count == 0) break;
+            tb.n = count;
+            tb.groups = groups;
+            tb.group_wgs = (unsigned)(cus / groups);
+            tb.wait_ticks = g_resident_wait_us.load(std::memory_order_relaxed) * 100u;  // the wall clock runs at 100 MHz
+            tb.arrivals = tb.group_wgs + g_resident_extra_arrivals.load(std::memory_order_relaxed);
+            if (tb.arrivals > (unsigned)kMeetSlots) tb.arrivals = (unsigned)kMeetSlots;
+            static std::atomic<unsigned> launches{0};
+            tb.launch_tag = (launches.fetch_add(1, std::memory_order_relaxed) % 1023u) << 6;
+            static_assert(kMaxBatch < 64, "a tensor's number fits six bits");
+            // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
+            // GPU that no other grid holds they are
+            hipLaunchKernelGGL(tensorwise_meet_clear_kernel, dim3(1), dim3(256), 0, st);
+            hipLaunchKernelGGL(tensorwise_resident_kernel, dim3((unsigned)cus), dim3(kResWaves * 64), kResLdsBytes, st, tb);
+            // tensors that the launch gave up (none, normally) are redone as two ordinary passes
+            hipLaunchKernelGGL(tensorwise_repair_amax_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
+            hipLaunchKernelGGL(tensorwise_repair_cast_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
         }
-        if (count == 0) break;
-        tb.n = count;
-        tb.wait_ticks = g_resident_wait_us.load(std::memory_order_relaxed) * 100u;  // the wall clock runs at 100 MHz
-        tb.arrivals = (unsigned)cus + g_resident_extra_arrivals.load(std::memory_order_relaxed);
-        if (tb.arrivals > (unsigned)kMeetSlots) tb.arrivals = (unsigned)kMeetSlots;
-        static std::atomic<unsigned> launches{0};
-        tb.launch_tag = (launches.fetch_add(1, std::memory_order_relaxed) % 1023u) << 6;
-        static_assert(kMaxBatch < 64, "a tensor's number fits six bits");
-        // all workgroups must be resident together: one per CU, and a workgroup fills a CU (all of its LDS), so on a
-        // GPU that no other grid holds they are
-        hipLaunchKernelGGL(tensorwise_meet_clear_kernel, dim3(1), dim3(256), 0, st);
-        hipLaunchKernelGGL(tensorwise_resident_kernel, dim3((unsigned)cus), dim3(kResWaves * 64), kResLdsBytes, st, tb);
-        // tensors that the launch gave up (none, normally) are redone as two ordinary passes
-        hipLaunchKernelGGL(tensorwise_repair_amax_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
-        hipLaunchKernelGGL(tensorwise_repair_cast_kernel, dim3((unsigned)(cus * kRepairBlocksPerCu)), dim3(256), 0, st, tb);
     }
 }
 

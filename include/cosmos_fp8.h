@@ -104,7 +104,8 @@ int cfp8_quant_rowwise_multi(const cfp8_rowwise_desc* descs, int64_t n, void* st
  * With the read-once form switched on (cfp8_tensorwise_resident, off by default), tensors that fill three quarters
  * or more of the GPU's registers and LDS and still fit (106-141 MB of bf16 on a 256-CU MI355X, numel % 512 == 0:
  * the MLP weights of a 7-8 B model) are read once: one launch of one workgroup per CU keeps them on the chip
- * between the two passes; in between the workgroups meet through a small array in device memory that the library
+ * between the two passes.  Smaller tensors that fill three quarters of a half, a third ... an eighth of the chip
+ * (down to 13 MB) are held several at a time, each by its share of the CUs, in the same kernel; in between the workgroups meet through a small array in device memory that the library
  * owns (one per GPU, so two read-once launches must not run on one GPU at the same time - which their need for
  * every CU rules out anyway).
  * The order in which the tensors of a call are quantised is unspecified; the results do not depend on it. */
