@@ -395,6 +395,49 @@ def test_tensorwise_read_once_launch_gives_up_and_is_repaired(dev):
         lib.cfp8_tensorwise_resident(prev)
 
 
+def test_tensorwise_read_once_several_tensors_at_a_time(dev):
+    """Tensors of a half to an eighth of the chip's capacity are held several at a time, each by a group of CUs that
+    meets within itself.  Every group count the library uses (8, 5, 3, 2 and 1 on 256 CUs), more tensors than groups so
+    that a second round runs with some groups idle, sizes that differ within a class, a NaN, an infinity and an
+    all-zero tensor among them: the bits of the two separate passes, and again after every meeting has been made to
+    give up from the host (all 26 tensors reported, all repaired)."""
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    if cus != 256:
+        pytest.skip("the shapes below are sized for the group capacities of 256 CUs")
+    g = torch.Generator(device=dev).manual_seed(81)
+    rows = [2048] * 6 + [2304] * 5 + [3584] * 4 + [3840] * 3 + [6000] * 2 + [6400] * 2 + [8192, 9000, 9728] + [18944]
+    ws = [(torch.randn(r, 3584, generator=g, device=dev) * (0.01 * (i % 7 + 1))).to(torch.bfloat16) for i, r in enumerate(rows)]
+    ws[3][2047, 3583] = float("nan")       # group count 8, first round
+    ws[9][0, 0] = float("inf")             # group count 8, second round
+    ws[12].zero_()                          # group count 5: the scale floor
+    ws[16][3839, 3583] = 250.0             # the maximum in the tensor's last element
+    ws[20][5999, 0] = -300.0
+    want_q, want_s = _two_pass(ws, dev)
+    prev = lib.cfp8_tensorwise_resident(1)
+    try:
+        for _ in range(2):
+            qs, scales, given_up = ops.quant_tensorwise_multi(ws, return_status=True)
+            assert int(given_up) == 0
+            assert torch.equal(bits(scales), bits(want_s)), "scales differ from the two passes"
+            for i in range(len(ws)):
+                assert torch.equal(u8(qs[i]), u8(want_q[i])), f"tensor {i} ({rows[i]} rows): bytes differ from the two passes"
+        assert int(bits(scales)[12]) == 0x2720D7C5 and int(u8(qs[12]).max()) == 0
+        _lib.check(lib.cfp8_tensorwise_resident_tuning(1000, 1))
+        try:
+            torch.cuda.synchronize()
+            qs, scales, given_up = ops.quant_tensorwise_multi(ws, return_status=True)
+            torch.cuda.synchronize()
+            assert int(given_up) == len(ws), f"{int(given_up)} tensors reported as given up, {len(ws)} took the read-once launch"
+            assert torch.equal(bits(scales), bits(want_s)), "scales after repair differ from the two passes"
+            for i in range(len(ws)):
+                assert torch.equal(u8(qs[i]), u8(want_q[i])), f"tensor {i}: bytes after repair differ from the two passes"
+        finally:
+            _lib.check(lib.cfp8_tensorwise_resident_tuning(20000, 0))
+    finally:
+        lib.cfp8_tensorwise_resident(prev)
+
+
 def test_tensorwise_read_once_launches_on_two_streams(dev):
     """Two read-once calls at the same time on two streams of one process - what the entry point's contract rules out.
     Each launch needs every CU, so they cannot both be resident, and they share the array through which workgroups
