@@ -470,7 +470,9 @@ def scaled_mm(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: 
               out_dtype: torch.dtype = torch.bfloat16, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rowwise ``torch._scaled_mm``: a fp8 [M, K] row-major, b fp8 [K, N] column-major (the
     ``.t()`` of a contiguous [N, K] weight, monkey_patch_for_fp8.py:52), scale_a [M, 1],
-    scale_b [1, N] (or [N, 1]); out = (a @ b) * scale_a * scale_b (+ bias)."""
+    scale_b [1, N] (or [N, 1]); out = (a @ b) * scale_a * scale_b (+ bias).  A scale of one element
+    (the tensorwise form of ``torch._scaled_mm``) stands for every row / column: the kernels read one
+    scale per row and per column, so it is spread into a vector here."""
     _need_gpu(a, b, scale_a, scale_b)
     if a.dtype != FP8_DTYPE or b.dtype != FP8_DTYPE:
         raise ValueError("scaled_mm takes float8_e4m3fn operands")
@@ -482,10 +484,12 @@ def scaled_mm(a: torch.Tensor, b: torch.Tensor, scale_a: torch.Tensor, scale_b: 
         raise ValueError("a must be row-major")
     if not (b.stride(0) == 1 or K == 1):
         raise ValueError("b must be column-major (pass weight.t() of a contiguous [N, K] weight)")
-    if scale_a.numel() != M or scale_b.numel() != N:
-        raise ValueError("scaled_mm needs rowwise scales: scale_a [M, 1] and scale_b [1, N]")
-    sa = scale_a.reshape(-1).contiguous().float()
-    sb = scale_b.reshape(-1).contiguous().float()
+    if scale_a.numel() not in (1, M) or scale_b.numel() not in (1, N):
+        raise ValueError("scaled_mm needs rowwise scales, scale_a [M, 1] and scale_b [1, N], or scales of one element")
+    sa = scale_a.reshape(-1).float()
+    sb = scale_b.reshape(-1).float()
+    sa = sa.expand(M).contiguous() if sa.numel() != M else sa.contiguous()
+    sb = sb.expand(N).contiguous() if sb.numel() != N else sb.contiguous()
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     ld_a = a.stride(0) if M > 1 else K
     ld_b = b.stride(1) if N > 1 else K

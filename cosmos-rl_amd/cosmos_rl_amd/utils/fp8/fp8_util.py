@@ -99,8 +99,7 @@ class Float8Linear(nn.Linear):
         else:
             qw, sw = ops.quant_tensorwise(w)
             qx, sx = ops.quant_tensorwise(x2)
-            out = ops.scaled_mm(qx, qw.t(), sx.expand(x2.shape[0]).contiguous(),
-                                sw.expand(self.out_features).contiguous(), out_dtype=torch.bfloat16)
+            out = ops.scaled_mm(qx, qw.t(), sx, sw, out_dtype=torch.bfloat16)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out.reshape(*input.shape[:-1], self.out_features).to(input.dtype)

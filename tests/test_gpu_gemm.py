@@ -76,6 +76,21 @@ def test_scaled_mm_rowwise(dev, M, N, K):
     check_bf16(out16, ref, f"rowwise {M}x{N}x{K}")
 
 
+def test_scaled_mm_one_element_scales(dev):
+    """Scales of one element - the tensorwise form of ``torch._scaled_mm`` that the converted linear of the tensorwise
+    recipe uses - give the bits of the same call with the scale repeated for every row and column."""
+    M, N, K = 96, 528, 384
+    x, w, qx, sx, qw, sw = rowwise_operands(M, N, K, seed=5, dev=dev)
+    a, b = f8(qx, dev), f8(qw, dev)
+    s1, s2 = sx[3].to(dev), sw[7].to(dev)
+    for dt in (torch.float32, torch.bfloat16):
+        one = ops.scaled_mm(a, b.t(), s1, s2.reshape(1, 1), out_dtype=dt)
+        rep = ops.scaled_mm(a, b.t(), s1.expand(M, 1).contiguous(), s2.expand(1, N).contiguous(), out_dtype=dt)
+        assert torch.equal(one, rep)
+    with pytest.raises(ValueError):
+        ops.scaled_mm(a, b.t(), sx[:2].to(dev), sw.to(dev).t())
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 16, 16), (5, 48, 80), (16, 64, 144), (17, 200 * 16, 1200), (64, 96, 2880), (100, 528, 1200),
                                    (300, 272, 80), (513, 1024, 2192), (2, 18944, 3600)])
 def test_rowwise_k_not_a_multiple_of_128(dev, M, N, K):
