@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void tensorwise_cast_kernel(const TensorTable 
 // quantises.
 // ---------------------------------------------------------------------------
 static std::atomic<int> g_resident_enabled{0};
-static std::atomic<unsigned> g_resident_wait_us{20000};   // bound of a workgroup's wait at a tensor's counter
+static std::atomic<unsigned> g_resident_wait_us{20000};   // bound of a workgroup's wait at a tensor's meeting
 static std::atomic<unsigned> g_resident_extra_arrivals{0};  // test hook: arrivals expected beyond the grid (never come)
 
 
@@ -446,8 +446,8 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
 // The two passes over exactly those tensors of a resident launch whose status word says that the launch gave them
 // up.  Small fixed grids behind every resident launch: a workgroup reads the status words of the launch's tensors
 // with one wave-wide load and leaves at once when none is set, which is the normal case.  Maxima go to slots
-// 1 .. 62 (slot 0 holds the resident kernel's counter; what that kernel's workgroups published there before giving
-// up are maxima of parts of the same tensor and do no harm).
+// 1 .. 62 of the tensor's amax slots (the resident kernel writes none of them: its maxima travel through the
+// meeting array); slot 63 is the status word.
 // ---------------------------------------------------------------------------
 constexpr int kRepairBlocksPerCu = 8;
 
