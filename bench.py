@@ -177,7 +177,12 @@ def main() -> int:
     d_big, n_big, numel_big = sub_table(lambda t: resident_groups(t) == 1)
     d_mid, n_mid, numel_mid = sub_table(lambda t: resident_groups(t) > 1)
     d_rest, n_rest, numel_rest = sub_table(lambda t: resident_groups(t) == 0)
-    assert (n_big, n_mid, n_rest) == (84, 56, 57), (n_big, n_mid, n_rest)
+    if (n_big, n_mid, n_rest) != (84, 56, 57):
+        # (a GPU with another CU count draws the lines between the kinds elsewhere; the figures below then describe
+        # other sets of tensors than their texts say)
+        print(f"bench.py: {cus} CUs: {n_big} / {n_mid} / {n_rest} tensors in the three kinds, 84 / 56 / 57 expected", file=sys.stderr)
+    if min(n_big, n_mid, n_rest) == 0:
+        raise SystemExit("bench.py: the headline workload does not split into the three kinds of tensorwise launch on this GPU")
     res_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_big, n_big, amax_ws.data_ptr(), stream)), reps)
     mid_ms = time_phase(lambda: _lib.check(lib.cfp8_quant_tensorwise_multi(d_mid, n_mid, amax_ws.data_ptr(), stream)), reps)
     amax_ms = time_phase(lambda: _lib.check(lib.cfp8_tensorwise_amax_multi(d_rest, n_rest, amax_ws.data_ptr(), stream)), reps)
