@@ -634,13 +634,20 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256_kernel(const GemmArgs p)
 // epilogue (the tile's scales and the buffer that turns the wave's block into row-contiguous stores, 16 rows at a
 // time); it is filled right after.  Requires K >= 384.
 // ---------------------------------------------------------------------------
+// A last round that is at most half full (p.tail_tiles tiles, the last ones in the workgroups' order) would cost every
+// workgroup's wait for the few that have a tile in it.  Those tiles are cut into quarters of 128 x 128 instead, dealt
+// to all workgroups behind their last full tile and computed by the strip kernel's ring pipeline (same products in
+// the same order of K, same epilogue arithmetic: the same bits).
+template <int BM, int TN, bool OUT_F32>
+__device__ __forceinline__ void rowwise_strip_block(const GemmArgs& p, uint8_t* const smem, const int m0, const int n0, const int t);
+
 template <bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_rowwise_256p_kernel(const GemmArgs p) {
     constexpr int BM = 256, BN = 256;
     constexpr int XS = BM * 128, WS = BN * 128;
     constexpr int WBASE = 2 * XS;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int ntiles = p.tiles_m * p.tiles_n;
+    const int ntiles = p.tiles_m * p.tiles_n - p.tail_tiles;  // tiles taken whole
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave & 1, wn = wave >> 1;
@@ -849,6 +856,33 @@ __global__ __launch_bounds__(256) void gemm_rowwise_256p_kernel(const GemmArgs p
     }
     // the loads past the last tile (they fetched its first steps once more) land before the workgroup gives up its LDS
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the quarters of the tiles of the last round.  (The thread's number is formed anew here, from the wave's number and
+    // a count of the lanes below, and passes through an empty asm: everything the quarter tiles derive from it would
+    // otherwise be computed at the kernel's start and kept in registers through the tiles' K loops, which have none to
+    // spare.)
+    int t_late = wave * 64 + (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(t_late));
+    // (likewise the kernel's arguments: read again from the kernel-argument segment, through a pointer the compiler
+    // cannot see through, instead of being held in scalar registers from the kernel's start)
+    uint64_t args_at = reinterpret_cast<uint64_t>(__builtin_amdgcn_kernarg_segment_ptr());
+    uint32_t args_lo = (uint32_t)args_at, args_hi = (uint32_t)(args_at >> 32);
+    asm volatile("" : "+s"(args_lo), "+s"(args_hi));
+    args_lo = __builtin_amdgcn_readfirstlane(args_lo);  // (wave-uniform, which the compiler does not assume of an asm's result)
+    args_hi = __builtin_amdgcn_readfirstlane(args_hi);
+    typedef __attribute__((address_space(4))) const uint32_t ConstWord;  // (the segment is constant memory: scalar loads)
+    const ConstWord* const words = reinterpret_cast<const ConstWord*>(((uint64_t)args_hi << 32) | args_lo);
+    static_assert(sizeof(GemmArgs) % 4 == 0, "copied word by word");
+    uint32_t copy[sizeof(GemmArgs) / 4];
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(GemmArgs) / 4; ++i) copy[i] = words[i];
+    GemmArgs late;
+    __builtin_memcpy(&late, copy, sizeof(late));
+    for (int u = (int)blockIdx.x; u < 4 * late.tail_tiles; u += (int)gridDim.x) {
+        __syncthreads();  // every wave is done with the stages (the last tile's epilogue buffer, the quarter before)
+        int tm, tn;
+        tile_of_block(late.tiles_m * late.tiles_n - late.tail_tiles + (u >> 2), late.tiles_m, late.tiles_n, tm, tn);
+        rowwise_strip_block<128, 8, OUT_F32>(late, smem, tm * BM + (u & 1) * 128, tn * BN + ((u >> 1) & 1) * 128, t_late);
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1748,6 +1782,10 @@ static int launch_rowwise_256p(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     const int cus = cu_count();
     const int64_t blocks = tiles < cus ? tiles : cus;
+    // a last round that is at most half full is taken apart into quarter tiles (the strip kernel's ring needs K >= 128
+    // only; its stores take any pitch)
+    const int64_t rem = tiles % blocks;
+    p.tail_tiles = (tiles > blocks && rem > 0 && rem * 2 <= blocks) ? (int)rem : 0;
     constexpr size_t lds = (size_t)(2 + 3) * 256 * 128;
     static std::atomic<bool> raised[65][2];  // zero-initialised
     const int v = out_dtype == CFP8_OUT_F32 ? 1 : 0;
@@ -1756,7 +1794,13 @@ static int launch_rowwise_256p(GemmArgs& p, int out_dtype, hipStream_t st) {
     const int slot = device_slot();
     if (slot == 64) raised[64][v].store(false, std::memory_order_relaxed);
     if (int rc = raise_lds_limit(fn, lds, raised[slot][v])) return rc;
-    if (!note_launch("gemm_rowwise_256p", (unsigned)blocks, 256, lds)) return CFP8_OK;
+    static_assert(lds == (size_t)5 * (128 + 128) * 128, "the ring of the quarter tiles takes the same LDS");
+    {
+        char name[64];
+        if (p.tail_tiles) snprintf(name, sizeof(name), "gemm_rowwise_256p tail=%d", p.tail_tiles);
+        else snprintf(name, sizeof(name), "gemm_rowwise_256p");
+        if (!note_launch(name, (unsigned)blocks, 256, lds)) return CFP8_OK;
+    }
     if (v) hipLaunchKernelGGL(gemm_rowwise_256p_kernel<true>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     else hipLaunchKernelGGL(gemm_rowwise_256p_kernel<false>, dim3((unsigned)blocks), dim3(256), lds, st, p);
     return check_launch("gemm");
@@ -2160,7 +2204,7 @@ static int launch_rowwise_gemv(GemmArgs& p, int out_dtype, hipStream_t st) {
 // lane beyond its descriptor.  Wave w computes token rows w BM / 4 ... against all TN weight tiles.
 // ---------------------------------------------------------------------------
 template <int BM, int TN, bool OUT_F32>
-__global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs p) {
+__device__ __forceinline__ void rowwise_strip_block(const GemmArgs& p, uint8_t* const smem, const int m0, const int n0, const int t) {
     constexpr int BN = TN * 16;
     constexpr int WROWS = (BN + 31) / 32 * 32;          // weight rows requested per step: 8 per wave and load
     constexpr int LX = BM / 32, LW = WROWS / 32;        // loads per wave and step
@@ -2168,12 +2212,8 @@ __global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs 
     constexpr int S = BM == 64 ? 8 : 5;                 // ring depth: what the LDS holds (160 / 140 KiB)
     constexpr int XT = BM / 64;                         // token tiles per wave
     constexpr uint32_t kEnd = 0xEFFFFFFFu;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // S activation stages, then S weight stages
-    constexpr int WBASE = S * XS;
-    // token blocks of one weight strip are neighbours in the grid: they run at the same time and the second reads the
-    // strip from the caches
-    const int m0 = (int)(blockIdx.x % (unsigned)p.tiles_m) * BM, n0 = (int)(blockIdx.x / (unsigned)p.tiles_m) * BN;
-    const int t = threadIdx.x, lane = t & 63;
+    constexpr int WBASE = S * XS;  // smem: S activation stages, then S weight stages
+    const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int lrow = lane & 15, quarter = lane >> 4;
     const int KT = p.K >> 7;
@@ -2205,18 +2245,24 @@ __global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs 
                                                      (uint32_t)i * b_step + ((uint32_t)kt << 7), 0, 2);
     };
 
+    // (the argument block may be a copy read from memory, whose pointers the compiler takes for generic ones: said
+    // here that they point to global memory)
+    typedef __attribute__((address_space(1))) const float gbl_float;
+    typedef __attribute__((address_space(1))) const f32x4 gbl_f32x4;
+    const gbl_float* const sa_g = (const gbl_float*)p.sa;
+    const gbl_float* const sb_g = (const gbl_float*)p.sb;
     // the scales of the epilogue first: they are the oldest loads, every later wait covers them
     float sam[XT];
     f32x4 sbn[TN];
 #pragma unroll
     for (int j = 0; j < XT; ++j) {
         const int m = m0 + wave * (BM / 4) + j * 16 + lrow;
-        sam[j] = p.sa[m < p.M ? m : p.M - 1];
+        sam[j] = sa_g[m < p.M ? m : p.M - 1];
     }
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
         const int n = n0 + i * 16 + quarter * 4;
-        sbn[i] = *reinterpret_cast<const f32x4*>(p.sb + (n < p.N ? n : 0));
+        sbn[i] = *(const gbl_f32x4*)(sb_g + (n < p.N ? n : 0));
     }
 
     f32x4 acc[TN][XT];
@@ -2277,11 +2323,23 @@ __global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs 
             f32x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e] * sam[j] * sbn[i][e];
-            if (OUT_F32) *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + (int64_t)m * p.ld_out + n) = v;
-            else *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.out) + (int64_t)m * p.ld_out + n) =
-                    make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            typedef __attribute__((address_space(1))) f32x4 gbl_out4;
+            typedef __attribute__((address_space(1))) u32x2 gbl_out2;
+            typedef __attribute__((address_space(1))) float gbl_outf;
+            typedef __attribute__((address_space(1))) uint16_t gbl_outh;
+            if (OUT_F32) *(gbl_out4*)((gbl_outf*)p.out + (int64_t)m * p.ld_out + n) = v;
+            else *(gbl_out2*)((gbl_outh*)p.out + (int64_t)m * p.ld_out + n) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
         }
     }
+}
+
+template <int BM, int TN, bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_rowwise_strip_kernel(const GemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    // token blocks of one weight strip are neighbours in the grid: they run at the same time and the second reads the
+    // strip from the caches
+    rowwise_strip_block<BM, TN, OUT_F32>(p, smem, (int)(blockIdx.x % (unsigned)p.tiles_m) * BM, (int)(blockIdx.x / (unsigned)p.tiles_m) * TN * 16,
+                                         (int)threadIdx.x);
 }
 
 template <int BM, int TN>
@@ -3100,6 +3158,10 @@ static int launch_gemm(GemmArgs& p, int out_dtype, hipStream_t st) {
         const int64_t tm = p.M / 256, tn = p.N / 256, rem = (tm * tn) % 256;
         const int64_t cut = (rem + tm - 1) / tm;  // tile-columns that hold the partial round
         if (tm * tn > 256 && rem > 0 && rem <= 128 && cut < tn) {
+            // the walking kernel deals the partial round's tiles to all its workgroups as quarter tiles itself
+            // (1024 x 18944 x 3584: 81.8 against 84.2 us with the last ten tile-columns as a launch of their own; 8192 tokens:
+            // 410 against 411 us)
+            if (p.K >= 384) return launch_rowwise_256(p, out_dtype, st);
             GemmArgs head = p;
             head.N = (int)((tn - cut) * 256);
             if (int rc = launch_rowwise_256(head, out_dtype, st)) return rc;

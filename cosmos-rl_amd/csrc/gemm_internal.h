@@ -30,6 +30,8 @@ struct GemmArgs {
     int64_t ld_hs;
     // gemm_grouped_xres_kernel: pieces along N of the tile rows that are not whole-row units
     int unit_parts;
+    // gemm_rowwise_256p_kernel: tiles of the last, at most half-full round, computed as quarter tiles by all workgroups
+    int tail_tiles;
 };
 
 // ---- host side (gemm_fp8.hip) ---------------------------------------------

@@ -27,13 +27,15 @@ def w8_lds(bm, bn, kt):
 
 CASES = [
     # benchmark config 3 (rowwise linear, N = 18944, K = 3584)
-    ("cfg3 M=8192", (ROW, 8192, 18944, 3584),
-     f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
+    # (9.25 rounds of 256 x 256 tiles: the 64 tiles of the last round as quarter tiles inside the walking kernel's launch)
+    ("cfg3 M=8192", (ROW, 8192, 18944, 3584), f"gemm_rowwise_256p tail=64 grid=256 block=256 lds={LDS_ROW}"),
     ("cfg3 M=8192 linear", (LIN, 8192, 18944, 3584),
-     f"quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}; "
-     "gemm_kernel<128,128,2,2,rowwise> grid=256 block=256 lds=65536"),
-    ("cfg3 M=1024", (ROW, 1024, 18944, 3584),
-     f"gemm_rowwise_256 grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=160 block=256 lds=65536"),
+     f"quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_256p tail=64 grid=256 block=256 lds={LDS_ROW}"),
+    ("cfg3 M=1024", (ROW, 1024, 18944, 3584), f"gemm_rowwise_256p tail=40 grid=256 block=256 lds={LDS_ROW}"),
+    ("partial round above a half: whole tiles", (ROW, 2304, 11520, 512), f"gemm_rowwise_256p grid=256 block=256 lds={LDS_ROW}"),
+    ("partial round of a half", (ROW, 2048, 12288, 512), f"gemm_rowwise_256p tail=128 grid=256 block=256 lds={LDS_ROW}"),
+    ("short K keeps the second launch", (ROW, 2048, 8704, 256),
+     f"gemm_rowwise_256 grid=256 block=256 lds={LDS_ROW}; gemm_kernel<128,128,2,2,rowwise> grid=64 block=256 lds=65536"),
     ("cfg3 M=512: one round of 256 x 256 tiles", (ROW, 512, 18944, 3584), f"gemm_rowwise_256 grid=148 block=256 lds={LDS_ROW}"),
     ("cfg3 M=64", (LIN, 64, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),
     ("cfg3 M=17", (LIN, 17, 18944, 3584), "quant_rowwise grid=0 block=256 lds=0; gemm_rowwise_strip<64,5> grid=237 block=256 lds=163840"),

@@ -49,10 +49,12 @@ def rowwise_operands(M, N, K, seed, dev):
                                    (256, 128, 128), (512, 256, 256), (256, 2176, 384), (768, 384, 512), (1024, 1152, 640), (1024, 3584, 896),
                                    # more 256 x 256 tiles than CUs: every workgroup walks several tiles and loads the next
                                    # one under the current one; 408 tiles and K of 3 steps, 405 tiles and 4 steps (a second
-                                   # round that not every workgroup takes part in), 512 tiles (+ 16 as a second launch) and 5 steps
+                                   # round that not every workgroup takes part in), 512 tiles (+ 16 as quarter tiles behind them) and 5 steps
                                    (4352, 6144, 384), (2304, 11520, 512), (2048, 16896, 640),
                                    # 8 x 33 tiles = one full round of 256 + 8: the last tile-column runs as a second launch
                                    (2048, 8448, 256),
+                                   # a last round of 16 tiles as quarter tiles inside the walking kernel; with rows beyond a multiple of 256
+                                   (2048, 8704, 384), (2100, 8704, 384),
                                    # M not a multiple of 256: aligned body on the 256x256 kernel + the last rows as their own launch
                                    (1000, 512, 384), (520, 256, 256),
                                    # 17..64 tokens: the strip kernel with 32 or 80 weight rows per workgroup (chosen from
@@ -662,7 +664,9 @@ def test_walking_kernels_equal_to_sliced_calls(dev):
     """Rowwise and block-scaled: a problem with more tiles than CUs (the walking kernels) against the same problem cut
     along N into calls that fit one round of workgroups (one tile per workgroup, or the generic kernel): same bits."""
     g = torch.Generator(device=dev).manual_seed(9)
-    for mode, (M, N, K), cuts in (("row", (2304, 11520, 512), 3), ("row", (8192, 7680, 896), 6), ("blk", (1024, 12288, 1536), 2),
+    # (the third to fifth: a last round of 16, 96 and 40 tiles, which the walking kernel's workgroups take as quarter tiles)
+    for mode, (M, N, K), cuts in (("row", (2304, 11520, 512), 3), ("row", (8192, 7680, 896), 6), ("row", (2048, 8704, 512), 2),
+                                  ("row", (2048, 11264, 640), 2), ("row", (1024, 18944, 3584), 2), ("blk", (1024, 12288, 1536), 2),
                                   ("blk", (2048, 6400, 640), 2)):
         qx = torch.randint(0, 256, (M, K), generator=g, device=dev, dtype=torch.uint8)
         qw = torch.randint(0, 256, (N, K), generator=g, device=dev, dtype=torch.uint8)

@@ -102,9 +102,10 @@ def test_graph_tensorwise_read_once_launch(dev):
     _replay_matches_eager(dev, inputs, fn)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 2048, 3584), (64, 2048, 3584), (48, 1024, 7168), (1024, 2048, 3584), (2304, 8448, 256)])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 3584), (64, 2048, 3584), (48, 1024, 7168), (1024, 2048, 3584), (2304, 8448, 256), (2048, 8704, 512)])
 def test_graph_fp8_linear(dev, M, N, K):
-    """single-token and 64-token kernels, the split-K pair of launches, 256x256 tiles, and the head + tail pair"""
+    """single-token and 64-token kernels, the split-K pair of launches, 256x256 tiles, the head + tail pair, and the
+    walking kernel with a last round taken as quarter tiles"""
     w = _bf16(dev, 5, N, K, std=0.02)
     qw, sw = ops.quant_rowwise(w)
 
