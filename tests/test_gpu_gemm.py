@@ -123,7 +123,7 @@ def test_rowwise_k_not_a_multiple_of_128(dev, M, N, K):
         assert bool(torch.isnan(out[:, 1]).all()) and torch.equal(out[:, 2:], out32[:, 2:]) and torch.equal(out[:, 0], out32[:, 0])
 
 
-@pytest.mark.parametrize("M,N,K", [(768, 512, 384), (1024, 768, 1024)])
+@pytest.mark.parametrize("M,N,K", [(768, 512, 384), (1024, 768, 1024), (2048, 8704, 384)])  # (the last: walking kernel + quarter tiles)
 def test_scaled_mm_rowwise_pitched_operands(dev, M, N, K):
     """The 256x256 kernel fetches its tiles with per-lane addresses built from the leading dimensions: operands that are
     column slices of wider buffers (row pitch K + 128 and K + 256, data pointers offset into the buffer) give the
