@@ -178,6 +178,7 @@ constexpr int kResWaves = 12;     // per workgroup
 constexpr int kResRegVecs = 32;
 constexpr int kResLdsVecs = 13;
 constexpr int kResVecs = kResRegVecs + kResLdsVecs;
+constexpr int kResTouch = 2;      // chunks of the next tensor a wave touches while the workgroups meet
 static_assert(kResLdsVecs <= kResRegVecs, "the LDS part passes through registers");
 constexpr size_t kResLdsBytes = (size_t)kResWaves * kResLdsVecs * 64 * 16 + 64;
 static_assert(kResLdsBytes <= 160 * 1024, "LDS of one CU");
@@ -300,6 +301,22 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
             const u32 w = wave_max(pk_fold(m));
             if (lane == 0) red[wave] = w;
         }
+        // ---- while the workgroups meet, memory has nothing to do: every wave but the one that reads the meeting words
+        // (whose reads would queue behind it) touches the lines of its first kResTouch chunks of the next tensor, one
+        // dword per line, so that they are on their way into the caches during the meeting; the phase behind the meeting
+        // asks for those chunks first.  (Through a descriptor of no bytes where there is nothing to touch.  A tensor that
+        // takes this kernel has more chunks than its group has waves: chunk gw exists.)  Measured: 37.8 against 38.2 us
+        // per 136 MB tensor with two chunks, nothing with one or three, slower with four and more.
+        u32 touched;
+        {
+            const bool touch = wave != 0 && t + tb.groups < tb.n;
+            const int tn = touch ? t + tb.groups : t;
+            const u32 ci = (u32)(lane >> 3) < (u32)kResTouch ? (u32)(lane >> 3) : (u32)kResTouch - 1u;
+            u32 c = gw + ci * nw;
+            c = c < tb.nchunks[tn] ? c : gw;
+            const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(tb.x[tn]), 0, touch ? 0xFFFFFFFF : 0, 0x00020000);
+            touched = __builtin_amdgcn_raw_buffer_load_b32(rt, c * 1024u + (u32)(lane & 7) * 128u, 0, 0);
+        }
         // ---- the meeting.  The workgroup's maximum goes, tagged with the tensor's number, to the workgroup's own word
         // of the meeting array (side t & 1) by one atomic whose result nobody waits for; the first wave then reads all
         // the workgroups' words until every one carries the tag, and has the tensor's maximum in hand when they do:
@@ -380,6 +397,7 @@ __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(
         // otherwise put a wait for the kept registers' loads in front of every use of one, inside the phase below,
         // where it would bound the stores and loads in flight.)
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters left alone
+        asm volatile("" ::"v"(touched));         // (the touch load's register stays the wave's until it has landed)
         const float amax = amax_from_bits(red[kResWaves]);
         const float scale = scale_from_amax(amax);
         if (gw == 0 && lane == 0) *tb.scale[t] = scale;
