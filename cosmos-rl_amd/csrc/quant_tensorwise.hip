@@ -213,7 +213,7 @@ struct ResidentTable {
 
 __global__ __launch_bounds__(kResWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tensorwise_resident_kernel(const ResidentTable tb) {
     extern __shared__ __attribute__((aligned(16))) uint4 res_lds[];  // [waves][kResLdsVecs][64 lanes], then the give-up flag
-    u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);  // this tensor's verdict
+    u32* const gave_up = reinterpret_cast<u32*>(res_lds + kResWaves * kResLdsVecs * 64);  // this tensor's outcome
     u32* const red = gave_up + 1;  // [kResWaves] maxima of the waves, then the tensor's maximum
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
